@@ -1,0 +1,170 @@
+/*
+ * protenix_amd.h - C ABI of the MI355X (gfx950) Pairformer pair-stack kernels.
+ *
+ * One shared library, libprotenix_amd.so.  Every entry point
+ *   - takes raw DEVICE pointers, sizes, a dtype code and a hipStream_t (as
+ *     void*); no framework types cross the boundary;
+ *   - allocates nothing and keeps no state: the caller owns inputs, outputs
+ *     and workspaces; work is enqueued on `stream` and not waited for;
+ *   - returns PTX_OK or an error code; ptx_last_error_string() describes the
+ *     last failure of the calling thread.
+ *
+ * Tensors are dense, row-major, in the layouts named per function.  `dtype`
+ * selects fp32 or bf16 storage for every tensor of the call unless said
+ * otherwise; accumulation and statistics are always fp32.  The pair tensor is
+ * "z[N][N][c]"; a "logical row" p = outer*N + inner addresses z[outer][inner]
+ * (transposed = 0) or z[inner][outer] (transposed = 1), which is how the
+ * ending-node attention and the incoming triangle product are served without
+ * a transposed copy.
+ *
+ * Reference interfaces replaced (paths relative to bytedance/Protenix):
+ *   protenix/model/layer_norm/kernel/layer_norm_cuda.cpp:142-179 (pybind module
+ *     fast_layer_norm_cuda_v2), protenix/model/tri_attention/op.py:37-77
+ *     (TriAttentionFunction), protenix/model/triangular/triangular.py:77-90
+ *     (triangle_multiplicative_update), and the torch-path arithmetic of
+ *     triangular.py:519-566, 657-715, layers.py:276-296, 361-398,
+ *     primitives.py:190-230, transformer.py:184-194.
+ */
+#ifndef PROTENIX_AMD_H_
+#define PROTENIX_AMD_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define PTX_ABI_VERSION 1
+#define PTX_API __attribute__((visibility("default")))
+
+enum ptx_dtype { PTX_F32 = 0, PTX_BF16 = 1 };
+
+enum ptx_status {
+  PTX_OK = 0,
+  PTX_ERR_BAD_ARG = 1,     /* null pointer, negative size, unknown dtype       */
+  PTX_ERR_UNSUPPORTED = 2, /* a shape this build has no kernel for             */
+  PTX_ERR_LAUNCH = 3       /* hipGetLastError() after the launch was not clean */
+};
+
+/* ABI version of the loaded library (== PTX_ABI_VERSION it was built with). */
+PTX_API int ptx_version(void);
+
+/* Text of the calling thread's last error ("" if none).  Never NULL. */
+PTX_API const char* ptx_last_error_string(void);
+
+/*
+ * Row pitch (in elements) of the intermediate tensors whose last axis is the
+ * contracted / key axis: the smallest multiple of 64 that is >= n.  Padding
+ * elements are never read as data and need no initialisation.
+ */
+PTX_API int ptx_key_pitch(int n);
+
+/*
+ * LayerNorm forward over the last dimension.
+ * Replaces fast_layer_norm_cuda_v2.forward_{none,with_bias,with_weight,
+ * with_both}_affine (layer_norm_cuda.cpp:142-157; kernel
+ * layer_norm_cuda_kernel.cu:145-229): gamma and/or beta may be NULL.
+ *   x, y   [rows][cols]     y may alias x
+ *   mean, rstd  fp32 [rows], each may be NULL
+ */
+PTX_API int ptx_layernorm_fwd(const void* x, const void* gamma, const void* beta, void* y,
+                      float* mean, float* rstd, int64_t rows, int cols, float eps,
+                      int dtype, void* stream);
+
+/*
+ * Triangle multiplication, stage 1 (triangular.py:537-543):
+ *   zn = LN(z);  a = mask * sigmoid(W_ag zn) * (W_ap zn);  b likewise,
+ * written channel-major so that stage 2 is a plain batched matrix product:
+ *   outgoing (incoming = 0):  a[c][i][k] = a(z[i][k])[c]
+ *   incoming (incoming = 1):  a[c][i][k] = a(z[k][i])[c]      (same for b)
+ *   z [n][n][c_z], mask [n][n] in `dtype` or NULL (= ones),
+ *   w_* [c_hidden][c_z], a, b [c_hidden][n][k_pitch], k_pitch = ptx_key_pitch(n).
+ *   c_z = c_hidden = 128.
+ */
+PTX_API int ptx_trimul_project(const void* z, const void* mask, const void* ln_w, const void* ln_b,
+                       const void* w_ap, const void* w_ag, const void* w_bp, const void* w_bg,
+                       void* a, void* b, int n, int c_z, int c_hidden, int k_pitch, int incoming,
+                       float eps, int dtype, void* stream);
+
+/*
+ * Triangle multiplication, stage 2 (triangular.py:123-150): for every channel
+ *   x[c][i][j] = sum_k a[c][i][k] * b[c][j][k]
+ * which with the stage-1 layouts is 'ikc,jkc->ijc' (outgoing) or
+ * 'kic,kjc->ijc' (incoming).  a, b [c][n][k_pitch]; x [c][n][n] dense.
+ */
+PTX_API int ptx_trimul_contract(const void* a, const void* b, void* x, int n, int c, int k_pitch,
+                        int dtype, void* stream);
+
+/*
+ * Triangle multiplication, stage 3 (triangular.py:560-565):
+ *   out = [residual z +] W_z LN_out(x) * sigmoid(W_g LN_in(z))
+ *   x [c_hidden][n][n] from stage 2, z [n][n][c_z], out [n][n][c_z] (may alias z).
+ * add_residual = 1 gives z + update (the reference's `_add_with_inplace`).
+ */
+PTX_API int ptx_trimul_output(const void* x, const void* z, const void* ln_in_w, const void* ln_in_b,
+                      const void* ln_out_w, const void* ln_out_b, const void* w_z,
+                      const void* w_g, void* out, int n, int c_z, int c_hidden,
+                      int add_residual, float eps, int dtype, void* stream);
+
+/*
+ * Triangle attention, stage 1 (triangular.py:683-692, layers.py:361-382, 386):
+ *   xn = LN(x);  q = W_q xn / sqrt(d);  k = W_k xn;  v = W_v xn;
+ *   g = sigmoid(W_g xn);  tri_bias = W_b xn
+ * over logical rows p = i*n + j of x = z (transposed = 0) or z^T (transposed = 1).
+ *   q, k, g [n][n][heads*d];  vt [n][heads*d][key_pitch] (v transposed per row i);
+ *   tri_bias [heads][n][key_pitch];  key_pitch = ptx_key_pitch(n).
+ *   c_in = heads*d = 128, d = 32.
+ */
+PTX_API int ptx_triattn_project(const void* z, const void* ln_w, const void* ln_b, const void* w_q,
+                        const void* w_k, const void* w_v, const void* w_g, const void* w_b,
+                        void* q, void* k, void* vt, void* g, void* tri_bias, int n, int c_in,
+                        int heads, int d, int key_pitch, int transposed, float eps, int dtype,
+                        void* stream);
+
+/*
+ * Triangle attention, stage 2: the fused op of tri_attention/op.py:37-77 with
+ * the gate of layers.py:386-390 applied on the way out.  For every row i, head h:
+ *   o[i][j][h] = g[i][j][h] * sum_k softmax_k( q[i][j][h].k[i][k][h]
+ *                + inf*(mask(i,k)-1) + tri_bias[h][j][k] ) v[i][k][h]
+ * The N^3 logits are never materialised.  The two biases are added in the
+ * reference's order in fp32, so a fully masked row gives the mean of v, as
+ * layers.py:286-291 does.
+ *   mask [n][n] in `dtype` or NULL; mask(i,k) = mask[i][k], or mask[k][i] when
+ *   mask_transposed = 1.   o [n][n][heads*d] (may alias g, not q/k/vt).
+ */
+PTX_API int ptx_triattn_fwd(const void* q, const void* k, const void* vt, const void* g,
+                    const void* tri_bias, const void* mask, void* o, int n, int heads, int d,
+                    int key_pitch, int mask_transposed, float inf, int dtype, void* stream);
+
+/*
+ * Triangle attention, stage 3 (layers.py:392-396 + the caller's residual add,
+ * pairformer.py:189-213):  out(p) = [z(p) +] W_o o[p], where logical row p maps
+ * to z[i][j] or, transposed = 1, z[j][i].  out may alias z.
+ */
+PTX_API int ptx_triattn_output(const void* o, const void* w_o, const void* z, void* out, int n,
+                       int c_in, int transposed, int add_residual, int dtype, void* stream);
+
+/*
+ * Transition (primitives.py:190-230):
+ *   out = [x +] W_o ( silu(W_a LN(x)) * (W_b LN(x)) )
+ *   x, out [rows][c] (out may alias x), w_a, w_b [n_factor*c][c], w_o [c][n_factor*c],
+ *   hidden: caller-provided workspace [rows][n_factor*c].   c = 128.
+ */
+PTX_API int ptx_transition_fwd(const void* x, const void* ln_w, const void* ln_b, const void* w_a,
+                       const void* w_b, const void* w_o, void* hidden, void* out, int64_t rows,
+                       int c, int n_factor, int add_residual, float eps, int dtype,
+                       void* stream);
+
+/*
+ * Pair bias of the single-representation attention (transformer.py:191-194):
+ *   bias[h][i][j] = (W LN(z[i][j]))[h],  W [heads][c_z], heads <= 32, c_z = 128.
+ * ln_b may be NULL.  bias is fp32 when out_f32 = 1, else `dtype`.
+ */
+PTX_API int ptx_pair_bias_fwd(const void* z, const void* ln_w, const void* ln_b, const void* w,
+                      void* bias, int n, int c_z, int heads, int out_f32, float eps, int dtype,
+                      void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PROTENIX_AMD_H_ */

@@ -1,0 +1,25 @@
+"""MI355X-native Pairformer pair stack: drop-in modules for Protenix's
+TriangleMultiplication*, TriangleAttention, LayerNorm, Transition,
+AttentionPairBias, PairformerBlock and PairformerStack, backed by hand-written
+gfx950 kernels in libprotenix_amd.so (C ABI: include/protenix_amd.h)."""
+
+from .layer_norm import FusedLayerNorm, LayerNorm
+from .pairformer import PairformerBlock, PairformerStack
+from .primitives import Linear, LinearNoBias, Transition
+from .transformer import AttentionPairBias
+from .triangular import (
+    TriangleAttention,
+    TriangleAttentionEndingNode,
+    TriangleAttentionStartingNode,
+    TriangleMultiplicationIncoming,
+    TriangleMultiplicationOutgoing,
+    TriangleMultiplicativeUpdate,
+)
+
+__all__ = [
+    "AttentionPairBias", "FusedLayerNorm", "LayerNorm", "Linear", "LinearNoBias",
+    "PairformerBlock", "PairformerStack", "Transition", "TriangleAttention",
+    "TriangleAttentionEndingNode", "TriangleAttentionStartingNode",
+    "TriangleMultiplicationIncoming", "TriangleMultiplicationOutgoing",
+    "TriangleMultiplicativeUpdate",
+]

@@ -1,0 +1,238 @@
+// extern "C" boundary of libprotenix_amd.so: argument validation, dtype
+// dispatch, launch-error capture.  See include/protenix_amd.h for the contract.
+#include <stdarg.h>
+#include <stdio.h>
+
+#include "../../include/protenix_amd.h"
+#include "common.h"
+#include "kernels.h"
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+int after_launch(const char* what) {
+  const hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(PTX_ERR_LAUNCH, "%s: %s", what, hipGetErrorString(e));
+  g_err[0] = 0;
+  return PTX_OK;
+}
+
+bool dtype_ok(int dtype) { return dtype == PTX_F32 || dtype == PTX_BF16; }
+
+size_t esize(int dtype) { return dtype == PTX_BF16 ? 2 : 4; }
+
+bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
+
+#define PTX_REQUIRE(cond, code, ...) \
+  do {                               \
+    if (!(cond)) return fail(code, __VA_ARGS__); \
+  } while (0)
+
+#define PTX_DISPATCH(dtype, CALL)        \
+  do {                                   \
+    if ((dtype) == PTX_BF16) {           \
+      typedef ptx::bf16_t T;             \
+      CALL;                              \
+    } else {                             \
+      typedef float T;                   \
+      CALL;                              \
+    }                                    \
+  } while (0)
+
+}  // namespace
+
+extern "C" {
+
+PTX_API int ptx_version(void) { return PTX_ABI_VERSION; }
+
+PTX_API const char* ptx_last_error_string(void) { return g_err; }
+
+PTX_API int ptx_key_pitch(int n) { return n <= 0 ? 0 : ((n + 63) / 64) * 64; }
+
+PTX_API int ptx_layernorm_fwd(const void* x, const void* gamma, const void* beta, void* y, float* mean,
+                      float* rstd, int64_t rows, int cols, float eps, int dtype, void* stream) {
+  PTX_REQUIRE(dtype_ok(dtype), PTX_ERR_BAD_ARG, "layernorm: unknown dtype %d", dtype);
+  PTX_REQUIRE(rows >= 0 && cols > 0, PTX_ERR_BAD_ARG, "layernorm: rows=%lld cols=%d",
+              (long long)rows, cols);
+  if (rows == 0) return PTX_OK;
+  PTX_REQUIRE(x && y, PTX_ERR_BAD_ARG, "layernorm: null x or y");
+  PTX_REQUIRE(rows < ((int64_t)1 << 31), PTX_ERR_UNSUPPORTED, "layernorm: rows=%lld too large",
+              (long long)rows);
+  PTX_DISPATCH(dtype, ptx::layernorm_fwd<T>((const T*)x, (const T*)gamma, (const T*)beta, (T*)y,
+                                            mean, rstd, rows, cols, eps, (hipStream_t)stream));
+  return after_launch("layernorm");
+}
+
+PTX_API int ptx_trimul_project(const void* z, const void* mask, const void* ln_w, const void* ln_b,
+                       const void* w_ap, const void* w_ag, const void* w_bp, const void* w_bg,
+                       void* a, void* b, int n, int c_z, int c_hidden, int k_pitch, int incoming,
+                       float eps, int dtype, void* stream) {
+  PTX_REQUIRE(dtype_ok(dtype), PTX_ERR_BAD_ARG, "trimul_project: unknown dtype %d", dtype);
+  PTX_REQUIRE(n >= 0, PTX_ERR_BAD_ARG, "trimul_project: n=%d", n);
+  PTX_REQUIRE(c_z == 128 && c_hidden == 128, PTX_ERR_UNSUPPORTED,
+              "trimul_project: only c_z = c_hidden = 128 is built (got %d, %d)", c_z, c_hidden);
+  PTX_REQUIRE(k_pitch == ptx_key_pitch(n), PTX_ERR_BAD_ARG,
+              "trimul_project: k_pitch=%d, expected ptx_key_pitch(%d)=%d", k_pitch, n,
+              ptx_key_pitch(n));
+  PTX_REQUIRE(n < 32768, PTX_ERR_UNSUPPORTED, "trimul_project: n=%d too large", n);
+  if (n == 0) return PTX_OK;
+  PTX_REQUIRE(z && w_ap && w_ag && w_bp && w_bg && a && b, PTX_ERR_BAD_ARG,
+              "trimul_project: null pointer");
+  PTX_REQUIRE(aligned16(z) && aligned16(w_ap) && aligned16(w_ag) && aligned16(w_bp) &&
+                  aligned16(w_bg) && (!ln_w || aligned16(ln_w)) && (!ln_b || aligned16(ln_b)),
+              PTX_ERR_BAD_ARG, "trimul_project: pointers must be 16-byte aligned");
+  PTX_DISPATCH(dtype, ptx::trimul_project<T>(z, mask, ln_w, ln_b, w_ap, w_ag, w_bp, w_bg, a, b, n,
+                                             k_pitch, incoming, eps, (hipStream_t)stream));
+  return after_launch("trimul_project");
+}
+
+PTX_API int ptx_trimul_contract(const void* a, const void* b, void* x, int n, int c, int k_pitch, int dtype,
+                        void* stream) {
+  PTX_REQUIRE(dtype_ok(dtype), PTX_ERR_BAD_ARG, "trimul_contract: unknown dtype %d", dtype);
+  PTX_REQUIRE(n >= 0 && c >= 0, PTX_ERR_BAD_ARG, "trimul_contract: n=%d c=%d", n, c);
+  PTX_REQUIRE(k_pitch == ptx_key_pitch(n), PTX_ERR_BAD_ARG,
+              "trimul_contract: k_pitch=%d, expected %d", k_pitch, ptx_key_pitch(n));
+  PTX_REQUIRE(n < 32768, PTX_ERR_UNSUPPORTED, "trimul_contract: n=%d too large", n);
+  if (n == 0 || c == 0) return PTX_OK;
+  PTX_REQUIRE(a && b && x, PTX_ERR_BAD_ARG, "trimul_contract: null pointer");
+  PTX_REQUIRE(aligned16(a) && aligned16(b), PTX_ERR_BAD_ARG,
+              "trimul_contract: a and b must be 16-byte aligned");
+  PTX_DISPATCH(dtype, ptx::nt_gemm_batched<T>((const T*)a, (const T*)b, (T*)x, n, k_pitch, c,
+                                              (hipStream_t)stream));
+  return after_launch("trimul_contract");
+}
+
+PTX_API int ptx_trimul_output(const void* x, const void* z, const void* ln_in_w, const void* ln_in_b,
+                      const void* ln_out_w, const void* ln_out_b, const void* w_z,
+                      const void* w_g, void* out, int n, int c_z, int c_hidden, int add_residual,
+                      float eps, int dtype, void* stream) {
+  PTX_REQUIRE(dtype_ok(dtype), PTX_ERR_BAD_ARG, "trimul_output: unknown dtype %d", dtype);
+  PTX_REQUIRE(n >= 0, PTX_ERR_BAD_ARG, "trimul_output: n=%d", n);
+  PTX_REQUIRE(c_z == 128 && c_hidden == 128, PTX_ERR_UNSUPPORTED,
+              "trimul_output: only c_z = c_hidden = 128 is built (got %d, %d)", c_z, c_hidden);
+  PTX_REQUIRE(n < 32768, PTX_ERR_UNSUPPORTED, "trimul_output: n=%d too large", n);
+  if (n == 0) return PTX_OK;
+  PTX_REQUIRE(x && z && ln_out_w && ln_out_b && w_z && w_g && out, PTX_ERR_BAD_ARG,
+              "trimul_output: null pointer");
+  PTX_REQUIRE(aligned16(z) && aligned16(w_z) && aligned16(w_g) && aligned16(ln_out_w) &&
+                  aligned16(ln_out_b) && (!ln_in_w || aligned16(ln_in_w)) &&
+                  (!ln_in_b || aligned16(ln_in_b)),
+              PTX_ERR_BAD_ARG, "trimul_output: pointers must be 16-byte aligned");
+  PTX_DISPATCH(dtype, ptx::trimul_output<T>(x, z, ln_in_w, ln_in_b, ln_out_w, ln_out_b, w_z, w_g,
+                                            out, n, add_residual, eps, (hipStream_t)stream));
+  return after_launch("trimul_output");
+}
+
+PTX_API int ptx_triattn_project(const void* z, const void* ln_w, const void* ln_b, const void* w_q,
+                        const void* w_k, const void* w_v, const void* w_g, const void* w_b,
+                        void* q, void* k, void* vt, void* g, void* tri_bias, int n, int c_in,
+                        int heads, int d, int key_pitch, int transposed, float eps, int dtype,
+                        void* stream) {
+  PTX_REQUIRE(dtype_ok(dtype), PTX_ERR_BAD_ARG, "triattn_project: unknown dtype %d", dtype);
+  PTX_REQUIRE(n >= 0, PTX_ERR_BAD_ARG, "triattn_project: n=%d", n);
+  PTX_REQUIRE(c_in == 128 && d == 32 && heads == 4, PTX_ERR_UNSUPPORTED,
+              "triattn_project: only c_in=128, 4 heads x 32 is built (got c_in=%d heads=%d d=%d)",
+              c_in, heads, d);
+  PTX_REQUIRE(key_pitch == ptx_key_pitch(n), PTX_ERR_BAD_ARG,
+              "triattn_project: key_pitch=%d, expected %d", key_pitch, ptx_key_pitch(n));
+  PTX_REQUIRE(n < 32768, PTX_ERR_UNSUPPORTED, "triattn_project: n=%d too large", n);
+  if (n == 0) return PTX_OK;
+  PTX_REQUIRE(z && w_q && w_k && w_v && w_g && w_b && q && k && vt && g && tri_bias,
+              PTX_ERR_BAD_ARG, "triattn_project: null pointer");
+  PTX_REQUIRE(aligned16(z) && aligned16(w_q) && aligned16(w_k) && aligned16(w_v) &&
+                  aligned16(w_g) && aligned16(w_b) && (!ln_w || aligned16(ln_w)) &&
+                  (!ln_b || aligned16(ln_b)),
+              PTX_ERR_BAD_ARG, "triattn_project: pointers must be 16-byte aligned");
+  PTX_DISPATCH(dtype, ptx::triattn_project<T>(z, ln_w, ln_b, w_q, w_k, w_v, w_g, w_b, q, k, vt, g,
+                                              tri_bias, n, heads, d, key_pitch, transposed, eps,
+                                              (hipStream_t)stream));
+  return after_launch("triattn_project");
+}
+
+PTX_API int ptx_triattn_fwd(const void* q, const void* k, const void* vt, const void* g,
+                    const void* tri_bias, const void* mask, void* o, int n, int heads, int d,
+                    int key_pitch, int mask_transposed, float inf, int dtype, void* stream) {
+  PTX_REQUIRE(dtype_ok(dtype), PTX_ERR_BAD_ARG, "triattn_fwd: unknown dtype %d", dtype);
+  PTX_REQUIRE(n >= 0 && heads >= 0, PTX_ERR_BAD_ARG, "triattn_fwd: n=%d heads=%d", n, heads);
+  PTX_REQUIRE(d == 32, PTX_ERR_UNSUPPORTED, "triattn_fwd: only head dim 32 is built (got %d)", d);
+  PTX_REQUIRE(key_pitch == ptx_key_pitch(n), PTX_ERR_BAD_ARG,
+              "triattn_fwd: key_pitch=%d, expected %d", key_pitch, ptx_key_pitch(n));
+  PTX_REQUIRE(n < 32768, PTX_ERR_UNSUPPORTED, "triattn_fwd: n=%d too large", n);
+  if (n == 0 || heads == 0) return PTX_OK;
+  PTX_REQUIRE(q && k && vt && g && tri_bias && o, PTX_ERR_BAD_ARG, "triattn_fwd: null pointer");
+  PTX_REQUIRE(aligned16(q) && aligned16(k) && aligned16(vt) && aligned16(g) &&
+                  aligned16(tri_bias) && aligned16(o),
+              PTX_ERR_BAD_ARG, "triattn_fwd: pointers must be 16-byte aligned");
+  PTX_DISPATCH(dtype, ptx::triattn_fwd<T>((const T*)q, (const T*)k, (const T*)vt, (const T*)g,
+                                          (const T*)tri_bias, (const T*)mask, (T*)o, n, heads,
+                                          key_pitch, mask_transposed, inf, (hipStream_t)stream));
+  return after_launch("triattn_fwd");
+}
+
+PTX_API int ptx_triattn_output(const void* o, const void* w_o, const void* z, void* out, int n, int c_in,
+                       int transposed, int add_residual, int dtype, void* stream) {
+  PTX_REQUIRE(dtype_ok(dtype), PTX_ERR_BAD_ARG, "triattn_output: unknown dtype %d", dtype);
+  PTX_REQUIRE(n >= 0, PTX_ERR_BAD_ARG, "triattn_output: n=%d", n);
+  PTX_REQUIRE(c_in == 128, PTX_ERR_UNSUPPORTED, "triattn_output: only c_in=128 is built (got %d)",
+              c_in);
+  PTX_REQUIRE(n < 32768, PTX_ERR_UNSUPPORTED, "triattn_output: n=%d too large", n);
+  if (n == 0) return PTX_OK;
+  PTX_REQUIRE(o && w_o && out && (!add_residual || z), PTX_ERR_BAD_ARG,
+              "triattn_output: null pointer");
+  PTX_REQUIRE(aligned16(o) && aligned16(w_o), PTX_ERR_BAD_ARG,
+              "triattn_output: pointers must be 16-byte aligned");
+  PTX_DISPATCH(dtype, ptx::triattn_output<T>(o, w_o, z, out, n, transposed, add_residual,
+                                             (hipStream_t)stream));
+  return after_launch("triattn_output");
+}
+
+PTX_API int ptx_transition_fwd(const void* x, const void* ln_w, const void* ln_b, const void* w_a,
+                       const void* w_b, const void* w_o, void* hidden, void* out, int64_t rows,
+                       int c, int n_factor, int add_residual, float eps, int dtype,
+                       void* stream) {
+  PTX_REQUIRE(dtype_ok(dtype), PTX_ERR_BAD_ARG, "transition: unknown dtype %d", dtype);
+  PTX_REQUIRE(rows >= 0 && n_factor > 0, PTX_ERR_BAD_ARG, "transition: rows=%lld n_factor=%d",
+              (long long)rows, n_factor);
+  PTX_REQUIRE(c == 128, PTX_ERR_UNSUPPORTED, "transition: only c=128 is built (got %d)", c);
+  PTX_REQUIRE(rows < ((int64_t)1 << 30), PTX_ERR_UNSUPPORTED, "transition: rows=%lld too large",
+              (long long)rows);
+  if (rows == 0) return PTX_OK;
+  PTX_REQUIRE(x && w_a && w_b && w_o && hidden && out, PTX_ERR_BAD_ARG,
+              "transition: null pointer");
+  PTX_REQUIRE(aligned16(x) && aligned16(w_a) && aligned16(w_b) && aligned16(w_o) &&
+                  aligned16(hidden) && (!ln_w || aligned16(ln_w)) && (!ln_b || aligned16(ln_b)),
+              PTX_ERR_BAD_ARG, "transition: pointers must be 16-byte aligned");
+  PTX_DISPATCH(dtype, ptx::transition_fwd<T>(x, ln_w, ln_b, w_a, w_b, w_o, hidden, out, rows,
+                                             n_factor, add_residual, eps, (hipStream_t)stream));
+  return after_launch("transition");
+}
+
+PTX_API int ptx_pair_bias_fwd(const void* z, const void* ln_w, const void* ln_b, const void* w, void* bias,
+                      int n, int c_z, int heads, int out_f32, float eps, int dtype,
+                      void* stream) {
+  PTX_REQUIRE(dtype_ok(dtype), PTX_ERR_BAD_ARG, "pair_bias: unknown dtype %d", dtype);
+  PTX_REQUIRE(n >= 0, PTX_ERR_BAD_ARG, "pair_bias: n=%d", n);
+  PTX_REQUIRE(c_z == 128, PTX_ERR_UNSUPPORTED, "pair_bias: only c_z=128 is built (got %d)", c_z);
+  PTX_REQUIRE(heads >= 1 && heads <= 32, PTX_ERR_UNSUPPORTED,
+              "pair_bias: heads=%d outside 1..32", heads);
+  PTX_REQUIRE(n < 32768, PTX_ERR_UNSUPPORTED, "pair_bias: n=%d too large", n);
+  if (n == 0) return PTX_OK;
+  PTX_REQUIRE(z && w && bias, PTX_ERR_BAD_ARG, "pair_bias: null pointer");
+  PTX_REQUIRE(aligned16(z) && aligned16(w) && (!ln_w || aligned16(ln_w)) &&
+                  (!ln_b || aligned16(ln_b)),
+              PTX_ERR_BAD_ARG, "pair_bias: pointers must be 16-byte aligned");
+  PTX_DISPATCH(dtype, ptx::pair_bias_fwd<T>(z, ln_w, ln_b, w, bias, n, heads, out_f32, eps,
+                                            (hipStream_t)stream));
+  return after_launch("pair_bias");
+}
+
+}  // extern "C"

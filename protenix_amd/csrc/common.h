@@ -1,0 +1,109 @@
+// Shared device helpers for the gfx950 (CDNA4) Pairformer pair-stack kernels.
+//
+// MFMA convention used by every kernel in this directory ("mma32"):
+//   acc[32 x 32] += A[32 x 16] * B[16 x 32]
+//   lane l supplies row    m = l % 32 of A, K-slots 8*(l/32) .. 8*(l/32)+7
+//   lane l supplies column n = l % 32 of B, the same K-slots
+//   lane l receives column n = l % 32 of acc; register r holds row
+//        8*(r/4) + 4*(l/32) + (r%4)
+// An operand "fragment" is therefore 8 consecutive K elements per lane, for
+// bf16 (one v_mfma_f32_32x32x16_bf16) and for fp32 (eight
+// v_mfma_f32_32x32x2_f32, slot t of both operands per instruction).  Because
+// both operands use the same slot numbering, which physical K index a slot
+// stands for is the kernel's choice.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace ptx {
+
+typedef __bf16 bf16_t;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(2))) float f32x2;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(8))) float f32x8;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+
+constexpr int kWave = 64;
+
+template <typename T> struct Vec8;
+template <> struct Vec8<bf16_t> { typedef bf16x8 type; };
+template <> struct Vec8<float> { typedef f32x8 type; };
+template <typename T> struct Vec4;
+template <> struct Vec4<bf16_t> { typedef bf16x4 type; };
+template <> struct Vec4<float> { typedef f32x4 type; };
+
+__device__ __forceinline__ f32x8 to_f32(bf16x8 v) { return __builtin_convertvector(v, f32x8); }
+__device__ __forceinline__ f32x8 to_f32(f32x8 v) { return v; }
+__device__ __forceinline__ f32x4 to_f32(bf16x4 v) { return __builtin_convertvector(v, f32x4); }
+__device__ __forceinline__ f32x4 to_f32(f32x4 v) { return v; }
+__device__ __forceinline__ float to_f32(bf16_t v) { return (float)v; }
+__device__ __forceinline__ float to_f32(float v) { return v; }
+
+template <typename T> __device__ __forceinline__ typename Vec8<T>::type from_f32(f32x8 v);
+template <> __device__ __forceinline__ bf16x8 from_f32<bf16_t>(f32x8 v) { return __builtin_convertvector(v, bf16x8); }
+template <> __device__ __forceinline__ f32x8 from_f32<float>(f32x8 v) { return v; }
+template <typename T> __device__ __forceinline__ typename Vec4<T>::type from_f32(f32x4 v);
+template <> __device__ __forceinline__ bf16x4 from_f32<bf16_t>(f32x4 v) { return __builtin_convertvector(v, bf16x4); }
+template <> __device__ __forceinline__ f32x4 from_f32<float>(f32x4 v) { return v; }
+template <typename T> __device__ __forceinline__ T from_f32(float v);
+template <> __device__ __forceinline__ bf16_t from_f32<bf16_t>(float v) { return (bf16_t)v; }
+template <> __device__ __forceinline__ float from_f32<float>(float v) { return v; }
+
+// acc += A * B for one 16-deep K step (see the convention above).
+__device__ __forceinline__ void mma32(f32x16& acc, bf16x8 a, bf16x8 b) {
+  acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc, 0, 0, 0);
+}
+__device__ __forceinline__ void mma32(f32x16& acc, f32x8 a, f32x8 b) {
+#pragma unroll
+  for (int t = 0; t < 8; ++t) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[t], b[t], acc, 0, 0, 0);
+}
+
+// Row of acc held by register r of a lane in half-wave g (= lane / 32).
+__device__ __forceinline__ int acc_row(int r, int g) { return 8 * (r >> 2) + 4 * g + (r & 3); }
+
+// Value of the lane 32 places away (the other half-wave).
+__device__ __forceinline__ float swap32(float v) { return __shfl_xor(v, 32, 64); }
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
+// sigmoid(x) = 1 / (1 + 2^(-x*log2 e)); |rel err| ~ 1e-7, saturates cleanly at +-inf.
+__device__ __forceinline__ float sigmoidf_fast(float x) {
+  return fast_rcp(1.0f + fast_exp2(-1.4426950408889634f * x));
+}
+
+// 16-byte (8 x bf16) or 32-byte (8 x fp32) global accesses.
+template <typename T>
+__device__ __forceinline__ typename Vec8<T>::type load8(const T* p) {
+  return *reinterpret_cast<const typename Vec8<T>::type*>(p);
+}
+template <typename T>
+__device__ __forceinline__ void store8(T* p, typename Vec8<T>::type v) {
+  *reinterpret_cast<typename Vec8<T>::type*>(p) = v;
+}
+template <typename T>
+__device__ __forceinline__ typename Vec8<T>::type zero8() {
+  typename Vec8<T>::type z;
+#pragma unroll
+  for (int t = 0; t < 8; ++t) z[t] = (T)0.0f;
+  return z;
+}
+
+// Position of a logical pair-tensor row p = outer * n_inner + inner in a tensor
+// whose (outer, inner) axes have arbitrary element strides.  The ending-node
+// attention and the incoming triangle product read z[inner, outer] this way,
+// so no transposed copy of the pair tensor is ever made.
+struct RowMap {
+  int64_t stride_outer;
+  int64_t stride_inner;
+  int n_inner;
+  __device__ __forceinline__ int64_t operator()(int64_t p) const {
+    int64_t o = p / n_inner;
+    int64_t i = p - o * n_inner;
+    return o * stride_outer + i * stride_inner;
+  }
+};
+
+}  // namespace ptx

@@ -1,0 +1,49 @@
+// Host-callable launchers, one per kernel family; api.hip validates arguments
+// and dispatches on dtype.  All return 0 after enqueueing on `stream`.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace ptx {
+
+template <typename T>
+int layernorm_fwd(const T* x, const T* gamma, const T* beta, T* y, float* mean, float* rstd,
+                  int64_t rows, int cols, float eps, hipStream_t stream);
+
+template <typename T>
+int trimul_project(const void* z, const void* mask, const void* ln_w, const void* ln_b,
+                   const void* w_ap, const void* w_ag, const void* w_bp, const void* w_bg, void* a,
+                   void* b, int n, int k_pitch, int incoming, float eps, hipStream_t stream);
+template <typename T>
+int trimul_output(const void* x, const void* z, const void* ln_in_w, const void* ln_in_b,
+                  const void* ln_out_w, const void* ln_out_b, const void* w_z, const void* w_g,
+                  void* out, int n, int add_residual, float eps, hipStream_t stream);
+template <typename T>
+int triattn_project(const void* z, const void* ln_w, const void* ln_b, const void* w_q,
+                    const void* w_k, const void* w_v, const void* w_g, const void* w_b, void* q,
+                    void* k, void* vt, void* g, void* tri_bias, int n, int heads, int d,
+                    int key_pitch, int transposed, float eps, hipStream_t stream);
+template <typename T>
+int triattn_output(const void* o, const void* w_o, const void* z, void* out, int n, int transposed,
+                   int add_residual, hipStream_t stream);
+template <typename T>
+int transition_fwd(const void* x, const void* ln_w, const void* ln_b, const void* w_a,
+                   const void* w_b, const void* w_o, void* hidden, void* out, int64_t rows,
+                   int n_factor, int add_residual, float eps, hipStream_t stream);
+template <typename T>
+int pair_bias_fwd(const void* z, const void* ln_w, const void* ln_b, const void* w, void* bias,
+                  int n, int heads, int out_f32, float eps, hipStream_t stream);
+
+// x[c][i][j] = sum_k a[c][i][k] * b[c][j][k] for `batch` independent products;
+// a, b rows have pitch k_pitch (a multiple of 64, >= n), x is dense [batch][n][n].
+template <typename T>
+int nt_gemm_batched(const T* a, const T* b, T* x, int n, int k_pitch, int batch,
+                    hipStream_t stream);
+
+// Flash-style triangle attention core (see triattn.hip).
+template <typename T>
+int triattn_fwd(const T* q, const T* k, const T* vt, const T* g, const T* tri_bias, const T* mask,
+                T* o, int n, int heads, int key_pitch, int mask_transposed, float inf,
+                hipStream_t stream);
+
+}  // namespace ptx

@@ -1,0 +1,65 @@
+"""LayerNorm over the last dimension on the HIP kernel.
+
+Mirrors protenix/model/layer_norm/layer_norm.py:190-233 (FusedLayerNorm) and
+the factory protenix/model/triangular/layers.py:246-256: parameters `weight`
+and `bias` (either may be absent), fp32 statistics, gamma/beta cast to the
+input dtype, output in the input dtype.  Forward only.
+"""
+from __future__ import annotations
+
+import numbers
+from typing import Optional, Union
+
+import torch
+import torch.nn as nn
+
+from . import ops
+
+
+def _forward_only(*tensors: Optional[torch.Tensor]) -> None:
+    if torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in tensors):
+        raise RuntimeError(
+            "protenix_amd kernels are forward-only: call under torch.no_grad() "
+            "(backward kernels are not part of this build)")
+
+
+class FusedLayerNorm(nn.Module):
+    def __init__(self, normalized_shape: Union[int, list, torch.Size], create_scale: bool = True,
+                 create_offset: bool = True, eps: float = 1e-5) -> None:
+        super().__init__()
+        if isinstance(normalized_shape, numbers.Integral):
+            normalized_shape = (normalized_shape,)
+        self.normalized_shape = torch.Size(normalized_shape)
+        if len(self.normalized_shape) != 1:
+            raise ValueError("FusedLayerNorm normalises over the last dimension only")
+        self.eps = eps
+        if create_scale:
+            self.weight = nn.Parameter(torch.ones(*normalized_shape))
+        else:
+            self.register_parameter("weight", None)
+        if create_offset:
+            self.bias = nn.Parameter(torch.zeros(*normalized_shape))
+        else:
+            self.register_parameter("bias", None)
+
+    def reset_parameters(self) -> None:
+        if self.weight is not None:
+            nn.init.ones_(self.weight)
+        if self.bias is not None:
+            nn.init.zeros_(self.bias)
+
+    def forward(self, input: torch.Tensor) -> torch.Tensor:  # noqa: A002
+        if input.shape[-1] != self.normalized_shape[0]:
+            raise RuntimeError(
+                f"expected last dimension {self.normalized_shape[0]}, got {tuple(input.shape)}")
+        _forward_only(input, self.weight, self.bias)
+        return ops.layer_norm(input, self.weight, self.bias, self.eps)
+
+    def extra_repr(self) -> str:
+        return f"{tuple(self.normalized_shape)}, eps={self.eps}"
+
+
+def LayerNorm(c_in: int, create_scale: bool = True, create_offset: bool = True,
+              eps: float = 1e-5) -> nn.Module:
+    """Same call as the reference factory (layers.py:246-256)."""
+    return FusedLayerNorm(c_in, create_scale=create_scale, create_offset=create_offset, eps=eps)

@@ -1,0 +1,185 @@
+"""Tensor-level wrappers over the C ABI: validate, allocate outputs and
+workspaces with torch, pass raw device pointers and the current HIP stream."""
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+
+from . import _lib
+
+_DTYPES = {torch.float32: _lib.PTX_F32, torch.bfloat16: _lib.PTX_BF16}
+
+
+def _dt(t: torch.Tensor) -> int:
+    try:
+        return _DTYPES[t.dtype]
+    except KeyError:
+        raise RuntimeError(f"protenix_amd kernels take float32 or bfloat16 tensors, got {t.dtype}")
+
+
+def _dev(t: torch.Tensor, name: str) -> None:
+    if not t.is_cuda:
+        raise RuntimeError(
+            f"protenix_amd: `{name}` is on {t.device}; the HIP kernels need a GPU tensor "
+            "(there is no CPU fallback)")
+
+
+def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _same(t: Optional[torch.Tensor], like: torch.Tensor, name: str) -> Optional[torch.Tensor]:
+    """Parameter tensor in the activation dtype/device, contiguous."""
+    if t is None:
+        return None
+    if t.dtype != like.dtype or t.device != like.device:
+        t = t.to(device=like.device, dtype=like.dtype)
+    return t.contiguous()
+
+
+def key_pitch(n: int) -> int:
+    return _lib.load().ptx_key_pitch(n)
+
+
+def layer_norm(x: torch.Tensor, weight: Optional[torch.Tensor], bias: Optional[torch.Tensor],
+               eps: float = 1e-5, return_stats: bool = False):
+    """LayerNorm over the last dim (reference: layer_norm.py:70-112)."""
+    _dev(x, "input")
+    lib = _lib.load()
+    x = x.contiguous()
+    cols = x.shape[-1]
+    rows = x.numel() // cols if cols else 0
+    w = _same(weight, x, "weight")
+    b = _same(bias, x, "bias")
+    y = torch.empty_like(x)
+    mean = rstd = None
+    if return_stats:
+        mean = torch.empty(rows, dtype=torch.float32, device=x.device)
+        rstd = torch.empty(rows, dtype=torch.float32, device=x.device)
+    with torch.cuda.device(x.device):
+        _lib.check(lib.ptx_layernorm_fwd(_ptr(x), _ptr(w), _ptr(b), _ptr(y), _ptr(mean), _ptr(rstd),
+                                         rows, cols, eps, _dt(x), _stream()), "layernorm")
+    return (y, mean, rstd) if return_stats else y
+
+
+def _mask_for(mask: Optional[torch.Tensor], z: torch.Tensor) -> Optional[torch.Tensor]:
+    if mask is None:
+        return None
+    return mask.to(device=z.device, dtype=z.dtype).contiguous()
+
+
+def triangle_multiplication(z: torch.Tensor, mask: Optional[torch.Tensor], w: dict, incoming: bool,
+                            add_residual: bool, out: Optional[torch.Tensor] = None,
+                            eps: float = 1e-5) -> torch.Tensor:
+    """One [N, N, c_z] pair tensor through project -> contract -> output.
+    `w` holds the parameters already in z's dtype (see triangular.py)."""
+    _dev(z, "z")
+    lib = _lib.load()
+    n, c_z = z.shape[0], z.shape[-1]
+    c_h = w["w_ap"].shape[0]
+    dt, st = _dt(z), _stream()
+    pitch = key_pitch(n)
+    mask = _mask_for(mask, z)
+    a = torch.empty((c_h, n, pitch), dtype=z.dtype, device=z.device)
+    b = torch.empty((c_h, n, pitch), dtype=z.dtype, device=z.device)
+    with torch.cuda.device(z.device):
+        _lib.check(lib.ptx_trimul_project(
+            _ptr(z), _ptr(mask), _ptr(w["ln_in_w"]), _ptr(w["ln_in_b"]), _ptr(w["w_ap"]),
+            _ptr(w["w_ag"]), _ptr(w["w_bp"]), _ptr(w["w_bg"]), _ptr(a), _ptr(b), n, c_z, c_h, pitch,
+            int(incoming), eps, dt, st), "trimul_project")
+        x = torch.empty((c_h, n, n), dtype=z.dtype, device=z.device)
+        _lib.check(lib.ptx_trimul_contract(_ptr(a), _ptr(b), _ptr(x), n, c_h, pitch, dt, st),
+                   "trimul_contract")
+        del a, b
+        if out is None:
+            out = torch.empty_like(z)
+        _lib.check(lib.ptx_trimul_output(
+            _ptr(x), _ptr(z), _ptr(w["ln_in_w"]), _ptr(w["ln_in_b"]), _ptr(w["ln_out_w"]),
+            _ptr(w["ln_out_b"]), _ptr(w["w_z"]), _ptr(w["w_g"]), _ptr(out), n, c_z, c_h,
+            int(add_residual), eps, dt, st), "trimul_output")
+    return out
+
+
+def triangle_attention(z: torch.Tensor, mask: Optional[torch.Tensor], w: dict, heads: int, d: int,
+                       inf: float, transposed: bool, add_residual: bool,
+                       out: Optional[torch.Tensor] = None, eps: float = 1e-5) -> torch.Tensor:
+    """Starting-node attention over z (transposed=False) or over z^T with the
+    result written back transposed (transposed=True), i.e. the ending node as
+    the Pairformer block uses it, without materialising z^T.  `mask` is indexed
+    like z: the key mask of logical row i is mask[i, :] (or mask[:, i])."""
+    _dev(z, "z")
+    lib = _lib.load()
+    n, c = z.shape[0], z.shape[-1]
+    dt, st = _dt(z), _stream()
+    pitch = key_pitch(n)
+    mask = _mask_for(mask, z)
+    hd = heads * d
+    dev = z.device
+    q = torch.empty((n, n, hd), dtype=z.dtype, device=dev)
+    k = torch.empty((n, n, hd), dtype=z.dtype, device=dev)
+    g = torch.empty((n, n, hd), dtype=z.dtype, device=dev)
+    vt = torch.empty((n, hd, pitch), dtype=z.dtype, device=dev)
+    tb = torch.empty((heads, n, pitch), dtype=z.dtype, device=dev)
+    with torch.cuda.device(dev):
+        _lib.check(lib.ptx_triattn_project(
+            _ptr(z), _ptr(w["ln_w"]), _ptr(w["ln_b"]), _ptr(w["w_q"]), _ptr(w["w_k"]), _ptr(w["w_v"]),
+            _ptr(w["w_g"]), _ptr(w["w_b"]), _ptr(q), _ptr(k), _ptr(vt), _ptr(g), _ptr(tb), n, c,
+            heads, d, pitch, int(transposed), eps, dt, st), "triattn_project")
+        # o overwrites g: each element of g is read once, by the thread that then writes o there
+        _lib.check(lib.ptx_triattn_fwd(_ptr(q), _ptr(k), _ptr(vt), _ptr(g), _ptr(tb), _ptr(mask),
+                                       _ptr(g), n, heads, d, pitch, int(transposed), float(inf), dt,
+                                       st), "triattn_fwd")
+        del q, k, vt, tb
+        if out is None:
+            out = torch.empty_like(z)
+        _lib.check(lib.ptx_triattn_output(_ptr(g), _ptr(w["w_o"]), _ptr(z), _ptr(out), n, c,
+                                          int(transposed), int(add_residual), dt, st),
+                   "triattn_output")
+    return out
+
+
+def transition(x: torch.Tensor, w: dict, n_factor: int, add_residual: bool,
+               out: Optional[torch.Tensor] = None, eps: float = 1e-5,
+               max_rows: int = 1 << 21) -> torch.Tensor:
+    """x [..., 128] -> [x +] W_o(silu(W_a LN x) * W_b LN x), rows processed in
+    slabs of `max_rows` so the hidden workspace stays bounded."""
+    _dev(x, "x")
+    lib = _lib.load()
+    c = x.shape[-1]
+    x2 = x.reshape(-1, c)
+    if not x2.is_contiguous():
+        x2 = x2.contiguous()
+    rows = x2.shape[0]
+    dt, st = _dt(x), _stream()
+    if out is None:
+        out = torch.empty_like(x2)
+    o2 = out.view(-1, c)
+    slab = min(rows, max_rows)
+    hidden = torch.empty((slab, n_factor * c), dtype=x.dtype, device=x.device)
+    with torch.cuda.device(x.device):
+        for r0 in range(0, rows, slab):
+            r1 = min(rows, r0 + slab)
+            _lib.check(lib.ptx_transition_fwd(
+                _ptr(x2[r0:r1]), _ptr(w["ln_w"]), _ptr(w["ln_b"]), _ptr(w["w_a"]), _ptr(w["w_b"]),
+                _ptr(w["w_o"]), _ptr(hidden), _ptr(o2[r0:r1]), r1 - r0, c, n_factor,
+                int(add_residual), eps, dt, st), "transition")
+    return out.view(x.shape)
+
+
+def pair_bias(z: torch.Tensor, ln_w: Optional[torch.Tensor], ln_b: Optional[torch.Tensor],
+              w: torch.Tensor, out_f32: bool = True, eps: float = 1e-5) -> torch.Tensor:
+    """bias[h, i, j] = (W LN(z[i, j]))[h] for one [N, N, 128] pair tensor."""
+    _dev(z, "z")
+    lib = _lib.load()
+    n, c = z.shape[0], z.shape[-1]
+    heads = w.shape[0]
+    out = torch.empty((heads, n, n), dtype=torch.float32 if out_f32 else z.dtype, device=z.device)
+    with torch.cuda.device(z.device):
+        _lib.check(lib.ptx_pair_bias_fwd(_ptr(z), _ptr(ln_w), _ptr(ln_b), _ptr(w), _ptr(out), n, c,
+                                         heads, int(out_f32), eps, _dt(z), _stream()), "pair_bias")
+    return out

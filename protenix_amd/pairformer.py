@@ -1,0 +1,105 @@
+"""PairformerBlock / PairformerStack on the gfx950 kernels.
+
+Same constructor arguments, sub-module names (= state-dict keys) and forward
+signatures as protenix/model/modules/pairformer.py:42-340.  Eval / no-grad
+forward only.  The five pair updates of a block run as fused kernels that add
+their result into the pair tensor on the way out; the ending-node attention
+reads and writes the pair tensor through transposed addressing, so the two
+`transpose(-2, -3).contiguous()` copies of the reference (pairformer.py:201,
+214) do not exist here.
+"""
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+import torch.nn as nn
+
+from .primitives import Transition
+from .transformer import AttentionPairBias
+from .triangular import (TriangleAttention, TriangleMultiplicationIncoming,
+                         TriangleMultiplicationOutgoing)
+
+
+class PairformerBlock(nn.Module):
+    def __init__(self, n_heads: int = 16, c_z: int = 128, c_s: int = 384, c_hidden_mul: int = 128,
+                 c_hidden_pair_att: int = 32, no_heads_pair: int = 4,
+                 num_intermediate_factor: int = 4, dropout: float = 0.25,
+                 hidden_scale_up: bool = False) -> None:
+        super().__init__()
+        self.n_heads = n_heads
+        if hidden_scale_up:
+            no_heads_pair = c_z // c_hidden_pair_att
+            c_hidden_mul = c_z
+        self.tri_mul_out = TriangleMultiplicationOutgoing(c_z=c_z, c_hidden=c_hidden_mul)
+        self.tri_mul_in = TriangleMultiplicationIncoming(c_z=c_z, c_hidden=c_hidden_mul)
+        self.tri_att_start = TriangleAttention(c_in=c_z, c_hidden=c_hidden_pair_att,
+                                               no_heads=no_heads_pair)
+        self.tri_att_end = TriangleAttention(c_in=c_z, c_hidden=c_hidden_pair_att,
+                                             no_heads=no_heads_pair)
+        self.p_drop = dropout
+        self.pair_transition = Transition(c_in=c_z, n=num_intermediate_factor)
+        self.c_s = c_s
+        if self.c_s > 0:
+            self.attention_pair_bias = AttentionPairBias(has_s=False, create_offset_ln_z=True,
+                                                         n_heads=n_heads, c_a=c_s, c_z=c_z)
+            self.single_transition = Transition(c_in=c_s, n=4)
+
+    def forward(self, s: Optional[torch.Tensor], z: torch.Tensor, pair_mask: Optional[torch.Tensor],
+                triangle_multiplicative: str = "torch", triangle_attention: str = "torch",
+                inplace_safe: bool = False, chunk_size: Optional[int] = None
+                ) -> Tuple[Optional[torch.Tensor], torch.Tensor]:
+        """s [..., N, c_s] or None, z [..., N, N, c_z], pair_mask [..., N, N] or
+        None -> (s, z).  With `inplace_safe` z is updated in place, as the
+        reference's inference path does; otherwise the inputs are left untouched."""
+        if self.training:
+            raise RuntimeError("protenix_amd.PairformerBlock is inference-only: call .eval()")
+        if triangle_multiplicative not in ("torch", "cuequivariance"):
+            raise ValueError(
+                "triangle_multiplicative must be 'cuequivariance' or 'torch', but got "
+                f"{triangle_multiplicative}")
+        assert triangle_attention in ("torch", "deepspeed", "triattention", "cuequivariance")
+        if not inplace_safe or not z.is_contiguous():
+            z = z.clone(memory_format=torch.contiguous_format)
+        # every update below is "z += f(z)" fused into the kernel epilogues
+        self.tri_mul_out(z, mask=pair_mask, inplace_safe=True, _add_with_inplace=True)
+        self.tri_mul_in(z, mask=pair_mask, inplace_safe=True, _add_with_inplace=True)
+        self.tri_att_start._run(z, pair_mask, transposed=False, residual_inplace=True)
+        # ending node: the starting-node module of the reference applied to z^T with
+        # mask^T, expressed through transposed addressing of z and mask
+        self.tri_att_end._run(z, pair_mask, transposed=True, residual_inplace=True)
+        self.pair_transition(z, _residual_out=z)
+        if self.c_s > 0:
+            s = s + self.attention_pair_bias(a=s, s=None, z=z)
+            s = s + self.single_transition(s)
+        return s, z
+
+
+class PairformerStack(nn.Module):
+    def __init__(self, n_blocks: int = 48, n_heads: int = 16, c_z: int = 128, c_s: int = 384,
+                 num_intermediate_factor: int = 4, dropout: float = 0.25,
+                 blocks_per_ckpt: Optional[int] = None, hidden_scale_up: bool = False) -> None:
+        super().__init__()
+        self.n_blocks = n_blocks
+        self.n_heads = n_heads
+        self.blocks_per_ckpt = blocks_per_ckpt
+        self.blocks = nn.ModuleList()
+        for _ in range(n_blocks):
+            self.blocks.append(PairformerBlock(n_heads=n_heads, c_z=c_z, c_s=c_s,
+                                               num_intermediate_factor=num_intermediate_factor,
+                                               dropout=dropout, hidden_scale_up=hidden_scale_up))
+
+    def forward(self, s: torch.Tensor, z: torch.Tensor, pair_mask: Optional[torch.Tensor],
+                triangle_multiplicative: str = "torch", triangle_attention: str = "torch",
+                inplace_safe: bool = False, chunk_size: Optional[int] = None
+                ) -> Tuple[torch.Tensor, torch.Tensor]:
+        """Blocks in sequence (pairformer.py:291-340); activation checkpointing is
+        a training device and does nothing under no-grad, as in the reference."""
+        if not inplace_safe and len(self.blocks) > 0:
+            # one private copy for the whole stack; the blocks then work in place
+            z = z.clone(memory_format=torch.contiguous_format)
+        for blk in self.blocks:
+            s, z = blk(s, z, pair_mask, triangle_multiplicative=triangle_multiplicative,
+                       triangle_attention=triangle_attention, inplace_safe=True,
+                       chunk_size=chunk_size)
+        return s, z

@@ -1,0 +1,121 @@
+"""Linear layers and the SwiGLU Transition of the Pairformer block.
+
+Mirrors protenix/model/modules/primitives.py:33-101 (Linear / LinearNoBias),
+:166-230 (Transition) and protenix/model/triangular/layers.py:104-197
+(OpenfoldLinear, by its initialiser names).  The pair Transition (c_in = 128)
+runs on the fused HIP kernels; other widths (the single track, c_in = 384) use
+the HIP LayerNorm and library GEMMs.
+"""
+from __future__ import annotations
+
+import math
+from functools import partial
+from typing import Optional
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from . import ops
+from .layer_norm import LayerNorm, _forward_only
+
+
+def _trunc_normal_(w: torch.Tensor, scale: float) -> None:
+    fan_in = w.shape[1]
+    std = math.sqrt(scale / max(1, fan_in)) / 0.87962566103423978  # std of N(0,1) cut at +-2
+    nn.init.trunc_normal_(w, mean=0.0, std=std, a=-2.0 * std, b=2.0 * std)
+
+
+class Linear(nn.Linear):
+    """nn.Linear with the reference's initialisers: "default" (LeCun truncated
+    normal), "relu" (He), "zeros" / "final" / "gating" (weight 0; gating bias 1)."""
+
+    def __init__(self, in_features: int, out_features: int, bias: bool = True, device=None,
+                 dtype=None, precision: Optional[torch.dtype] = None,
+                 initializer: str = "default") -> None:
+        self.use_bias = bias
+        self.precision = precision
+        self.initializer = initializer
+        super().__init__(in_features, out_features, bias=bias, device=device, dtype=dtype)
+        self._init_params()
+
+    @torch.no_grad()
+    def _init_params(self) -> None:
+        if self.use_bias:
+            nn.init.zeros_(self.bias)
+        if self.initializer == "default":
+            _trunc_normal_(self.weight, 1.0)
+        elif self.initializer == "relu":
+            _trunc_normal_(self.weight, 2.0)
+        elif self.initializer in ("zeros", "final"):
+            nn.init.zeros_(self.weight)
+        elif self.initializer == "gating":
+            nn.init.zeros_(self.weight)
+            if self.use_bias:
+                nn.init.ones_(self.bias)
+        else:
+            raise ValueError(f"Invalid initializer: {self.initializer}.")
+
+    def forward(self, input: torch.Tensor) -> torch.Tensor:  # noqa: A002
+        d = input.dtype
+        cd = self.precision if self.precision is not None else d
+        b = self.bias.to(cd) if self.bias is not None else None
+        return F.linear(input.to(cd), self.weight.to(cd), b).to(d)
+
+
+LinearNoBias = partial(Linear, bias=False)
+
+
+class _WeightCache:
+    """Parameters converted once to the activation dtype/device; rebuilt when a
+    parameter is modified in place or replaced."""
+
+    def __init__(self) -> None:
+        self._key = None
+        self._val = None
+
+    def get(self, params, dtype, device, build):
+        key = (dtype, device) + tuple((id(p), p._version, p.data_ptr()) if p is not None else None
+                                      for p in params)
+        if key != self._key:
+            self._val = build()
+            self._key = key
+        return self._val
+
+
+def _cv(p: Optional[torch.Tensor], dtype, device) -> Optional[torch.Tensor]:
+    return None if p is None else p.detach().to(device=device, dtype=dtype).contiguous()
+
+
+class Transition(nn.Module):
+    def __init__(self, c_in: int, n: int) -> None:
+        super().__init__()
+        self.n = n
+        self.c_in = c_in
+        self.layernorm1 = LayerNorm(c_in)
+        self.linear_no_bias_a = LinearNoBias(c_in, n * c_in, initializer="relu")
+        self.linear_no_bias_b = LinearNoBias(c_in, n * c_in, initializer="relu")
+        self.linear_no_bias = LinearNoBias(n * c_in, c_in, initializer="zeros")
+        self._cache = _WeightCache()
+
+    def _weights(self, dtype, device) -> dict:
+        ps = (self.layernorm1.weight, self.layernorm1.bias, self.linear_no_bias_a.weight,
+              self.linear_no_bias_b.weight, self.linear_no_bias.weight)
+        return self._cache.get(ps, dtype, device, lambda: dict(
+            zip(("ln_w", "ln_b", "w_a", "w_b", "w_o"), (_cv(p, dtype, device) for p in ps))))
+
+    def forward(self, x: torch.Tensor, _residual_out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """Returns the update; with `_residual_out` (may be x itself) writes
+        x + update there instead and returns it."""
+        _forward_only(x, *self.parameters())
+        add = _residual_out is not None
+        if self.c_in == 128:
+            return ops.transition(x, self._weights(x.dtype, x.device), self.n, add_residual=add,
+                                  out=_residual_out)
+        # other widths: HIP LayerNorm + library GEMMs
+        y = self.layernorm1(x)
+        h = F.silu(self.linear_no_bias_a(y)) * self.linear_no_bias_b(y)
+        u = self.linear_no_bias(h)
+        if add:
+            return _residual_out.copy_(x + u) if _residual_out is not x else x.add_(u)
+        return u

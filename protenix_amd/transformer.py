@@ -1,0 +1,115 @@
+"""Single-representation attention with pair bias, the has_s=False flavour the
+Pairformer block uses (protenix/model/modules/transformer.py:40-254 with
+pairformer.py:98-100; attention arithmetic of primitives.py:233-291, 636-879).
+
+The only pass over the pair tensor - LayerNorm(z) followed by the c_z -> heads
+projection - runs on the fused HIP kernel and never materialises LN(z).  The
+rest lives on the [N, c_s] single track: HIP LayerNorm, library GEMMs, and an
+fp32 softmax over [heads, N, N].
+"""
+from __future__ import annotations
+
+import math
+from typing import Optional
+
+import torch
+import torch.nn as nn
+
+from . import ops
+from .layer_norm import LayerNorm, _forward_only
+from .primitives import Linear, LinearNoBias, _cv, _WeightCache
+
+
+class Attention(nn.Module):
+    """primitives.py:636-879 restricted to global attention with an additive
+    bias: q carries a bias, output gated by sigmoid(linear_g(q_x))."""
+
+    def __init__(self, c_q: int, c_k: int, c_v: int, c_hidden: int, num_heads: int,
+                 gating: bool = True, q_linear_bias: bool = True,
+                 local_attention_method: str = "global_attention_with_bias",
+                 use_efficient_implementation: bool = True, zero_init: bool = True) -> None:
+        super().__init__()
+        self.c_q, self.c_k, self.c_v = c_q, c_k, c_v
+        self.c_hidden = c_hidden
+        self.num_heads = num_heads
+        self.gating = gating
+        self.linear_q = Linear(c_q, c_hidden * num_heads, bias=q_linear_bias)
+        self.linear_k = LinearNoBias(c_k, c_hidden * num_heads)
+        self.linear_v = LinearNoBias(c_v, c_hidden * num_heads)
+        self.linear_o = LinearNoBias(c_hidden * num_heads, c_q)
+        self.linear_g = None
+        if gating:
+            self.linear_g = LinearNoBias(c_q, c_hidden * num_heads, initializer="zeros")
+            self.sigmoid = nn.Sigmoid()
+        self.zero_init = zero_init
+        if zero_init:
+            nn.init.zeros_(self.linear_o.weight)
+
+    def forward(self, q_x: torch.Tensor, kv_x: torch.Tensor,
+                attn_bias: Optional[torch.Tensor] = None, **_unused) -> torch.Tensor:
+        H = self.num_heads
+        q = self.linear_q(q_x).unflatten(-1, (H, -1)).transpose(-2, -3)
+        k = self.linear_k(kv_x).unflatten(-1, (H, -1)).transpose(-2, -3)
+        v = self.linear_v(kv_x).unflatten(-1, (H, -1)).transpose(-2, -3)
+        q = q / math.sqrt(self.c_hidden)
+        # logits, softmax and the weighted sum in fp32 (the reference upcasts q, k
+        # and the bias and relies on autocast for v; here v is upcast as well)
+        d = q.dtype
+        w = torch.matmul(q.float(), k.float().transpose(-1, -2))
+        if attn_bias is not None:
+            if attn_bias.dim() != w.dim():
+                attn_bias = attn_bias.unsqueeze(-3)
+            w = w + attn_bias.float()
+        w = torch.softmax(w, dim=-1)
+        o = torch.matmul(w, v.float()).to(d).transpose(-2, -3)
+        if self.linear_g is not None:
+            o = o * torch.sigmoid(self.linear_g(q_x)).unflatten(-1, (H, -1))
+        return self.linear_o(o.flatten(-2))
+
+
+class AttentionPairBias(nn.Module):
+    def __init__(self, has_s: bool = True, create_offset_ln_z: bool = False, n_heads: int = 16,
+                 c_a: int = 768, c_s: int = 384, c_z: int = 128, biasinit: float = -2.0,
+                 cross_attention_mode: bool = False) -> None:
+        super().__init__()
+        if has_s or cross_attention_mode:
+            raise NotImplementedError(
+                "protenix_amd.AttentionPairBias covers the Pairformer-block flavour "
+                "(has_s=False, cross_attention_mode=False); the diffusion-module flavours "
+                "are outside this package")
+        assert c_a % n_heads == 0
+        self.n_heads = n_heads
+        self.has_s = has_s
+        self.create_offset_ln_z = create_offset_ln_z
+        self.cross_attention_mode = cross_attention_mode
+        self.layernorm_a = LayerNorm(c_a)
+        self.local_attention_method = "local_cross_attention"
+        self.attention = Attention(c_q=c_a, c_k=c_a, c_v=c_a, c_hidden=c_a // n_heads,
+                                   num_heads=n_heads, gating=True, q_linear_bias=True,
+                                   local_attention_method=self.local_attention_method,
+                                   zero_init=not has_s)
+        self.layernorm_z = LayerNorm(c_z, create_offset=create_offset_ln_z)
+        self.linear_nobias_z = LinearNoBias(in_features=c_z, out_features=n_heads)
+        self._cache = _WeightCache()
+
+    def pair_bias(self, z: torch.Tensor) -> torch.Tensor:
+        """[*, N, N, c_z] -> fp32 [*, heads, N, N] = permute(linear(LN(z)))
+        (transformer.py:191-194)."""
+        ps = (self.layernorm_z.weight, self.layernorm_z.bias, self.linear_nobias_z.weight)
+        ln_w, ln_b, w = self._cache.get(ps, z.dtype, z.device,
+                                        lambda: tuple(_cv(p, z.dtype, z.device) for p in ps))
+        n, c = z.shape[-2], z.shape[-1]
+        zb = z.contiguous().reshape(-1, n, n, c)
+        out = torch.stack([ops.pair_bias(zb[i], ln_w, ln_b, w, out_f32=True)
+                           for i in range(zb.shape[0])])
+        return out.reshape(*z.shape[:-3], self.n_heads, n, n)
+
+    def forward(self, a: torch.Tensor, s: Optional[torch.Tensor], z: torch.Tensor,
+                n_queries: Optional[int] = None, n_keys: Optional[int] = None,
+                inplace_safe: bool = False, chunk_size: Optional[int] = None,
+                enable_efficient_fusion: bool = False) -> torch.Tensor:
+        if n_queries or n_keys:
+            raise NotImplementedError("local attention belongs to the diffusion module")
+        _forward_only(a, z, *self.parameters())
+        a = self.layernorm_a(a)
+        return self.attention(q_x=a, kv_x=a, attn_bias=self.pair_bias(z))

@@ -1,0 +1,203 @@
+"""Triangle multiplication and triangle attention on the gfx950 kernels.
+
+Same classes, constructor arguments, parameter names and forward signatures as
+protenix/model/triangular/triangular.py:93-197, 470-586 (TriangleMultiplicative
+Update and its Outgoing/Incoming flavours) and :589-727 (TriangleAttention),
+with the attention sub-module of protenix/model/triangular/layers.py:299-473
+kept as the parameter container `mha`.  The kernel-selection strings of the
+reference are accepted and validated; every valid value runs the HIP kernels.
+Forward only, c_z = c_hidden = 128 and 4 heads x 32 (anything else is refused by
+the library with an "unsupported shape" error).
+"""
+from __future__ import annotations
+
+from typing import List, Optional
+
+import torch
+import torch.nn as nn
+
+from . import ops
+from .layer_norm import LayerNorm, _forward_only
+from .primitives import Linear, _cv, _WeightCache
+
+
+def OpenfoldLinear(in_dim: int, out_dim: int, bias: bool = True, init: str = "default") -> Linear:
+    """layers.py:104-197 by its `init` names."""
+    if init not in ("default", "relu", "gating", "final"):
+        raise ValueError("Invalid init string.")
+    return Linear(in_dim, out_dim, bias=bias, initializer=init)
+
+
+def _per_batch(z: torch.Tensor, mask: Optional[torch.Tensor]):
+    """[*, N, N, C] -> list of ([N, N, C], [N, N] or None) sharing storage with z."""
+    if z.dim() < 3:
+        raise RuntimeError(f"expected [*, N, N, C], got {tuple(z.shape)}")
+    n, c = z.shape[-2], z.shape[-1]
+    if z.shape[-3] != n:
+        raise RuntimeError(f"pair tensor must be square, got {tuple(z.shape)}")
+    zb = z.reshape(-1, n, n, c)
+    mb = None
+    if mask is not None:
+        if mask.shape != z.shape[:-1]:
+            mask = mask.expand(z.shape[:-1])
+        mb = mask.reshape(-1, n, n)
+    return zb, mb
+
+
+class TriangleMultiplicativeUpdate(nn.Module):
+    """Algorithms 11 and 12 of AF3 (triangular.py:172-570)."""
+
+    def __init__(self, c_z: int, c_hidden: int, _outgoing: bool = True) -> None:
+        super().__init__()
+        self.c_z = c_z
+        self.c_hidden = c_hidden
+        self._outgoing = _outgoing
+        self.linear_g = OpenfoldLinear(c_z, c_z, bias=False, init="gating")
+        self.linear_z = OpenfoldLinear(c_hidden, c_z, bias=False, init="final")
+        self.layer_norm_in = LayerNorm(c_z)
+        self.layer_norm_out = LayerNorm(c_hidden)
+        self.sigmoid = nn.Sigmoid()
+        self.linear_a_p = OpenfoldLinear(c_z, c_hidden, bias=False)
+        self.linear_a_g = OpenfoldLinear(c_z, c_hidden, bias=False, init="gating")
+        self.linear_b_p = OpenfoldLinear(c_z, c_hidden, bias=False)
+        self.linear_b_g = OpenfoldLinear(c_z, c_hidden, bias=False, init="gating")
+        self._cache = _WeightCache()
+
+    def _weights(self, dtype, device) -> dict:
+        ps = (self.layer_norm_in.weight, self.layer_norm_in.bias, self.layer_norm_out.weight,
+              self.layer_norm_out.bias, self.linear_a_p.weight, self.linear_a_g.weight,
+              self.linear_b_p.weight, self.linear_b_g.weight, self.linear_z.weight,
+              self.linear_g.weight)
+        names = ("ln_in_w", "ln_in_b", "ln_out_w", "ln_out_b", "w_ap", "w_ag", "w_bp", "w_bg",
+                 "w_z", "w_g")
+        return self._cache.get(ps, dtype, device,
+                               lambda: dict(zip(names, (_cv(p, dtype, device) for p in ps))))
+
+    def forward(self, z: torch.Tensor, mask: Optional[torch.Tensor] = None,
+                inplace_safe: bool = False, _add_with_inplace: bool = False,
+                _inplace_chunk_size: Optional[int] = 256,
+                triangle_multiplicative: str = "torch") -> torch.Tensor:
+        """z [*, N, N, c_z], mask [*, N, N] -> update [*, N, N, c_z]; with
+        `inplace_safe and _add_with_inplace` z is overwritten with z + update and
+        returned (triangular.py:470-566)."""
+        if triangle_multiplicative not in ("torch", "cuequivariance"):
+            raise ValueError(
+                "triangle_multiplicative must be 'cuequivariance' or 'torch', but got "
+                f"{triangle_multiplicative}")
+        _forward_only(z, *self.parameters())
+        add_inplace = bool(inplace_safe and _add_with_inplace)
+        w = self._weights(z.dtype, z.device)
+        src = z if z.is_contiguous() else z.contiguous()
+        zb, mb = _per_batch(src, mask)
+        out = src if add_inplace else torch.empty_like(src)
+        ob = out.view(zb.shape)
+        for bi in range(zb.shape[0]):
+            ops.triangle_multiplication(zb[bi], None if mb is None else mb[bi], w,
+                                        incoming=not self._outgoing, add_residual=add_inplace,
+                                        out=ob[bi])
+        if add_inplace and out is not z:
+            z.copy_(out)
+            return z
+        return out
+
+
+class TriangleMultiplicationOutgoing(TriangleMultiplicativeUpdate):
+    """Algorithm 11."""
+
+    def __init__(self, c_z: int, c_hidden: int) -> None:
+        super().__init__(c_z=c_z, c_hidden=c_hidden, _outgoing=True)
+
+
+class TriangleMultiplicationIncoming(TriangleMultiplicativeUpdate):
+    """Algorithm 12."""
+
+    def __init__(self, c_z: int, c_hidden: int) -> None:
+        super().__init__(c_z=c_z, c_hidden=c_hidden, _outgoing=False)
+
+
+class Attention(nn.Module):
+    """Parameter container with the names of layers.py:299-359; the arithmetic
+    lives in TriangleAttention.forward (fused kernels)."""
+
+    def __init__(self, c_q: int, c_k: int, c_v: int, c_hidden: int, no_heads: int,
+                 gating: bool = True) -> None:
+        super().__init__()
+        self.c_q, self.c_k, self.c_v = c_q, c_k, c_v
+        self.c_hidden = c_hidden
+        self.no_heads = no_heads
+        self.gating = gating
+        self.linear_q = OpenfoldLinear(c_q, c_hidden * no_heads, bias=False)
+        self.linear_k = OpenfoldLinear(c_k, c_hidden * no_heads, bias=False)
+        self.linear_v = OpenfoldLinear(c_v, c_hidden * no_heads, bias=False)
+        self.linear_o = OpenfoldLinear(c_hidden * no_heads, c_q, bias=False, init="final")
+        self.linear_g = None
+        if gating:
+            self.linear_g = OpenfoldLinear(c_q, c_hidden * no_heads, bias=False, init="gating")
+        self.sigmoid = nn.Sigmoid()
+
+    def forward(self, *args, **kwargs):
+        raise RuntimeError(
+            "protenix_amd: the triangle-attention sub-module is fused into "
+            "TriangleAttention.forward and cannot be called on its own")
+
+
+class TriangleAttention(nn.Module):
+    """Algorithms 13 / 14 of AF3 (triangular.py:589-715)."""
+
+    def __init__(self, c_in: int, c_hidden: int, no_heads: int, starting: bool = True,
+                 inf: float = 1e9) -> None:
+        super().__init__()
+        self.c_in = c_in
+        self.c_hidden = c_hidden
+        self.no_heads = no_heads
+        self.starting = starting
+        self.inf = inf
+        self.layer_norm = LayerNorm(c_in)
+        self.linear = OpenfoldLinear(c_in, no_heads, bias=False)
+        self.mha = Attention(c_in, c_in, c_in, c_hidden, no_heads)
+        self._cache = _WeightCache()
+
+    def _weights(self, dtype, device) -> dict:
+        m = self.mha
+        ps = (self.layer_norm.weight, self.layer_norm.bias, m.linear_q.weight, m.linear_k.weight,
+              m.linear_v.weight, m.linear_g.weight, self.linear.weight, m.linear_o.weight)
+        names = ("ln_w", "ln_b", "w_q", "w_k", "w_v", "w_g", "w_b", "w_o")
+        return self._cache.get(ps, dtype, device,
+                               lambda: dict(zip(names, (_cv(p, dtype, device) for p in ps))))
+
+    def _run(self, x: torch.Tensor, mask: Optional[torch.Tensor], transposed: bool,
+             residual_inplace: bool) -> torch.Tensor:
+        _forward_only(x, *self.parameters())
+        w = self._weights(x.dtype, x.device)
+        src = x if x.is_contiguous() else x.contiguous()
+        xb, mb = _per_batch(src, mask)
+        out = src if residual_inplace else torch.empty_like(src)
+        ob = out.view(xb.shape)
+        for bi in range(xb.shape[0]):
+            ops.triangle_attention(xb[bi], None if mb is None else mb[bi], w, self.no_heads,
+                                   self.c_hidden, self.inf, transposed=transposed,
+                                   add_residual=residual_inplace, out=ob[bi])
+        if residual_inplace and out is not x:
+            x.copy_(out)
+            return x
+        return out
+
+    def forward(self, x: torch.Tensor, mask: Optional[torch.Tensor] = None,
+                chunk_size: Optional[int] = None, triangle_attention: str = "torch",
+                inplace_safe: bool = False) -> torch.Tensor:
+        """x [*, I, J, c_in], mask [*, I, J] -> update [*, I, J, c_in].  Keys are
+        masked per row with inf*(mask-1); `chunk_size` only bounds memory in the
+        reference (rows are independent) and is not needed here, since the logits
+        are never materialised."""
+        assert triangle_attention in ("torch", "deepspeed", "triattention", "cuequivariance")
+        return self._run(x, mask, transposed=not self.starting, residual_inplace=False)
+
+
+TriangleAttentionStartingNode = TriangleAttention
+
+
+class TriangleAttentionEndingNode(TriangleAttention):
+    """Algorithm 14."""
+
+    def __init__(self, c_in: int, c_hidden: int, no_heads: int, inf: float = 1e9) -> None:
+        super().__init__(c_in, c_hidden, no_heads, starting=False, inf=inf)

@@ -1,0 +1,197 @@
+"""Parity of the HIP path (through the C ABI) against the CPU oracle on the same
+seeded inputs.  Reference for every comparison: the fp32 oracle evaluated on the
+dtype-rounded inputs and parameters.  Tolerances (BASELINE): fp32 1e-4, bf16 2e-2,
+both max-abs error relative to max |reference|."""
+import pytest
+import torch
+
+import protenix_amd as P
+from oracle import pairformer_oracle as O
+from tests.util import oracle_and_product, pad_mask, rel_err, tol
+
+pytestmark = pytest.mark.gpu
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+def _z(n, dtype, seed=1234, c=128):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randn(1, n, n, c, generator=g).to(dtype)
+
+
+# ------------------------------------------------------------------ LayerNorm
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("rows,cols", [(1000, 128), (4099, 128), (77, 384), (33, 64), (19, 100),
+                                       (5, 7), (3, 4096), (2, 5000), (0, 128)])
+@pytest.mark.parametrize("affine", ["both", "none", "scale", "offset"])
+def test_layernorm(dtype, rows, cols, affine):
+    g = torch.Generator().manual_seed(rows * 131 + cols)
+    x = (torch.randn(rows, cols, generator=g) * 3 + 1.5).to(dtype)
+    ln = P.LayerNorm(cols, create_scale=affine in ("both", "scale"),
+                     create_offset=affine in ("both", "offset"))
+    with torch.no_grad():
+        if ln.weight is not None:
+            ln.weight.copy_(1 + 0.1 * torch.randn(cols, generator=g))
+        if ln.bias is not None:
+            ln.bias.copy_(0.1 * torch.randn(cols, generator=g))
+    ln = ln.to("cuda", dtype)
+    with torch.no_grad():
+        y = ln(x.cuda())
+    assert y.dtype == dtype and y.shape == x.shape
+    if rows == 0:
+        return
+    w = ln.weight.float().cpu() if ln.weight is not None else None
+    b = ln.bias.float().cpu() if ln.bias is not None else None
+    ref = O.layer_norm(x.float(), w, b)
+    assert rel_err(y, ref) <= (1e-5 if dtype == torch.float32 else 2 ** -7)
+
+
+def test_layernorm_stats_and_closed_forms():
+    from protenix_amd import ops
+    x = torch.randn(513, 128, device="cuda") * 2 + 3
+    y, mean, rstd = ops.layer_norm(x, None, None, 1e-5, return_stats=True)
+    assert torch.allclose(mean, x.mean(-1), atol=1e-5)
+    assert torch.allclose(rstd, torch.rsqrt(x.var(-1, unbiased=False) + 1e-5), rtol=1e-4)
+    beta = torch.randn(128, device="cuda")
+    const = torch.full((9, 128), 4.25, device="cuda")
+    assert torch.allclose(ops.layer_norm(const, torch.randn(128, device="cuda"), beta), beta.expand(9, 128), atol=1e-6)
+
+
+# ------------------------------------------------------------------ TriMul
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("cls", ["TriangleMultiplicationOutgoing", "TriangleMultiplicationIncoming"])
+@pytest.mark.parametrize("n,n_pad", [(64, 0), (100, 7), (37, 0), (200, 16)])
+def test_trimul(dtype, cls, n, n_pad):
+    ref, prod = oracle_and_product(getattr(O, cls), getattr(P, cls), 128, 128, dtype=dtype)
+    z = _z(n, dtype)
+    mask = pad_mask(n, n_pad, dtype) if n_pad else None
+    with torch.no_grad():
+        want = ref(z.float(), None if mask is None else mask.float())
+        got = prod(z.cuda(), None if mask is None else mask.cuda())
+        assert rel_err(got, want) <= tol(dtype)
+        # z + update, in place
+        zc = z.cuda().clone()
+        got2 = prod(zc, None if mask is None else mask.cuda(), inplace_safe=True, _add_with_inplace=True)
+        assert got2.data_ptr() == zc.data_ptr()
+        assert rel_err(got2, z.float() + want) <= tol(dtype)
+
+
+def test_trimul_random_mask_and_errors():
+    ref, prod = oracle_and_product(O.TriangleMultiplicationOutgoing, P.TriangleMultiplicationOutgoing, 128, 128)
+    n = 48
+    z = _z(n, torch.float32)
+    mask = (torch.rand(1, n, n, generator=torch.Generator().manual_seed(3)) > 0.3).float()
+    with torch.no_grad():
+        assert rel_err(prod(z.cuda(), mask.cuda()), ref(z, mask)) <= 1e-4
+        with pytest.raises(ValueError):
+            prod(z.cuda(), triangle_multiplicative="bogus")
+        with pytest.raises(RuntimeError):
+            prod(z)                      # CPU tensor: no silent fallback
+    bad = P.TriangleMultiplicationOutgoing(64, 64).cuda()
+    with torch.no_grad(), pytest.raises(RuntimeError, match="unsupported"):
+        bad(torch.randn(1, 8, 8, 64, device="cuda"))
+
+
+# ------------------------------------------------------------------ TriAttn
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("starting", [True, False])
+@pytest.mark.parametrize("n,n_pad", [(64, 0), (100, 7), (37, 5), (256, 32), (320, 0)])
+def test_triattn(dtype, starting, n, n_pad):
+    ref, prod = oracle_and_product(O.TriangleAttention, P.TriangleAttention, 128, 32, 4,
+                                   starting=starting, dtype=dtype)
+    z = _z(n, dtype)
+    mask = pad_mask(n, n_pad, dtype) if n_pad else None
+    with torch.no_grad():
+        want = ref(z.float(), None if mask is None else mask.float(), chunk_size=64)
+        got = prod(z.cuda(), None if mask is None else mask.cuda())
+    # padded query rows (fully masked keys) are included: they must equal the
+    # reference's mean-of-v behaviour too
+    assert rel_err(got, want) <= tol(dtype)
+
+
+def test_triattn_random_mask_large_logits():
+    """Random key masks, rows with every key masked, and logits big enough that
+    the -1e9 absorption and the order of the two bias adds matter."""
+    ref, prod = oracle_and_product(O.TriangleAttention, P.TriangleAttention, 128, 32, 4)
+    n = 72
+    z = _z(n, torch.float32) * 4
+    g = torch.Generator().manual_seed(5)
+    mask = (torch.rand(1, n, n, generator=g) > 0.4).float()
+    mask[0, 3] = 0
+    mask[0, 70] = 0
+    with torch.no_grad():
+        for p_ref, p_prod in ((ref.linear, prod.linear), (ref.mha.linear_q, prod.mha.linear_q)):
+            p_ref.weight.mul_(3)
+            p_prod.weight.mul_(3)
+        want = ref(z, mask)
+        got = prod(z.cuda(), mask.cuda())
+    assert rel_err(got, want) <= 1e-4
+
+
+# ------------------------------------------------------------------ Transition / pair bias
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shape", [(1, 50, 50, 128), (3001, 128), (1, 64, 384)])
+def test_transition(dtype, shape):
+    ref, prod = oracle_and_product(O.Transition, P.Transition, shape[-1], 4, dtype=dtype)
+    x = torch.randn(*shape, generator=torch.Generator().manual_seed(11)).to(dtype)
+    with torch.no_grad():
+        assert rel_err(prod(x.cuda()), ref(x.float())) <= tol(dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_attention_pair_bias(dtype):
+    kw = dict(has_s=False, create_offset_ln_z=True, n_heads=16, c_a=384, c_z=128)
+    ref, prod = oracle_and_product(O.AttentionPairBias, P.AttentionPairBias, dtype=dtype, **kw)
+    n = 70
+    z = _z(n, dtype)
+    s = torch.randn(1, n, 384, generator=torch.Generator().manual_seed(2)).to(dtype)
+    with torch.no_grad():
+        bias = prod.pair_bias(z.cuda())
+        want_bias = ref.linear_nobias_z(ref.layernorm_z(z.float())).permute(0, 3, 1, 2)
+        assert bias.dtype == torch.float32
+        assert rel_err(bias, want_bias) <= tol(dtype)
+        assert rel_err(prod(a=s.cuda(), s=None, z=z.cuda()), ref(a=s.float(), s=None, z=z.float())) <= tol(dtype)
+
+
+# ------------------------------------------------------------------ block / stack
+def test_block_c1_fp32_n64():
+    """BASELINE config 1: one PairformerBlock, fp32, N=64, mask of ones."""
+    ref, prod = oracle_and_product(O.PairformerBlock, P.PairformerBlock)
+    s, z, pm = O.make_inputs(64)
+    with torch.no_grad():
+        s_ref, z_ref = ref(s, z, pm)
+        zc = z.cuda()
+        s_got, z_got = prod(s.cuda(), zc, pm.cuda())
+        assert torch.equal(zc.cpu(), z), "inputs must stay untouched without inplace_safe"
+        assert rel_err(z_got, z_ref) <= 1e-4 and rel_err(s_got, s_ref) <= 1e-4
+        s2, z2 = prod(s.cuda(), zc, None, inplace_safe=True)
+        assert z2.data_ptr() == zc.data_ptr()
+        assert rel_err(z2, z_ref) <= 1e-4 and rel_err(s2, s_ref) <= 1e-4
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("n,n_pad", [(96, 9), (130, 0)])
+def test_block_masked(dtype, n, n_pad):
+    ref, prod = oracle_and_product(O.PairformerBlock, P.PairformerBlock, dtype=dtype)
+    s, z, pm = O.make_inputs(n, n_pad=n_pad, dtype=dtype)
+    with torch.no_grad():
+        s_ref, z_ref = ref(s.float(), z.float(), pm.float())
+        s_got, z_got = prod(s.cuda(), z.cuda(), pm.cuda())
+    assert rel_err(z_got, z_ref) <= tol(dtype) and rel_err(s_got, s_ref) <= tol(dtype)
+
+
+def test_block_without_single_track():
+    ref, prod = oracle_and_product(O.PairformerBlock, P.PairformerBlock, c_s=0)
+    _, z, pm = O.make_inputs(40, n_pad=3)
+    with torch.no_grad():
+        s_got, z_got = prod(None, z.cuda(), pm.cuda())
+        assert s_got is None and rel_err(z_got, ref(None, z, pm)[1]) <= 1e-4
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_stack_4_blocks(dtype):
+    ref, prod = oracle_and_product(O.PairformerStack, P.PairformerStack, n_blocks=4, dtype=dtype)
+    s, z, pm = O.make_inputs(80, n_pad=6, dtype=dtype)
+    with torch.no_grad():
+        s_ref, z_ref = ref(s.float(), z.float(), pm.float())
+        s_got, z_got = prod(s.cuda(), z.cuda(), pm.cuda())
+    assert rel_err(z_got, z_ref) <= tol(dtype) and rel_err(s_got, s_ref) <= tol(dtype)

@@ -1,0 +1,89 @@
+"""CPU-side checks: the C-ABI library builds/loads and exports every symbol the
+header declares, argument validation answers without touching a GPU, and the
+drop-in modules keep the reference's state-dict layout."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+import protenix_amd as P
+from oracle import pairformer_oracle as O
+from protenix_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared():
+    text = open(os.path.join(ROOT, "include", "protenix_amd.h")).read()
+    return re.findall(r"PTX_API\s+[\w\s\*]+?\b(ptx_\w+)\s*\(", text)
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _lib.load()
+    names = _declared()
+    assert len(names) >= 12
+    for n in names:
+        assert hasattr(lib, n), n
+        assert n in _lib.SIGNATURES, f"{n} has no ctypes signature"
+    assert set(_lib.SIGNATURES) == set(names)
+    assert lib.ptx_version() == _lib.ABI_VERSION
+    assert lib.ptx_last_error_string() is not None
+
+
+def test_key_pitch():
+    lib = _lib.load()
+    assert [lib.ptx_key_pitch(n) for n in (0, 1, 64, 65, 768, 2048)] == [0, 64, 64, 128, 768, 2048]
+
+
+def test_argument_validation_without_gpu():
+    lib = _lib.load()
+    # unknown dtype, bad sizes, unsupported widths: rejected before any launch
+    assert lib.ptx_layernorm_fwd(None, None, None, None, None, None, 4, 128, 1e-5, 7, None) == 1
+    assert b"dtype" in lib.ptx_last_error_string()
+    assert lib.ptx_layernorm_fwd(None, None, None, None, None, None, 4, 128, 1e-5, 0, None) == 1
+    assert lib.ptx_layernorm_fwd(None, None, None, None, None, None, 0, 128, 1e-5, 0, None) == 0
+    assert lib.ptx_trimul_contract(None, None, None, 8, 128, 63, 1, None) == 1
+    assert b"k_pitch" in lib.ptx_last_error_string()
+    assert lib.ptx_trimul_project(*([None] * 10), 8, 64, 64, 64, 0, 1e-5, 1, None) == 2
+    assert b"128" in lib.ptx_last_error_string()
+    assert lib.ptx_triattn_fwd(*([None] * 7), 8, 4, 16, 64, 0, 1e9, 1, None) == 2
+    assert lib.ptx_triattn_project(*([None] * 13), 8, 128, 8, 16, 64, 0, 1e-5, 1, None) == 2
+    assert lib.ptx_transition_fwd(*([None] * 8), 10, 384, 4, 0, 1e-5, 0, None) == 2
+    assert lib.ptx_pair_bias_fwd(*([None] * 5), 8, 128, 33, 1, 1e-5, 0, None) == 2
+    assert lib.ptx_triattn_output(None, None, None, None, 8, 128, 0, 1, 0, None) == 1
+    with pytest.raises(RuntimeError, match="unsupported shape"):
+        _lib.check(2, "x")
+
+
+def test_modules_refuse_cpu_tensors_and_grad():
+    ln = P.LayerNorm(128)
+    with torch.no_grad(), pytest.raises(RuntimeError, match="GPU tensor"):
+        ln(torch.randn(4, 128))
+    with pytest.raises(RuntimeError, match="forward-only"):
+        ln(torch.randn(4, 128))
+    blk = P.PairformerBlock()
+    with pytest.raises(RuntimeError, match="inference-only"):
+        blk(torch.randn(1, 8, 384), torch.randn(1, 8, 8, 128), None)
+    with torch.no_grad(), pytest.raises(ValueError):
+        blk.eval()(torch.randn(1, 8, 384), torch.randn(1, 8, 8, 128), None, triangle_multiplicative="x")
+
+
+def test_state_dict_layout_matches_oracle_and_default_init_is_identity_shaped():
+    a, b = P.PairformerStack(n_blocks=2), O.PairformerStack(n_blocks=2)
+    sa, sb = a.state_dict(), b.state_dict()
+    assert list(sa.keys()) == list(sb.keys())
+    for k in sa:
+        assert sa[k].shape == sb[k].shape, k
+    a.load_state_dict(sb)
+    blk = P.PairformerBlock()
+    # the reference zero-initialises gates and output projections
+    for name in ("tri_mul_out.linear_z", "tri_mul_in.linear_g", "tri_att_start.mha.linear_o",
+                 "tri_att_end.mha.linear_g", "pair_transition.linear_no_bias",
+                 "attention_pair_bias.attention.linear_o", "attention_pair_bias.attention.linear_g"):
+        assert blk.get_submodule(name).weight.abs().sum() == 0, name
+    assert blk.tri_mul_out.linear_a_p.weight.std() > 0
+    assert P.TriangleAttentionEndingNode(128, 32, 4).starting is False
+    with pytest.raises(NotImplementedError):
+        P.AttentionPairBias(has_s=True)
