@@ -33,6 +33,30 @@ def _stream() -> int:
     return torch.cuda.current_stream().cuda_stream
 
 
+# Optional per-kernel timing: while `kernel_timer` is a dict, every C-ABI call
+# is bracketed by HIP events on the stream it is launched on and the pairs are
+# appended under the entry point's name; read them with kernel_times().
+kernel_timer: Optional[dict] = None
+
+
+def _call(name: str, fn, *args) -> None:
+    if kernel_timer is None:
+        _lib.check(fn(*args), name)
+        return
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    e0.record()
+    _lib.check(fn(*args), name)
+    e1.record()
+    kernel_timer.setdefault(name, []).append((e0, e1))
+
+
+def kernel_times(timer: dict) -> dict:
+    """name -> list of launch-to-completion durations in ms (synchronises)."""
+    torch.cuda.synchronize()
+    return {k: [a.elapsed_time(b) for a, b in v] for k, v in timer.items()}
+
+
 def _same(t: Optional[torch.Tensor], like: torch.Tensor, name: str) -> Optional[torch.Tensor]:
     """Parameter tensor in the activation dtype/device, contiguous."""
     if t is None:
@@ -62,8 +86,8 @@ def layer_norm(x: torch.Tensor, weight: Optional[torch.Tensor], bias: Optional[t
         mean = torch.empty(rows, dtype=torch.float32, device=x.device)
         rstd = torch.empty(rows, dtype=torch.float32, device=x.device)
     with torch.cuda.device(x.device):
-        _lib.check(lib.ptx_layernorm_fwd(_ptr(x), _ptr(w), _ptr(b), _ptr(y), _ptr(mean), _ptr(rstd),
-                                         rows, cols, eps, _dt(x), _stream()), "layernorm")
+        _call("layernorm", lib.ptx_layernorm_fwd, _ptr(x), _ptr(w), _ptr(b), _ptr(y), _ptr(mean), _ptr(rstd),
+                                         rows, cols, eps, _dt(x), _stream())
     return (y, mean, rstd) if return_stats else y
 
 
@@ -88,20 +112,17 @@ def triangle_multiplication(z: torch.Tensor, mask: Optional[torch.Tensor], w: di
     a = torch.empty((c_h, n, pitch), dtype=z.dtype, device=z.device)
     b = torch.empty((c_h, n, pitch), dtype=z.dtype, device=z.device)
     with torch.cuda.device(z.device):
-        _lib.check(lib.ptx_trimul_project(
-            _ptr(z), _ptr(mask), _ptr(w["ln_in_w"]), _ptr(w["ln_in_b"]), _ptr(w["w_ap"]),
+        _call("trimul_project", lib.ptx_trimul_project, _ptr(z), _ptr(mask), _ptr(w["ln_in_w"]), _ptr(w["ln_in_b"]), _ptr(w["w_ap"]),
             _ptr(w["w_ag"]), _ptr(w["w_bp"]), _ptr(w["w_bg"]), _ptr(a), _ptr(b), n, c_z, c_h, pitch,
-            int(incoming), eps, dt, st), "trimul_project")
+            int(incoming), eps, dt, st)
         x = torch.empty((c_h, n, n), dtype=z.dtype, device=z.device)
-        _lib.check(lib.ptx_trimul_contract(_ptr(a), _ptr(b), _ptr(x), n, c_h, pitch, dt, st),
-                   "trimul_contract")
+        _call("trimul_contract", lib.ptx_trimul_contract, _ptr(a), _ptr(b), _ptr(x), n, c_h, pitch, dt, st)
         del a, b
         if out is None:
             out = torch.empty_like(z)
-        _lib.check(lib.ptx_trimul_output(
-            _ptr(x), _ptr(z), _ptr(w["ln_in_w"]), _ptr(w["ln_in_b"]), _ptr(w["ln_out_w"]),
+        _call("trimul_output", lib.ptx_trimul_output, _ptr(x), _ptr(z), _ptr(w["ln_in_w"]), _ptr(w["ln_in_b"]), _ptr(w["ln_out_w"]),
             _ptr(w["ln_out_b"]), _ptr(w["w_z"]), _ptr(w["w_g"]), _ptr(out), n, c_z, c_h,
-            int(add_residual), eps, dt, st), "trimul_output")
+            int(add_residual), eps, dt, st)
     return out
 
 
@@ -126,20 +147,18 @@ def triangle_attention(z: torch.Tensor, mask: Optional[torch.Tensor], w: dict, h
     vt = torch.empty((n, hd, pitch), dtype=z.dtype, device=dev)
     tb = torch.empty((heads, n, pitch), dtype=z.dtype, device=dev)
     with torch.cuda.device(dev):
-        _lib.check(lib.ptx_triattn_project(
-            _ptr(z), _ptr(w["ln_w"]), _ptr(w["ln_b"]), _ptr(w["w_q"]), _ptr(w["w_k"]), _ptr(w["w_v"]),
+        _call("triattn_project", lib.ptx_triattn_project, _ptr(z), _ptr(w["ln_w"]), _ptr(w["ln_b"]), _ptr(w["w_q"]), _ptr(w["w_k"]), _ptr(w["w_v"]),
             _ptr(w["w_g"]), _ptr(w["w_b"]), _ptr(q), _ptr(k), _ptr(vt), _ptr(g), _ptr(tb), n, c,
-            heads, d, pitch, int(transposed), eps, dt, st), "triattn_project")
+            heads, d, pitch, int(transposed), eps, dt, st)
         # o overwrites g: each element of g is read once, by the thread that then writes o there
-        _lib.check(lib.ptx_triattn_fwd(_ptr(q), _ptr(k), _ptr(vt), _ptr(g), _ptr(tb), _ptr(mask),
+        _call("triattn_fwd", lib.ptx_triattn_fwd, _ptr(q), _ptr(k), _ptr(vt), _ptr(g), _ptr(tb), _ptr(mask),
                                        _ptr(g), n, heads, d, pitch, int(transposed), float(inf), dt,
-                                       st), "triattn_fwd")
+                                       st)
         del q, k, vt, tb
         if out is None:
             out = torch.empty_like(z)
-        _lib.check(lib.ptx_triattn_output(_ptr(g), _ptr(w["w_o"]), _ptr(z), _ptr(out), n, c,
-                                          int(transposed), int(add_residual), dt, st),
-                   "triattn_output")
+        _call("triattn_output", lib.ptx_triattn_output, _ptr(g), _ptr(w["w_o"]), _ptr(z), _ptr(out), n, c,
+                                          int(transposed), int(add_residual), dt, st)
     return out
 
 
@@ -164,10 +183,9 @@ def transition(x: torch.Tensor, w: dict, n_factor: int, add_residual: bool,
     with torch.cuda.device(x.device):
         for r0 in range(0, rows, slab):
             r1 = min(rows, r0 + slab)
-            _lib.check(lib.ptx_transition_fwd(
-                _ptr(x2[r0:r1]), _ptr(w["ln_w"]), _ptr(w["ln_b"]), _ptr(w["w_a"]), _ptr(w["w_b"]),
+            _call("transition", lib.ptx_transition_fwd, _ptr(x2[r0:r1]), _ptr(w["ln_w"]), _ptr(w["ln_b"]), _ptr(w["w_a"]), _ptr(w["w_b"]),
                 _ptr(w["w_o"]), _ptr(hidden), _ptr(o2[r0:r1]), r1 - r0, c, n_factor,
-                int(add_residual), eps, dt, st), "transition")
+                int(add_residual), eps, dt, st)
     return out.view(x.shape)
 
 
@@ -180,6 +198,6 @@ def pair_bias(z: torch.Tensor, ln_w: Optional[torch.Tensor], ln_b: Optional[torc
     heads = w.shape[0]
     out = torch.empty((heads, n, n), dtype=torch.float32 if out_f32 else z.dtype, device=z.device)
     with torch.cuda.device(z.device):
-        _lib.check(lib.ptx_pair_bias_fwd(_ptr(z), _ptr(ln_w), _ptr(ln_b), _ptr(w), _ptr(out), n, c,
-                                         heads, int(out_f32), eps, _dt(z), _stream()), "pair_bias")
+        _call("pair_bias", lib.ptx_pair_bias_fwd, _ptr(z), _ptr(ln_w), _ptr(ln_b), _ptr(w), _ptr(out), n, c,
+                                         heads, int(out_f32), eps, _dt(z), _stream())
     return out
