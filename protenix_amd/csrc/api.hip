@@ -88,7 +88,8 @@ PTX_API int ptx_trimul_project(const void* z, const void* mask, const void* ln_w
   PTX_REQUIRE(z && w_ap && w_ag && w_bp && w_bg && a && b, PTX_ERR_BAD_ARG,
               "trimul_project: null pointer");
   PTX_REQUIRE(aligned16(z) && aligned16(w_ap) && aligned16(w_ag) && aligned16(w_bp) &&
-                  aligned16(w_bg) && (!ln_w || aligned16(ln_w)) && (!ln_b || aligned16(ln_b)),
+                  aligned16(w_bg) && aligned16(a) && aligned16(b) && (!ln_w || aligned16(ln_w)) &&
+                  (!ln_b || aligned16(ln_b)),
               PTX_ERR_BAD_ARG, "trimul_project: pointers must be 16-byte aligned");
   PTX_DISPATCH(dtype, ptx::trimul_project<T>(z, mask, ln_w, ln_b, w_ap, w_ag, w_bp, w_bg, a, b, n,
                                              k_pitch, incoming, eps, (hipStream_t)stream));
@@ -123,8 +124,9 @@ PTX_API int ptx_trimul_output(const void* x, const void* z, const void* ln_in_w,
   if (n == 0) return PTX_OK;
   PTX_REQUIRE(x && z && ln_out_w && ln_out_b && w_z && w_g && out, PTX_ERR_BAD_ARG,
               "trimul_output: null pointer");
-  PTX_REQUIRE(aligned16(z) && aligned16(w_z) && aligned16(w_g) && aligned16(ln_out_w) &&
-                  aligned16(ln_out_b) && (!ln_in_w || aligned16(ln_in_w)) &&
+  PTX_REQUIRE(aligned16(x) && aligned16(out) && aligned16(z) && aligned16(w_z) &&
+                  aligned16(w_g) && aligned16(ln_out_w) && aligned16(ln_out_b) &&
+                  (!ln_in_w || aligned16(ln_in_w)) &&
                   (!ln_in_b || aligned16(ln_in_b)),
               PTX_ERR_BAD_ARG, "trimul_output: pointers must be 16-byte aligned");
   PTX_DISPATCH(dtype, ptx::trimul_output<T>(x, z, ln_in_w, ln_in_b, ln_out_w, ln_out_b, w_z, w_g,
@@ -149,7 +151,9 @@ PTX_API int ptx_triattn_project(const void* z, const void* ln_w, const void* ln_
   PTX_REQUIRE(z && w_q && w_k && w_v && w_g && w_b && q && k && vt && g && tri_bias,
               PTX_ERR_BAD_ARG, "triattn_project: null pointer");
   PTX_REQUIRE(aligned16(z) && aligned16(w_q) && aligned16(w_k) && aligned16(w_v) &&
-                  aligned16(w_g) && aligned16(w_b) && (!ln_w || aligned16(ln_w)) &&
+                  aligned16(w_g) && aligned16(w_b) && aligned16(q) && aligned16(k) &&
+                  aligned16(vt) && aligned16(g) && aligned16(tri_bias) &&
+                  (!ln_w || aligned16(ln_w)) &&
                   (!ln_b || aligned16(ln_b)),
               PTX_ERR_BAD_ARG, "triattn_project: pointers must be 16-byte aligned");
   PTX_DISPATCH(dtype, ptx::triattn_project<T>(z, ln_w, ln_b, w_q, w_k, w_v, w_g, w_b, q, k, vt, g,
@@ -188,7 +192,8 @@ PTX_API int ptx_triattn_output(const void* o, const void* w_o, const void* z, vo
   if (n == 0) return PTX_OK;
   PTX_REQUIRE(o && w_o && out && (!add_residual || z), PTX_ERR_BAD_ARG,
               "triattn_output: null pointer");
-  PTX_REQUIRE(aligned16(o) && aligned16(w_o), PTX_ERR_BAD_ARG,
+  PTX_REQUIRE(aligned16(o) && aligned16(w_o) && aligned16(out) && (!z || aligned16(z)),
+              PTX_ERR_BAD_ARG,
               "triattn_output: pointers must be 16-byte aligned");
   PTX_DISPATCH(dtype, ptx::triattn_output<T>(o, w_o, z, out, n, transposed, add_residual,
                                              (hipStream_t)stream));
@@ -209,7 +214,8 @@ PTX_API int ptx_transition_fwd(const void* x, const void* ln_w, const void* ln_b
   PTX_REQUIRE(x && w_a && w_b && w_o && hidden && out, PTX_ERR_BAD_ARG,
               "transition: null pointer");
   PTX_REQUIRE(aligned16(x) && aligned16(w_a) && aligned16(w_b) && aligned16(w_o) &&
-                  aligned16(hidden) && (!ln_w || aligned16(ln_w)) && (!ln_b || aligned16(ln_b)),
+                  aligned16(hidden) && aligned16(out) && (!ln_w || aligned16(ln_w)) &&
+                  (!ln_b || aligned16(ln_b)),
               PTX_ERR_BAD_ARG, "transition: pointers must be 16-byte aligned");
   PTX_DISPATCH(dtype, ptx::transition_fwd<T>(x, ln_w, ln_b, w_a, w_b, w_o, hidden, out, rows,
                                              n_factor, add_residual, eps, (hipStream_t)stream));
@@ -227,7 +233,7 @@ PTX_API int ptx_pair_bias_fwd(const void* z, const void* ln_w, const void* ln_b,
   PTX_REQUIRE(n < 32768, PTX_ERR_UNSUPPORTED, "pair_bias: n=%d too large", n);
   if (n == 0) return PTX_OK;
   PTX_REQUIRE(z && w && bias, PTX_ERR_BAD_ARG, "pair_bias: null pointer");
-  PTX_REQUIRE(aligned16(z) && aligned16(w) && (!ln_w || aligned16(ln_w)) &&
+  PTX_REQUIRE(aligned16(z) && aligned16(w) && aligned16(bias) && (!ln_w || aligned16(ln_w)) &&
                   (!ln_b || aligned16(ln_b)),
               PTX_ERR_BAD_ARG, "pair_bias: pointers must be 16-byte aligned");
   PTX_DISPATCH(dtype, ptx::pair_bias_fwd<T>(z, ln_w, ln_b, w, bias, n, heads, out_f32, eps,

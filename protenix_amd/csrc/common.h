@@ -99,10 +99,12 @@ struct RowMap {
   int64_t stride_outer;
   int64_t stride_inner;
   int n_inner;
+  // p < 2^31 (the API bounds n and the row counts), so 32-bit division suffices
   __device__ __forceinline__ int64_t operator()(int64_t p) const {
-    int64_t o = p / n_inner;
-    int64_t i = p - o * n_inner;
-    return o * stride_outer + i * stride_inner;
+    const uint32_t pp = (uint32_t)p;
+    const uint32_t o = pp / (uint32_t)n_inner;
+    const uint32_t i = pp - o * (uint32_t)n_inner;
+    return (int64_t)o * stride_outer + (int64_t)i * stride_inner;
   }
 };
 

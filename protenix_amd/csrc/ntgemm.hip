@@ -41,7 +41,7 @@ __global__ __launch_bounds__(256) void nt_gemm_batched_kernel(const T* __restric
   const T* a_c = a + (int64_t)c * n * k_pitch;
   const T* b_c = b + (int64_t)c * n * k_pitch;
 
-  // per-lane row pointers (rows beyond n read row 0 and are zeroed)
+  // per-lane row pointers (rows beyond n read row 0; those outputs are never stored)
   const T* a_ptr[2];
   bool a_ok[2];
 #pragma unroll
@@ -64,7 +64,7 @@ __global__ __launch_bounds__(256) void nt_gemm_batched_kernel(const T* __restric
     for (int kk = 0; kk < KK; ++kk) {
 #pragma unroll
       for (int rb = 0; rb < 2; ++rb) {
-        V8 v = a_ok[rb] ? load8<T>(a_ptr[rb] + k0 + 16 * kk) : zero8<T>();
+        V8 v = load8<T>(a_ptr[rb] + k0 + 16 * kk);   // rows beyond n: clamped, never stored
         if (tail) {
 #pragma unroll
           for (int t = 0; t < 8; ++t)
@@ -72,7 +72,7 @@ __global__ __launch_bounds__(256) void nt_gemm_batched_kernel(const T* __restric
         }
         a_nxt[rb][kk] = v;
       }
-      V8 v = b_ok ? load8<T>(b_ptr + k0 + 16 * kk) : zero8<T>();
+      V8 v = load8<T>(b_ptr + k0 + 16 * kk);
       if (tail) {
 #pragma unroll
         for (int t = 0; t < 8; ++t)

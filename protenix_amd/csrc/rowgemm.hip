@@ -1,18 +1,24 @@
 // Row-tile projections with K = 128: every pair-tensor row (one (i,j) position,
 // 128 channels) is normalised in registers and multiplied by small weight
 // matrices on MFMA; gates, masks, SwiGLU and residual adds are applied to the
-// accumulators before anything is written.
+// accumulators, and results leave through an LDS transpose as 16-byte, fully
+// coalesced stores.
 //
 // A wave owns RB blocks of 32 rows.  A row block lives in registers as 8
-// operand fragments (16-deep K steps, see common.h): lane (l%32) holds row
-// l%32, channels 16*kk + 8*(l/32) .. +7.  The same registers serve as the A
-// operand (result: lane <-> output column, used for row-major outputs) or as
-// the B operand (result: lane <-> row, used for channel-major outputs), so one
-// kernel writes both layouts with 64-byte-contiguous stores.
+// operand fragments (16-deep K steps, see common.h): lane l holds row l%32,
+// channels 16*kk + 8*(l/32) .. +7.  The same registers serve as the B operand
+// (result: lane <-> row, register <-> output column; used for row-major
+// outputs) or as the A operand (lane <-> output channel, register <-> row; used
+// for channel-major outputs).  Either way a 32 x 32 result tile sits in the
+// wave as "lane = major index, 4 consecutive minors per register quad", is
+// written to a per-wave LDS tile [major][minor] with 8-byte stores and read
+// back as vectors of consecutive minors, which is exactly the global layout.
 //
 // Weights are staged through LDS already permuted into fragment order
 // ([fragment][lane] -> conflict-free 16-byte reads), two 32-column tiles per
-// chunk, double-buffered, one barrier per chunk.
+// chunk, double-buffered for bf16.  All loads in the hot loops are
+// unconditional (indices are clamped, results of out-of-range rows are simply
+// not stored) so the MFMA loops carry no branches.
 #include "common.h"
 #include "kernels.h"
 
@@ -21,14 +27,68 @@ namespace ptx {
 constexpr int kC = 128;       // channels per pair-tensor row == K of every product here
 constexpr int kKSteps = 8;    // kC / 16
 
+template <typename T> struct Cfg {
+  static constexpr int VE = 16 / (int)sizeof(T);     // elements per 16-byte vector
+  static constexpr int LPM = 32 / VE;                // lanes that cover one 32-long major row
+  static constexpr int MPP = kWave / LPM;            // major rows per read-back pass
+  static constexpr int NPASS = 32 / MPP;             // passes per 32 x 32 tile
+  // Row pitch of the staging tile: bf16 36 elements = 18 dwords, fp32 34 elements = 34
+  // dwords; both spread the 16 lanes of an 8-byte store phase over all 32 banks.  Rows are
+  // 8-byte aligned, so the tile is accessed with 8-byte LDS operations only.
+  static constexpr int PITCH = 32 + 8 / (int)sizeof(T);
+  static constexpr int NBUF = sizeof(T) == 2 ? 2 : 1;    // weight buffers in LDS
+};
+
 template <typename T, int RB>
 struct RowFrags {
   typename Vec8<T>::type f[RB][kKSteps];
 };
 
-// Load RB*32 rows starting at row0 (rows >= n_rows read as zero) and, if LN,
-// normalise them: fp32 statistics, gamma/beta (either may be null) applied in
-// fp32, result rounded to T like the reference's LayerNorm output.
+// Mean / rstd of a 128-channel row spread over the two half-wave lanes that hold it,
+// then gamma/beta (either may be null); result rounded to T like the reference's
+// LayerNorm output.
+template <typename T>
+__device__ __forceinline__ void normalize_row(f32x8 (&v)[kKSteps], const T* __restrict__ gamma,
+                                              const T* __restrict__ beta, float eps, int g,
+                                              typename Vec8<T>::type (&out)[kKSteps]) {
+  float s = 0.0f;
+#pragma unroll
+  for (int kk = 0; kk < kKSteps; ++kk)
+#pragma unroll
+    for (int t = 0; t < 8; ++t) s += v[kk][t];
+  s += swap32(s);
+  const float mean = s * (1.0f / kC);
+  float q = 0.0f;
+#pragma unroll
+  for (int kk = 0; kk < kKSteps; ++kk)
+#pragma unroll
+    for (int t = 0; t < 8; ++t) {
+      const float d = v[kk][t] - mean;
+      q += d * d;
+    }
+  q += swap32(q);
+  const float rstd = rsqrtf(q * (1.0f / kC) + eps);
+#pragma unroll
+  for (int kk = 0; kk < kKSteps; ++kk) {
+    f32x8 o;
+#pragma unroll
+    for (int t = 0; t < 8; ++t) o[t] = (v[kk][t] - mean) * rstd;
+    if (gamma) {
+      const f32x8 gm = to_f32(load8<T>(gamma + 16 * kk + 8 * g));
+#pragma unroll
+      for (int t = 0; t < 8; ++t) o[t] *= gm[t];
+    }
+    if (beta) {
+      const f32x8 bt = to_f32(load8<T>(beta + 16 * kk + 8 * g));
+#pragma unroll
+      for (int t = 0; t < 8; ++t) o[t] += bt[t];
+    }
+    out[kk] = from_f32<T>(o);
+  }
+}
+
+// Load RB*32 rows starting at row0 (rows >= n_rows re-read the last valid row;
+// their results are never stored) and, if LN, normalise them.
 template <typename T, int RB, bool LN>
 __device__ __forceinline__ void load_rows(RowFrags<T, RB>& out, const T* __restrict__ x,
                                           const RowMap& map, int64_t row0, int64_t n_rows,
@@ -37,121 +97,100 @@ __device__ __forceinline__ void load_rows(RowFrags<T, RB>& out, const T* __restr
   const int n = lane & 31, g = lane >> 5;
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
-    const int64_t p = row0 + rb * 32 + n;
-    const bool valid = p < n_rows;
-    const T* rp = x + map(valid ? p : 0) + 8 * g;
+    int64_t p = row0 + rb * 32 + n;
+    p = p < n_rows ? p : n_rows - 1;
+    const T* rp = x + map(p) + 8 * g;
     if (!LN) {
 #pragma unroll
-      for (int kk = 0; kk < kKSteps; ++kk)
-        out.f[rb][kk] = valid ? load8<T>(rp + 16 * kk) : zero8<T>();
+      for (int kk = 0; kk < kKSteps; ++kk) out.f[rb][kk] = load8<T>(rp + 16 * kk);
     } else {
       f32x8 v[kKSteps];
 #pragma unroll
-      for (int kk = 0; kk < kKSteps; ++kk) v[kk] = to_f32(valid ? load8<T>(rp + 16 * kk) : zero8<T>());
-      float s = 0.0f;
-#pragma unroll
-      for (int kk = 0; kk < kKSteps; ++kk)
-#pragma unroll
-        for (int t = 0; t < 8; ++t) s += v[kk][t];
-      s += swap32(s);
-      const float mean = s * (1.0f / kC);
-      float q = 0.0f;
-#pragma unroll
-      for (int kk = 0; kk < kKSteps; ++kk)
-#pragma unroll
-        for (int t = 0; t < 8; ++t) {
-          const float d = v[kk][t] - mean;
-          q += d * d;
-        }
-      q += swap32(q);
-      const float rstd = rsqrtf(q * (1.0f / kC) + eps);
-#pragma unroll
-      for (int kk = 0; kk < kKSteps; ++kk) {
-        f32x8 o;
-#pragma unroll
-        for (int t = 0; t < 8; ++t) o[t] = (v[kk][t] - mean) * rstd;
-        if (gamma) {
-          const f32x8 gm = to_f32(load8<T>(gamma + 16 * kk + 8 * g));
-#pragma unroll
-          for (int t = 0; t < 8; ++t) o[t] *= gm[t];
-        }
-        if (beta) {
-          const f32x8 bt = to_f32(load8<T>(beta + 16 * kk + 8 * g));
-#pragma unroll
-          for (int t = 0; t < 8; ++t) o[t] += bt[t];
-        }
-        out.f[rb][kk] = from_f32<T>(o);
-      }
-    }
-  }
-}
-
-// Same, for a channel-major source x[c][p] (the triangle product): lane gathers
-// its 8 channels per fragment with element loads that are contiguous across
-// lanes (32 consecutive rows per channel).
-template <typename T, int RB>
-__device__ __forceinline__ void load_rows_channel_major_ln(RowFrags<T, RB>& out,
-                                                           const T* __restrict__ x,
-                                                           int64_t chan_stride, int64_t row0,
-                                                           int64_t n_rows,
-                                                           const T* __restrict__ gamma,
-                                                           const T* __restrict__ beta, float eps,
-                                                           int lane) {
-  const int n = lane & 31, g = lane >> 5;
-#pragma unroll
-  for (int rb = 0; rb < RB; ++rb) {
-    const int64_t p = row0 + rb * 32 + n;
-    const bool valid = p < n_rows;
-    const T* rp = x + (valid ? p : 0) + (int64_t)(8 * g) * chan_stride;
-    f32x8 v[kKSteps];
-#pragma unroll
-    for (int kk = 0; kk < kKSteps; ++kk)
-#pragma unroll
-      for (int t = 0; t < 8; ++t)
-        v[kk][t] = valid ? to_f32(rp[(int64_t)(16 * kk + t) * chan_stride]) : 0.0f;
-    float s = 0.0f;
-#pragma unroll
-    for (int kk = 0; kk < kKSteps; ++kk)
-#pragma unroll
-      for (int t = 0; t < 8; ++t) s += v[kk][t];
-    s += swap32(s);
-    const float mean = s * (1.0f / kC);
-    float q = 0.0f;
-#pragma unroll
-    for (int kk = 0; kk < kKSteps; ++kk)
-#pragma unroll
-      for (int t = 0; t < 8; ++t) {
-        const float d = v[kk][t] - mean;
-        q += d * d;
-      }
-    q += swap32(q);
-    const float rstd = rsqrtf(q * (1.0f / kC) + eps);
-#pragma unroll
-    for (int kk = 0; kk < kKSteps; ++kk) {
-      f32x8 o;
-      const f32x8 gm = to_f32(load8<T>(gamma + 16 * kk + 8 * g));
-      const f32x8 bt = to_f32(load8<T>(beta + 16 * kk + 8 * g));
-#pragma unroll
-      for (int t = 0; t < 8; ++t) o[t] = (v[kk][t] - mean) * rstd * gm[t] + bt[t];
-      out.f[rb][kk] = from_f32<T>(o);
+      for (int kk = 0; kk < kKSteps; ++kk) v[kk] = to_f32(load8<T>(rp + 16 * kk));
+      normalize_row<T>(v, gamma, beta, eps, g, out.f[rb]);
     }
   }
 }
 
 // One weight fragment: 32 output columns x 16 K values, lane -> (column l%32,
-// K = k0 + 8*(l/32) ..+7) of a row-major weight w[n_out][ldw].  Rows >= n_out
-// read as zero.
+// K = k0 + 8*(l/32) ..+7) of a row-major weight w[n_out][ldw].  Columns beyond
+// n_out re-read the last row: their outputs are never stored.
 template <typename T>
 __device__ __forceinline__ typename Vec8<T>::type load_wfrag(const T* __restrict__ w, int ldw,
                                                              int n_out, int col0, int k0,
                                                              int lane) {
-  const int col = col0 + (lane & 31);
-  if (col >= n_out) return zero8<T>();
+  int col = col0 + (lane & 31);
+  col = col < n_out ? col : n_out - 1;
   return load8<T>(w + (int64_t)col * ldw + k0 + 8 * (lane >> 5));
 }
 
+// ---- per-wave 32 x 32 staging tile -----------------------------------------
+template <typename T> struct VecE;
+template <> struct VecE<bf16_t> { typedef bf16x8 type; };
+template <> struct VecE<float> { typedef f32x4 type; };
+typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
+
+// put: lane n = major index, vals[r] = value at minor acc_row(r, g).
+template <typename T>
+__device__ __forceinline__ void stage_put(T* st, const float (&vals)[16], int lane) {
+  typedef typename Vec4<T>::type V4;
+  const int n = lane & 31, g = lane >> 5;
+#pragma unroll
+  for (int qd = 0; qd < 4; ++qd) {
+    f32x4 v;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[e] = vals[4 * qd + e];
+    const V4 pk = from_f32<T>(v);
+    T* dst = st + n * Cfg<T>::PITCH + 8 * qd + 4 * g;
+    if constexpr (sizeof(T) == 2) {
+      *reinterpret_cast<V4*>(dst) = pk;                        // 8 bytes
+    } else {
+      reinterpret_cast<f32x2*>(dst)[0] = f32x2{pk[0], pk[1]};  // 2 x 8 bytes
+      reinterpret_cast<f32x2*>(dst)[1] = f32x2{pk[2], pk[3]};
+    }
+  }
+}
+// Coordinates this lane serves in read-back pass `ps`: major row and first minor.
+template <typename T>
+__device__ __forceinline__ void stage_coord(int ps, int lane, int& major, int& minor0) {
+  major = ps * Cfg<T>::MPP + lane / Cfg<T>::LPM;
+  minor0 = (lane % Cfg<T>::LPM) * Cfg<T>::VE;
+}
+// get / put one 16-byte vector (VE consecutive minors of one major row), raw.
+template <typename T>
+__device__ __forceinline__ typename VecE<T>::type stage_get_vec(const T* st, int major,
+                                                                int minor0) {
+  const u32x2* src = reinterpret_cast<const u32x2*>(st + major * Cfg<T>::PITCH + minor0);
+  u32x2 h[2] = {src[0], src[1]};
+  return *reinterpret_cast<typename VecE<T>::type*>(h);
+}
+template <typename T>
+__device__ __forceinline__ void stage_put_vec(T* st, int major, int minor0,
+                                              typename VecE<T>::type v) {
+  u32x2* dst = reinterpret_cast<u32x2*>(st + major * Cfg<T>::PITCH + minor0);
+  const u32x2* s = reinterpret_cast<const u32x2*>(&v);
+  dst[0] = s[0];
+  dst[1] = s[1];
+}
+// v += residual (both in T, sum in fp32, rounded once more like the reference's `z + update`)
+template <typename T>
+__device__ __forceinline__ typename VecE<T>::type add_vec(typename VecE<T>::type v,
+                                                          typename VecE<T>::type r) {
+  typename VecE<T>::type o;
+#pragma unroll
+  for (int e = 0; e < Cfg<T>::VE; ++e) o[e] = from_f32<T>(to_f32(v[e]) + to_f32(r[e]));
+  return o;
+}
+
+// LDS traffic inside one wave: make the stores visible before the loads.
+__device__ __forceinline__ void wave_lds_sync() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+}
+
 // ---------------------------------------------------------------------------
-// rowgemm_in: [LayerNorm] -> chunks of two 32-column weight tiles -> epilogue.
+// rowgemm_in: LayerNorm -> chunks of two 32-column weight tiles -> epilogue.
 // ---------------------------------------------------------------------------
 struct RowGemmInParams {
   const void* x;        // pair tensor, rows addressed through xmap
@@ -186,8 +225,7 @@ __device__ __forceinline__ int n_chunks(const RowGemmInParams& p) {
   return 4;                                        // kTriMulOut: 4 column blocks
 }
 
-// Weight matrix, its row count, first row and whether the tile exists, for
-// tile `t` (0/1) of chunk `ch`.
+// Weight matrix, its row count and first row for tile `t` (0/1) of chunk `ch`.
 template <typename T, int MODE>
 __device__ __forceinline__ void chunk_tile(const RowGemmInParams& p, int ch, int t, const T*& w,
                                            int& n_out, int& col0) {
@@ -198,7 +236,7 @@ __device__ __forceinline__ void chunk_tile(const RowGemmInParams& p, int ch, int
   } else if (MODE == kTriAttnIn) {    // w: q, k, g, v, bias
     const int which = ch >> 1;
     w = (const T*)p.w[which];
-    n_out = which == 4 ? (t == 0 ? p.aux : 0) : kC;
+    n_out = which == 4 ? p.aux : kC;
     col0 = which == 4 ? 0 : ((ch & 1) * 2 + t) * 32;
   } else if (MODE == kTransitionIn) { // w: a, b ; tile0 = a, tile1 = b
     w = (const T*)p.w[t];
@@ -206,7 +244,7 @@ __device__ __forceinline__ void chunk_tile(const RowGemmInParams& p, int ch, int
     col0 = ch * 32;
   } else if (MODE == kPairBias) {
     w = (const T*)p.w[0];
-    n_out = t == 0 ? (p.aux & 0xff) : 0;
+    n_out = p.aux & 0xff;
     col0 = 0;
   } else {                            // kTriMulOut: w: z, g
     w = (const T*)p.w[t];
@@ -215,23 +253,106 @@ __device__ __forceinline__ void chunk_tile(const RowGemmInParams& p, int ch, int
   }
 }
 
+// Element offset of logical row p inside one channel plane [n][pitch], or -1 if p
+// is out of range.  With n % VE == 0, VE rows starting at a multiple of VE share
+// one plane row and are contiguous.
+__device__ __forceinline__ int64_t plane_offset(int64_t p, int64_t n_rows, int n, int64_t pitch) {
+  if (p >= n_rows) return -1;
+  const uint32_t i = (uint32_t)p / (uint32_t)n;
+  return (int64_t)i * pitch + ((uint32_t)p - i * (uint32_t)n);
+}
+
 template <typename T, int RB, int MODE>
 __global__ __launch_bounds__(256) void rowgemm_in_kernel(RowGemmInParams p) {
   typedef typename Vec8<T>::type V8;
-  __shared__ V8 lds_w[2][2 * kKSteps][kWave];
+  typedef typename VecE<T>::type VE_t;
+  typedef Cfg<T> C;
+  __shared__ V8 lds_w[C::NBUF][2 * kKSteps][kWave];
+  __shared__ __attribute__((aligned(16))) T lds_stage[4][32 * C::PITCH];
+  __shared__ __attribute__((aligned(16))) float lds_mask[4][RB * 32];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int n = lane & 31, g = lane >> 5;
   const int64_t row0 = ((int64_t)blockIdx.x * 4 + wave) * (RB * 32);
+  T* st = lds_stage[wave];
+  const bool vec_ok = (p.n % C::VE) == 0;   // channel-major vectors stay inside one plane row
 
   RowFrags<T, RB> xf;
   load_rows<T, RB, true>(xf, (const T*)p.x, p.xmap, row0, p.n_rows, (const T*)p.gamma,
                          (const T*)p.beta, p.eps, lane);
-  // second fragment set only exists for the triangle-product epilogue
+
+  // kTriMulOut: second fragment set = LayerNorm_out of the channel-major triangle product,
+  // transposed through the staging tile 32 channels at a time.
   RowFrags<T, RB> xf2;   // dead (and removed by the compiler) in the other modes
   if constexpr (MODE == kTriMulOut) {
-    load_rows_channel_major_ln<T, RB>(xf2, (const T*)p.x2, p.n_rows, row0, p.n_rows,
-                                      (const T*)p.gamma2, (const T*)p.beta2, p.eps, lane);
+    const T* x2 = (const T*)p.x2;
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) {
+      f32x8 v[kKSteps];
+#pragma unroll
+      for (int cg = 0; cg < 4; ++cg) {           // channels 32*cg .. +31
+        VE_t vec[C::NPASS];
+#pragma unroll
+        for (int ps = 0; ps < C::NPASS; ++ps) {
+          int chn, r0;
+          stage_coord<T>(ps, lane, chn, r0);
+          const int64_t pr = row0 + rb * 32 + r0;
+          const T* src = x2 + (int64_t)(32 * cg + chn) * p.n_rows;
+          if (vec_ok) {
+            const int64_t pc = pr + C::VE <= p.n_rows ? pr : 0;
+            vec[ps] = *reinterpret_cast<const VE_t*>(src + pc);
+          } else {
+#pragma unroll
+            for (int e = 0; e < C::VE; ++e) {
+              const int64_t pe = pr + e < p.n_rows ? pr + e : p.n_rows - 1;
+              vec[ps][e] = src[pe];
+            }
+          }
+        }
+        wave_lds_sync();
+#pragma unroll
+        for (int ps = 0; ps < C::NPASS; ++ps) {
+          int chn, r0;
+          stage_coord<T>(ps, lane, chn, r0);
+          stage_put_vec<T>(st, chn, r0, vec[ps]);
+        }
+        wave_lds_sync();
+        // lane (row n, half g) picks channels 16*kk + 8*g + t of this group
+#pragma unroll
+        for (int k2 = 0; k2 < 2; ++k2)
+#pragma unroll
+          for (int t = 0; t < 8; ++t)
+            v[2 * cg + k2][t] = to_f32(st[(16 * k2 + 8 * g + t) * C::PITCH + n]);
+      }
+      normalize_row<T>(v, (const T*)p.gamma2, (const T*)p.beta2, p.eps, g, xf2.f[rb]);
+    }
   }
+
+  // TriMulIn: the 32 mask values of each row block, shared through LDS
+  if constexpr (MODE == kTriMulIn) {
+    if (p.mask) {
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb) {
+        int64_t pr = row0 + rb * 32 + n;
+        pr = pr < p.n_rows ? pr : p.n_rows - 1;
+        const float mv = to_f32(((const T*)p.mask)[p.mmap(pr)]);
+        if (g == 0) lds_mask[wave][rb * 32 + n] = mv;
+      }
+      wave_lds_sync();
+    }
+  }
+
+  // Row-major destinations (kTriAttnIn q/k/g, kTransitionIn hidden, kTriMulOut out): the
+  // logical row this lane stores in each read-back pass, or -1.
+  int64_t rrow[RB][C::NPASS];
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+    for (int ps = 0; ps < C::NPASS; ++ps) {
+      int mj, m0;
+      stage_coord<T>(ps, lane, mj, m0);
+      const int64_t pr = row0 + rb * 32 + mj;
+      rrow[rb][ps] = pr < p.n_rows ? pr : -1;
+    }
 
   const int nch = n_chunks<MODE>(p);
   V8 pre[4];
@@ -253,15 +374,56 @@ __global__ __launch_bounds__(256) void rowgemm_in_kernel(RowGemmInParams p) {
   stash(0);
   __syncthreads();
 
+  // Row-major store of the staged tile (major = row, minor = 32 output columns at col0).
+  auto store_row_major = [&](T* outp, int64_t ld, int col0, int rb, const T* resp) {
+#pragma unroll
+    for (int ps = 0; ps < C::NPASS; ++ps) {
+      int mj, m0;
+      stage_coord<T>(ps, lane, mj, m0);
+      if (rrow[rb][ps] >= 0) {
+        const int64_t off = rrow[rb][ps] * ld + col0 + m0;
+        VE_t v = stage_get_vec<T>(st, mj, m0);
+        if (resp) v = add_vec<T>(v, *reinterpret_cast<const VE_t*>(resp + off));
+        *reinterpret_cast<VE_t*>(outp + off) = v;
+      }
+    }
+  };
+  // Channel-major store of the staged tile: major = channel (first = c_first, only
+  // channels < c_lim exist), minor = the 32 logical rows of row block rb; a channel's
+  // plane is [n][row_pitch] and planes are plane_stride apart.
+  auto store_channel_major = [&](T* plane0, int64_t plane_stride, int64_t row_pitch, int c_first,
+                                 int c_lim, int rb) {
+#pragma unroll
+    for (int ps = 0; ps < C::NPASS; ++ps) {
+      int chn, r0;
+      stage_coord<T>(ps, lane, chn, r0);
+      const int64_t pr = row0 + rb * 32 + r0;
+      if (c_first + chn < c_lim) {
+        T* dst = plane0 + (int64_t)(c_first + chn) * plane_stride;
+        const VE_t v = stage_get_vec<T>(st, chn, r0);
+        if (vec_ok) {
+          const int64_t off = plane_offset(pr, p.n_rows, p.n, row_pitch);
+          if (off >= 0) *reinterpret_cast<VE_t*>(dst + off) = v;
+        } else {
+#pragma unroll
+          for (int e = 0; e < C::VE; ++e) {
+            const int64_t off = plane_offset(pr + e, p.n_rows, p.n, row_pitch);
+            if (off >= 0) dst[off] = v[e];
+          }
+        }
+      }
+    }
+  };
+
   for (int ch = 0; ch < nch; ++ch) {
-    const int buf = ch & 1;
+    const int buf = C::NBUF == 2 ? (ch & 1) : 0;
     if (ch + 1 < nch) fetch(ch + 1);
 
-    // Orientation: channel-major outputs want lane <-> row (weights as A).
-    bool rows_on_lanes;
-    if (MODE == kTriMulIn || MODE == kPairBias) rows_on_lanes = true;
-    else if (MODE == kTriAttnIn) rows_on_lanes = (ch >= 6);   // v^T and the triangle bias
-    else rows_on_lanes = false;
+    // Orientation: channel-major outputs want lane <-> channel (x as A operand).
+    bool chan_on_lanes;
+    if (MODE == kTriMulIn || MODE == kPairBias) chan_on_lanes = true;
+    else if (MODE == kTriAttnIn) chan_on_lanes = (ch >= 6);   // v^T and the triangle bias
+    else chan_on_lanes = false;
 
     f32x16 acc[RB][2];
 #pragma unroll
@@ -271,22 +433,30 @@ __global__ __launch_bounds__(256) void rowgemm_in_kernel(RowGemmInParams p) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[rb][t][r] = 0.0f;
 
+    if (chan_on_lanes) {
 #pragma unroll
-    for (int kk = 0; kk < kKSteps; ++kk) {
-      const V8 w0 = lds_w[buf][kk][lane];
-      const V8 w1 = lds_w[buf][kKSteps + kk][lane];
+      for (int kk = 0; kk < kKSteps; ++kk) {
+        const V8 w0 = lds_w[buf][kk][lane];
+        const V8 w1 = lds_w[buf][kKSteps + kk][lane];
 #pragma unroll
-      for (int rb = 0; rb < RB; ++rb) {
-        if constexpr (MODE == kTriMulOut) {
-          mma32(acc[rb][0], xf2.f[rb][kk], w0);   // W_z LN_out(x)
-          mma32(acc[rb][1], xf.f[rb][kk], w1);    // W_g LN_in(z)
-        } else {
-          if (rows_on_lanes) {
+        for (int rb = 0; rb < RB; ++rb) {
+          mma32(acc[rb][0], xf.f[rb][kk], w0);
+          mma32(acc[rb][1], xf.f[rb][kk], w1);
+        }
+      }
+    } else {
+#pragma unroll
+      for (int kk = 0; kk < kKSteps; ++kk) {
+        const V8 w0 = lds_w[buf][kk][lane];
+        const V8 w1 = lds_w[buf][kKSteps + kk][lane];
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) {
+          if constexpr (MODE == kTriMulOut) {
+            mma32(acc[rb][0], w0, xf2.f[rb][kk]);   // W_z LN_out(x)
+            mma32(acc[rb][1], w1, xf.f[rb][kk]);    // W_g LN_in(z)
+          } else {
             mma32(acc[rb][0], w0, xf.f[rb][kk]);
             mma32(acc[rb][1], w1, xf.f[rb][kk]);
-          } else {
-            mma32(acc[rb][0], xf.f[rb][kk], w0);
-            mma32(acc[rb][1], xf.f[rb][kk], w1);
           }
         }
       }
@@ -294,134 +464,148 @@ __global__ __launch_bounds__(256) void rowgemm_in_kernel(RowGemmInParams p) {
 
     // ------------------------------ epilogues ------------------------------
     if constexpr (MODE == kTriMulIn) {
-      // a/b[c][p] = mask(p) * sigmoid(gate) * proj ; lane <-> row p, register <-> channel
+      // a/b[c][i][k] = mask * sigmoid(gate) * proj ; lane <-> channel, register <-> row
       T* outp = (T*)p.out[ch >> 2];
       const int c0 = (ch & 3) * 32;
 #pragma unroll
       for (int rb = 0; rb < RB; ++rb) {
-        const int64_t row = row0 + rb * 32 + n;
-        if (row < p.n_rows) {
-          const float m = p.mask ? to_f32(((const T*)p.mask)[p.mmap(row)]) : 1.0f;
-          const int64_t i = row / p.n, kq = row - i * p.n;
-          T* base = outp + i * p.pitch + kq;
-          const int64_t cstride = (int64_t)p.n * p.pitch;
+        float vals[16];
 #pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            const float v = m * sigmoidf_fast(acc[rb][1][r]) * acc[rb][0][r];
-            base[(c0 + acc_row(r, g)) * cstride] = from_f32<T>(v);
+        for (int qd = 0; qd < 4; ++qd) {
+          f32x4 m4 = {1.0f, 1.0f, 1.0f, 1.0f};
+          if (p.mask)
+            m4 = *reinterpret_cast<const f32x4*>(&lds_mask[wave][rb * 32 + 8 * qd + 4 * g]);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const int r = 4 * qd + e;
+            vals[r] = m4[e] * sigmoidf_fast(acc[rb][1][r]) * acc[rb][0][r];
           }
         }
+        wave_lds_sync();
+        stage_put<T>(st, vals, lane);
+        wave_lds_sync();
+        store_channel_major(outp, (int64_t)p.n * p.pitch, p.pitch, c0, kC, rb);
       }
     } else if constexpr (MODE == kTriAttnIn) {
       const int which = ch >> 1;
       if (which < 3) {
-        // q (scaled), k, sigmoid(g): row-major [p][128]; lane <-> column, register <-> row
+        // q (rounded, then scaled), k, sigmoid(g): row-major [p][128]
         T* outp = (T*)p.out[which];
 #pragma unroll
         for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
           for (int t = 0; t < 2; ++t) {
-            const int col = ((ch & 1) * 2 + t) * 32 + n;
+            float vals[16];
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-              const int64_t row = row0 + rb * 32 + acc_row(r, g);
-              if (row < p.n_rows) {
-                float v = acc[rb][t][r];
-                if (which == 0) v = to_f32(from_f32<T>(v)) * p.q_scale;   // q rounded, then scaled
-                if (which == 2) v = sigmoidf_fast(v);
-                outp[row * kC + col] = from_f32<T>(v);
-              }
+              float v = acc[rb][t][r];
+              if (which == 0) v = to_f32(from_f32<T>(v)) * p.q_scale;
+              if (which == 2) v = sigmoidf_fast(v);
+              vals[r] = v;
             }
+            wave_lds_sync();
+            stage_put<T>(st, vals, lane);
+            wave_lds_sync();
+            store_row_major(outp, kC, ((ch & 1) * 2 + t) * 32, rb, nullptr);
           }
       } else if (which == 3) {
-        // v^T[i][c][j]: lane <-> row p = i*n + j, register <-> channel
-        T* outp = (T*)p.out[3];
+        // v^T[i][c][key]: lane <-> channel, register <-> row p = i*n + key.  Channel c of
+        // row i starts at i*128*pitch + c*pitch: planes `pitch` apart, plane rows 128*pitch.
 #pragma unroll
-        for (int rb = 0; rb < RB; ++rb) {
-          const int64_t row = row0 + rb * 32 + n;
-          if (row < p.n_rows) {
-            const int64_t i = row / p.n, j = row - i * p.n;
-            T* base = outp + i * (int64_t)kC * p.pitch + j;
+        for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
-            for (int t = 0; t < 2; ++t)
+          for (int t = 0; t < 2; ++t) {
+            float vals[16];
 #pragma unroll
-              for (int r = 0; r < 16; ++r) {
-                const int c = ((ch & 1) * 2 + t) * 32 + acc_row(r, g);
-                base[(int64_t)c * p.pitch] = from_f32<T>(acc[rb][t][r]);
-              }
+            for (int r = 0; r < 16; ++r) vals[r] = acc[rb][t][r];
+            wave_lds_sync();
+            stage_put<T>(st, vals, lane);
+            wave_lds_sync();
+            store_channel_major((T*)p.out[3], (int64_t)p.pitch, (int64_t)p.pitch * kC,
+                                ((ch & 1) * 2 + t) * 32, kC, rb);
           }
-        }
       } else {
         // triangle bias [h][i][pitch]
-        T* outp = (T*)p.out[4];
 #pragma unroll
         for (int rb = 0; rb < RB; ++rb) {
-          const int64_t row = row0 + rb * 32 + n;
-          if (row < p.n_rows) {
-            const int64_t i = row / p.n, j = row - i * p.n;
-            T* base = outp + i * p.pitch + j;
+          float vals[16];
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-              const int h = acc_row(r, g);
-              if (h < p.aux) base[(int64_t)h * p.n * p.pitch] = from_f32<T>(acc[rb][0][r]);
-            }
-          }
+          for (int r = 0; r < 16; ++r) vals[r] = acc[rb][0][r];
+          wave_lds_sync();
+          stage_put<T>(st, vals, lane);
+          wave_lds_sync();
+          store_channel_major((T*)p.out[4], (int64_t)p.n * p.pitch, p.pitch, 0, p.aux, rb);
         }
       }
     } else if constexpr (MODE == kTransitionIn) {
-      // hidden[p][col] = silu(a) * b ; lane <-> column, register <-> row
-      T* outp = (T*)p.out[0];
-      const int64_t ldh = (int64_t)kC * p.aux;
-      const int col = ch * 32 + n;
+      // hidden[p][col] = silu(a) * b, row-major with leading dimension 128 * n_factor
 #pragma unroll
-      for (int rb = 0; rb < RB; ++rb)
+      for (int rb = 0; rb < RB; ++rb) {
+        float vals[16];
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-          const int64_t row = row0 + rb * 32 + acc_row(r, g);
-          if (row < p.n_rows) {
-            // the reference rounds a and b to T before the activation
-            const float a = to_f32(from_f32<T>(acc[rb][0][r]));
-            const float b = to_f32(from_f32<T>(acc[rb][1][r]));
-            outp[row * ldh + col] = from_f32<T>(a * sigmoidf_fast(a) * b);
-          }
+          // the reference rounds a and b to T before the activation
+          const float a = to_f32(from_f32<T>(acc[rb][0][r]));
+          const float b = to_f32(from_f32<T>(acc[rb][1][r]));
+          vals[r] = a * sigmoidf_fast(a) * b;
         }
+        wave_lds_sync();
+        stage_put<T>(st, vals, lane);
+        wave_lds_sync();
+        store_row_major((T*)p.out[0], (int64_t)kC * p.aux, ch * 32, rb, nullptr);
+      }
     } else if constexpr (MODE == kPairBias) {
+      // bias[h][p], dense planes of n*n elements, fp32 or T; lane <-> head, register <-> row
       const int heads = p.aux & 0xff;
       const bool f32_out = (p.aux >> 8) & 1;
 #pragma unroll
       for (int rb = 0; rb < RB; ++rb) {
-        const int64_t row = row0 + rb * 32 + n;
-        if (row < p.n_rows) {
+        const int64_t pr0 = row0 + rb * 32;
+        if (n < heads) {
 #pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            const int h = acc_row(r, g);
-            if (h < heads) {
-              if (f32_out) ((float*)p.out[0])[(int64_t)h * p.n_rows + row] = acc[rb][0][r];
-              else ((T*)p.out[0])[(int64_t)h * p.n_rows + row] = from_f32<T>(acc[rb][0][r]);
+          for (int qd = 0; qd < 4; ++qd) {
+            const int64_t pr = pr0 + 8 * qd + 4 * g;
+            if (f32_out) {
+              float* dst = (float*)p.out[0] + (int64_t)n * p.n_rows + pr;
+              if (pr + 4 <= p.n_rows && (p.n_rows & 3) == 0) {
+                *reinterpret_cast<f32x4*>(dst) =
+                    f32x4{acc[rb][0][4 * qd], acc[rb][0][4 * qd + 1], acc[rb][0][4 * qd + 2],
+                          acc[rb][0][4 * qd + 3]};
+              } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                  if (pr + e < p.n_rows) dst[e] = acc[rb][0][4 * qd + e];
+              }
+            } else {
+              T* dst = (T*)p.out[0] + (int64_t)n * p.n_rows + pr;
+#pragma unroll
+              for (int e = 0; e < 4; ++e)
+                if (pr + e < p.n_rows) dst[e] = from_f32<T>(acc[rb][0][4 * qd + e]);
             }
           }
         }
       }
     } else {
-      // kTriMulOut: out[p][col] = [z +] (W_z LN_out(x)) * sigmoid(W_g LN_in(z))
-      T* outp = (T*)p.out[0];
-      const T* zres = (const T*)p.x;
-      const int col = ch * 32 + n;
+      // kTriMulOut: out[p][col] = [z +] (W_z LN_out(x)) * sigmoid(W_g LN_in(z)), row-major.
+      // out may alias z: a lane reads the residual vector it is about to overwrite.
 #pragma unroll
-      for (int rb = 0; rb < RB; ++rb)
+      for (int rb = 0; rb < RB; ++rb) {
+        float vals[16];
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-          const int64_t row = row0 + rb * 32 + acc_row(r, g);
-          if (row < p.n_rows) {
-            // linear_z output is rounded to T before the gate multiply
-            float v = to_f32(from_f32<T>(acc[rb][0][r])) * sigmoidf_fast(acc[rb][1][r]);
-            if (p.add_residual) v = to_f32(from_f32<T>(v)) + to_f32(zres[row * kC + col]);
-            outp[row * kC + col] = from_f32<T>(v);
-          }
+          // linear_z output is rounded to T before the gate multiply
+          vals[r] = to_f32(from_f32<T>(acc[rb][0][r])) * sigmoidf_fast(acc[rb][1][r]);
         }
+        wave_lds_sync();
+        stage_put<T>(st, vals, lane);
+        wave_lds_sync();
+        store_row_major((T*)p.out[0], kC, ch * 32, rb,
+                        p.add_residual ? (const T*)p.x : nullptr);
+      }
     }
 
-    if (ch + 1 < nch) stash(buf ^ 1);
+    if (C::NBUF == 1) __syncthreads();      // everyone is done reading the single buffer
+    if (ch + 1 < nch) stash(C::NBUF == 2 ? (buf ^ 1) : 0);
     __syncthreads();
   }
 }
@@ -454,12 +638,15 @@ struct RowGemmOutParams {
 template <typename T, int RB>
 __global__ __launch_bounds__(256) void rowgemm_out_kernel(RowGemmOutParams p) {
   typedef typename Vec8<T>::type V8;
-  __shared__ V8 lds_w[2][2 * kKSteps][kWave];
+  typedef typename VecE<T>::type VE_t;
+  typedef Cfg<T> C;
+  __shared__ V8 lds_w[C::NBUF][2 * kKSteps][kWave];
+  __shared__ __attribute__((aligned(16))) T lds_stage[4][32 * C::PITCH];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int n = lane & 31, g = lane >> 5;
   const int64_t row0 = ((int64_t)blockIdx.x * 4 + wave) * (RB * 32);
   const int K = kC * p.n_slab;
   const T* w = (const T*)p.w;
+  T* st = lds_stage[wave];
 
   f32x16 acc[RB][4];
 #pragma unroll
@@ -469,8 +656,7 @@ __global__ __launch_bounds__(256) void rowgemm_out_kernel(RowGemmOutParams p) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[rb][t][r] = 0.0f;
 
-  // chunk index c -> (slab = c/2, column pair = c%2)
-  const int nch = 2 * p.n_slab;
+  // chunk c -> (slab = c/2, column pair = c%2); one slab (two chunks) per outer iteration
   V8 pre[4];
   auto fetch = [&](int ch) {
 #pragma unroll
@@ -488,51 +674,68 @@ __global__ __launch_bounds__(256) void rowgemm_out_kernel(RowGemmOutParams p) {
   stash(0);
   __syncthreads();
 
-  RowFrags<T, RB> af;
   const RowMap amap{(int64_t)K, 0, 1};   // row p -> p*K (n_inner = 1, so outer = p)
-  for (int ch = 0; ch < nch; ++ch) {
-    const int buf = ch & 1;
-    if (ch + 1 < nch) fetch(ch + 1);
-    if ((ch & 1) == 0) {
-      load_rows<T, RB, false>(af, (const T*)p.a + (ch >> 1) * kC, amap, row0, p.n_rows, nullptr,
-                              nullptr, 0.0f, lane);
-    }
+  const int nch = 2 * p.n_slab;
+  for (int slab = 0; slab < p.n_slab; ++slab) {
+    RowFrags<T, RB> af;
+    load_rows<T, RB, false>(af, (const T*)p.a + slab * kC, amap, row0, p.n_rows, nullptr, nullptr,
+                            0.0f, lane);
 #pragma unroll
-    for (int kk = 0; kk < kKSteps; ++kk) {
-      const V8 w0 = lds_w[buf][kk][lane];
-      const V8 w1 = lds_w[buf][kKSteps + kk][lane];
+    for (int half = 0; half < 2; ++half) {
+      const int ch = 2 * slab + half;
+      const int buf = C::NBUF == 2 ? half : 0;
+      if (ch + 1 < nch) fetch(ch + 1);
 #pragma unroll
-      for (int rb = 0; rb < RB; ++rb) {
-        if (ch & 1) {
-          mma32(acc[rb][2], af.f[rb][kk], w0);
-          mma32(acc[rb][3], af.f[rb][kk], w1);
-        } else {
-          mma32(acc[rb][0], af.f[rb][kk], w0);
-          mma32(acc[rb][1], af.f[rb][kk], w1);
+      for (int kk = 0; kk < kKSteps; ++kk) {
+        const V8 w0 = lds_w[buf][kk][lane];
+        const V8 w1 = lds_w[buf][kKSteps + kk][lane];
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) {
+          // lane <-> row, register <-> output column
+          mma32(acc[rb][2 * half], w0, af.f[rb][kk]);
+          mma32(acc[rb][2 * half + 1], w1, af.f[rb][kk]);
         }
       }
+      if (C::NBUF == 1) __syncthreads();
+      if (ch + 1 < nch) stash(C::NBUF == 2 ? (buf ^ 1) : 0);
+      __syncthreads();
     }
-    if (ch + 1 < nch) stash(buf ^ 1);
-    __syncthreads();
   }
 
+  // out may alias res: a lane reads the residual vector it is about to overwrite.
   T* outp = (T*)p.out;
   const T* resp = (const T*)p.res;
 #pragma unroll
-  for (int rb = 0; rb < RB; ++rb)
+  for (int rb = 0; rb < RB; ++rb) {
+    int64_t obase[C::NPASS];
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int64_t row = row0 + rb * 32 + acc_row(r, g);
-      if (row < p.n_rows) {
-        const int64_t off = p.omap(row) + n;
+    for (int ps = 0; ps < C::NPASS; ++ps) {
+      int mj, m0;
+      stage_coord<T>(ps, lane, mj, m0);
+      const int64_t pr = row0 + rb * 32 + mj;
+      obase[ps] = pr < p.n_rows ? p.omap(pr) + m0 : -1;
+    }
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
-          float v = acc[rb][t][r];
-          if (resp) v = to_f32(from_f32<T>(v)) + to_f32(resp[off + t * 32]);
-          outp[off + t * 32] = from_f32<T>(v);
+    for (int t = 0; t < 4; ++t) {
+      float vals[16];
+#pragma unroll
+      for (int r = 0; r < 16; ++r) vals[r] = acc[rb][t][r];
+      wave_lds_sync();
+      stage_put<T>(st, vals, lane);
+      wave_lds_sync();
+#pragma unroll
+      for (int ps = 0; ps < C::NPASS; ++ps) {
+        int mj, m0;
+        stage_coord<T>(ps, lane, mj, m0);
+        if (obase[ps] >= 0) {
+          const int64_t off = obase[ps] + t * 32;
+          VE_t v = stage_get_vec<T>(st, mj, m0);
+          if (resp) v = add_vec<T>(v, *reinterpret_cast<const VE_t*>(resp + off));
+          *reinterpret_cast<VE_t*>(outp + off) = v;
         }
       }
     }
+  }
 }
 
 template <typename T>
@@ -645,7 +848,7 @@ int transition_fwd(const void* x, const void* ln_w, const void* ln_b, const void
   p.eps = eps;
   p.w[0] = w_a; p.w[1] = w_b;
   p.out[0] = hidden;
-  p.n = 1;
+  p.n = 8;   // rows are independent here; a multiple of the vector width
   p.aux = n_factor;
   launch_rowgemm_in<T, kTransitionIn>(p, stream);
   RowGemmOutParams q = {};
@@ -679,13 +882,13 @@ int pair_bias_fwd(const void* z, const void* ln_w, const void* ln_b, const void*
 #define PTX_INSTANTIATE(T)                                                                          \
   template int trimul_project<T>(const void*, const void*, const void*, const void*, const void*,  \
                                  const void*, const void*, const void*, void*, void*, int, int,    \
-                                 int, float, hipStream_t);                                            \
+                                 int, float, hipStream_t);                                         \
   template int trimul_output<T>(const void*, const void*, const void*, const void*, const void*,   \
                                 const void*, const void*, const void*, void*, int, int, float,     \
                                 hipStream_t);                                                      \
   template int triattn_project<T>(const void*, const void*, const void*, const void*, const void*, \
                                   const void*, const void*, const void*, void*, void*, void*,      \
-                                  void*, void*, int, int, int, int, int, float, hipStream_t);         \
+                                  void*, void*, int, int, int, int, int, float, hipStream_t);      \
   template int triattn_output<T>(const void*, const void*, const void*, void*, int, int, int,      \
                                  hipStream_t);                                                     \
   template int transition_fwd<T>(const void*, const void*, const void*, const void*, const void*,  \

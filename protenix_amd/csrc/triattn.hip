@@ -65,10 +65,10 @@ __global__ __launch_bounds__(256) void triattn_fwd_kernel(
   V8 qf[NQ][2];
 #pragma unroll
   for (int qb = 0; qb < NQ; ++qb) {
-    const int qi = q0 + qb * 32 + ln;
+    // queries beyond n re-read the last one; their results are never stored
+    const int qi = min(q0 + qb * 32 + ln, n - 1);
 #pragma unroll
-    for (int kk = 0; kk < 2; ++kk)
-      qf[qb][kk] = qi < n ? load8<T>(q_row + (int64_t)qi * C + 16 * kk + 8 * g) : zero8<T>();
+    for (int kk = 0; kk < 2; ++kk) qf[qb][kk] = load8<T>(q_row + (int64_t)qi * C + 16 * kk + 8 * g);
   }
 
   const int n_tiles = (n + kKeyTile - 1) / kKeyTile;
@@ -76,8 +76,12 @@ __global__ __launch_bounds__(256) void triattn_fwd_kernel(
   // ---- cooperative tile loader: wave w fetches fragments 2w and 2w+1 ----
   V8 pre[2];
   float pre_mb = 0.0f;
+  // All loads are unconditional (indices clamped): keys beyond n get a -inf mask
+  // bias below, which removes them from the softmax whatever K holds; V^T is zeroed
+  // for them because 0 * garbage must stay 0.
   auto fetch = [&](int tile) {
     const int key0 = tile * kKeyTile;
+    const bool tail = key0 + kKeyTile > n;   // uniform
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
       const int fid = wave * 2 + j;
@@ -85,29 +89,27 @@ __global__ __launch_bounds__(256) void triattn_fwd_kernel(
       if (fid < 4) {
         // K (A operand): MFMA row m <-> key 32*((m>>2)&1) + 16u + 4*(m>>3) + (m&3); slots <-> d
         const int key = key0 + 32 * ((ln >> 2) & 1) + 16 * u + 4 * (ln >> 3) + (ln & 3);
-        pre[j] = key < n ? load8<T>(k_row + (int64_t)key * C + 16 * sub + 8 * g) : zero8<T>();
+        pre[j] = load8<T>(k_row + (int64_t)min(key, n - 1) * C + 16 * sub + 8 * g);
       } else {
         // V^T (A operand): MFMA row <-> d = ln; slots <-> keys 32g + 16u + 8s + t
         const int key = key0 + 32 * g + 16 * u + 8 * sub;
         V8 v = load8<T>(vt_row + (int64_t)ln * key_pitch + key);
-        if (key + 8 > n) {
+        if (tail) {
 #pragma unroll
-          for (int t = 0; t < 8; ++t)
-            if (key + t >= n) v[t] = (T)0.0f;
+          for (int t = 0; t < 8; ++t) v[t] = key + t < n ? v[t] : (T)0.0f;
         }
         pre[j] = v;
       }
     }
     if (wave == 0) {
       const int key = key0 + lane;
+      const int kc = min(key, n - 1);
       float mb = 0.0f;
-      if (key >= n) {
-        mb = -INFINITY;
-      } else if (mask) {
-        const int64_t mi = mask_transposed ? (int64_t)key * n + i : (int64_t)i * n + key;
+      if (mask) {
+        const int64_t mi = mask_transposed ? (int64_t)kc * n + i : (int64_t)i * n + kc;
         mb = inf * (to_f32(mask[mi]) - 1.0f);
       }
-      pre_mb = mb;
+      pre_mb = key < n ? mb : -INFINITY;
     }
   };
   auto stash = [&](int buf) {
@@ -267,6 +269,15 @@ __global__ __launch_bounds__(256) void triattn_fwd_kernel(
   }
 
   // ---- normalise, gate, store: lane <-> query, register r <-> d = acc_row(r, g) ----
+  // o may alias gate: every gate load is issued before the first store.
+  f32x4 gv[NQ][4];
+#pragma unroll
+  for (int qb = 0; qb < NQ; ++qb) {
+    const int qi = q0 + qb * 32 + ln;
+    const int64_t base = ((int64_t)i * n + (qi < n ? qi : 0)) * C + h * kD + 4 * g;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) gv[qb][c] = to_f32(*reinterpret_cast<const V4*>(gate + base + 8 * c));
+  }
 #pragma unroll
   for (int qb = 0; qb < NQ; ++qb) {
     const int qi = q0 + qb * 32 + ln;
@@ -276,12 +287,11 @@ __global__ __launch_bounds__(256) void triattn_fwd_kernel(
       const int64_t base = ((int64_t)i * n + qi) * C + h * kD + 4 * g;
 #pragma unroll
       for (int c = 0; c < 4; ++c) {
-        const f32x4 gv = to_f32(*reinterpret_cast<const V4*>(gate + base + 8 * c));
         f32x4 ov;
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
           // attention output rounded to T before the gate multiply, as the reference does
-          ov[t] = to_f32(from_f32<T>(acc_o[qb][4 * c + t] * inv)) * gv[t];
+          ov[t] = to_f32(from_f32<T>(acc_o[qb][4 * c + t] * inv)) * gv[qb][c][t];
         }
         *reinterpret_cast<V4*>(o + base + 8 * c) = from_f32<T>(ov);
       }
