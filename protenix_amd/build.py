@@ -15,6 +15,9 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libprotenix_amd.so")
 SOURCES = ["api.hip", "layernorm.hip", "rowgemm.hip", "triattn.hip", "ntgemm.hip"]
+# per-source extra flags: the attention kernel's max reductions need no NaN
+# canonicalisation (lets the compiler form v_max3_f32)
+EXTRA_FLAGS = {"triattn.hip": ["-fno-honor-nans"]}
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",
     # keep the compiler from forming packed-fp32 VALU ops
@@ -49,7 +52,7 @@ def build(verbose: bool = False) -> str:
         for src in SOURCES:
             obj = os.path.join(objdir, src.replace(".hip", ".o"))
             objs.append(obj)
-            cmd = [hipcc, *FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+            cmd = [hipcc, *FLAGS, *EXTRA_FLAGS.get(src, []), "-c", os.path.join(CSRC, src), "-o", obj]
             jobs.append(pool.submit(_run, cmd))
         for j in jobs:
             msg = j.result()

@@ -1,27 +1,31 @@
 // Triangle attention core: flash-style online softmax on MFMA, the N^3 logits
 // are never written anywhere.
 //
-// One workgroup (4 waves) owns one (row i, head h) pair and 4*NQ*32 queries;
-// each wave owns NQ blocks of 32 queries and walks over the keys in tiles of 64.
-// Per tile and query block:
-//   S^T[key][query]  = K Q^T            2 x 2 MFMA (two 32-key halves, d = 32)
+// One workgroup (4 waves) owns one (row i, head h) pair and 128 queries; each
+// wave owns 32 queries and walks over the keys in tiles of 64.  Per tile:
+//   S^T[key][query]  = K Q^T + bias     2 x (2 + 2) MFMA (two 32-key halves)
 //   online softmax along keys = along the registers of a lane (+ one exchange
 //   with the other half-wave), because MFMA puts the query on the lane
 //   O^T[d][query]   += V^T P^T          4 MFMA, P^T taken straight from the S^T
-//   accumulators with no shuffle: MFMA row m of half u is mapped to key
-//   32*((m>>2)&1) + 16*u + 4*(m>>3) + (m&3), which makes register r of half-wave
-//   g hold key 32*g + 16*u + r, i.e. 16 consecutive keys -> 16-byte bias loads
-//   and 8 consecutive keys per PV operand slot group.
+//   accumulators with no shuffle
+//   l[query]        += 1^T P^T          4 MFMA (row sums on the matrix pipe)
+// MFMA row m of half u is mapped to key 32*((m>>2)&1) + 16*u + 4*(m>>3) + (m&3),
+// which makes register r of half-wave g hold key 32*g + 16*u + r: 16 consecutive
+// keys -> 16-byte bias loads, and 8 consecutive keys per P.V operand slot group.
+// The triangle bias never touches the vector ALU: its raw bf16 registers are the
+// B operand of an MFMA whose A operand is the constant 0/1 matrix that undoes the
+// key permutation, accumulating straight into S^T.  Per logit the vector ALU
+// executes one fma, one exp2, half a max3 and half a packed bf16 convert.
 // K and V^T tiles are shared by the 4 waves through LDS in fragment order
-// (double-buffered, one barrier per tile); the triangle-bias tile is private to
-// a wave and read straight from global (L2-resident: workgroups are numbered so
-// that one XCD works on one head at a time).
+// (double-buffered, one barrier per tile); the bias tile is private to a wave
+// and read straight from global (L2-resident: workgroups are numbered so that
+// one XCD works on one head at a time).
 //
 // Mask semantics follow the reference's fp32 arithmetic exactly: on tiles that
 // contain a masked (or out-of-range) key the logit is (q.k + inf*(mask-1)) +
-// bias in that order, so -1e9 absorbs small logits and a fully masked row
-// averages v over all keys; tiles whose keys are all unmasked take a shorter
-// path with the bias preloaded into the MFMA accumulator.
+// bias in that order on the vector ALU, so -1e9 absorbs small logits and a fully
+// masked row averages v over all keys; tiles whose keys are all unmasked take
+// the matrix-pipe path above.
 #include "common.h"
 #include "kernels.h"
 
@@ -31,8 +35,8 @@ constexpr int kD = 32;          // head dim
 constexpr int kKeyTile = 64;
 constexpr float kLog2e = 1.4426950408889634f;
 
-template <typename T, int NQ>
-__global__ __launch_bounds__(256) void triattn_fwd_kernel(
+template <typename T>
+__global__ __launch_bounds__(256, 2) void triattn_fwd_kernel(
     const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ vt,
     const T* gate, const T* __restrict__ bias, const T* __restrict__ mask,
     T* o, int n, int heads, int key_pitch, int mask_transposed, float inf,
@@ -40,7 +44,7 @@ __global__ __launch_bounds__(256) void triattn_fwd_kernel(
   typedef typename Vec8<T>::type V8;
   typedef typename Vec4<T>::type V4;
   __shared__ V8 lds_kv[2][8][kWave];     // fragments 0-3: K (u,kk); 4-7: V^T (u,s)
-  __shared__ __attribute__((aligned(16))) float lds_mb[2][kKeyTile];  // additive mask bias of the tile's keys
+  __shared__ __attribute__((aligned(16))) float lds_mb[2][kKeyTile];  // mask bias of the tile's keys
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int ln = lane & 31, g = lane >> 5;
@@ -50,35 +54,45 @@ __global__ __launch_bounds__(256) void triattn_fwd_kernel(
   // (workgroups are dealt round-robin to the 8 XCDs).
   const int64_t per_xcd = (total_items + 7) / 8;
   const int64_t item = (int64_t)(blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-  if ((int64_t)(blockIdx.x >> 3) >= per_xcd || item >= total_items) return;
+  if (item >= total_items) return;
   const int qt = (int)(item % n_qtiles);
   const int i = (int)((item / n_qtiles) % n);
   const int h = (int)(item / ((int64_t)n_qtiles * n));
 
-  const int q0 = (qt * 4 + wave) * (NQ * 32);   // first query of this wave
-  const T* q_row = q + (int64_t)i * n * C + h * kD;
+  const int q0 = (qt * 4 + wave) * 32;   // first query of this wave
   const T* k_row = k + (int64_t)i * n * C + h * kD;
   const T* vt_row = vt + ((int64_t)i * C + h * kD) * key_pitch;
-  const T* bias_h = bias + (int64_t)h * n * key_pitch;
+  // queries beyond n re-read the last one; their results are never stored
+  const int qi = min(q0 + ln, n - 1);
+  const T* bias_q = bias + ((int64_t)h * n + qi) * key_pitch + 32 * g;
 
   // Q fragments (B operand): lane <-> query, slots <-> d = 16*kk + 8*g + t
-  V8 qf[NQ][2];
+  V8 qf[2];
 #pragma unroll
-  for (int qb = 0; qb < NQ; ++qb) {
-    // queries beyond n re-read the last one; their results are never stored
-    const int qi = min(q0 + qb * 32 + ln, n - 1);
+  for (int kk = 0; kk < 2; ++kk)
+    qf[kk] = load8<T>(q + ((int64_t)i * n + qi) * C + h * kD + 16 * kk + 8 * g);
+
+  // Constant operands.  sel[s]: A operand with sel[m][slot (g,t)] = 1 iff key(m) is the key
+  // behind slot (g,t) of step s, i.e. g == (m>>2)&1 and 8s+t == 4*(m>>3) + (m&3).
+  V8 sel[2], ones;
+  {
+    const int g_m = (ln >> 2) & 1, r_m = 4 * (ln >> 3) + (ln & 3);
 #pragma unroll
-    for (int kk = 0; kk < 2; ++kk) qf[qb][kk] = load8<T>(q_row + (int64_t)qi * C + 16 * kk + 8 * g);
+    for (int sgrp = 0; sgrp < 2; ++sgrp)
+#pragma unroll
+      for (int t = 0; t < 8; ++t) sel[sgrp][t] = (T)((g == g_m && 8 * sgrp + t == r_m) ? 1.0f : 0.0f);
+#pragma unroll
+    for (int t = 0; t < 8; ++t) ones[t] = (T)1.0f;
   }
 
   const int n_tiles = (n + kKeyTile - 1) / kKeyTile;
 
   // ---- cooperative tile loader: wave w fetches fragments 2w and 2w+1 ----
-  V8 pre[2];
-  float pre_mb = 0.0f;
   // All loads are unconditional (indices clamped): keys beyond n get a -inf mask
   // bias below, which removes them from the softmax whatever K holds; V^T is zeroed
   // for them because 0 * garbage must stay 0.
+  V8 pre[2];
+  float pre_mb = 0.0f;
   auto fetch = [&](int tile) {
     const int key0 = tile * kKeyTile;
     const bool tail = key0 + kKeyTile > n;   // uniform
@@ -118,30 +132,21 @@ __global__ __launch_bounds__(256) void triattn_fwd_kernel(
     if (wave == 0) lds_mb[buf][lane] = pre_mb;
   };
 
-  // ---- per-wave bias tile loader: lane <-> query, 16 consecutive keys per (qb,u) ----
-  V8 bias_nxt[NQ][2][16 / 8];
+  // ---- per-wave bias tile: lane <-> query, [u][c] = keys key0 + 32g + 16u + 8c .. +7 ----
+  V8 bias_nxt[2][2];
   auto fetch_bias = [&](int tile) {
-    const int key0 = tile * kKeyTile;
+    const T* bp = bias_q + tile * kKeyTile;
 #pragma unroll
-    for (int qb = 0; qb < NQ; ++qb) {
-      const int qi = q0 + qb * 32 + ln;
-      const T* bp = bias_h + (int64_t)(qi < n ? qi : 0) * key_pitch + key0 + 32 * g;
+    for (int u = 0; u < 2; ++u)
 #pragma unroll
-      for (int u = 0; u < 2; ++u)
-#pragma unroll
-        for (int c = 0; c < 2; ++c) bias_nxt[qb][u][c] = load8<T>(bp + 16 * u + 8 * c);
-    }
+      for (int c = 0; c < 2; ++c) bias_nxt[u][c] = load8<T>(bp + 16 * u + 8 * c);
   };
 
-  f32x16 acc_o[NQ];
-  float m_run[NQ], l_run[NQ];
+  f32x16 acc_o, acc_l;   // O^T and (in every register row) the running denominator
 #pragma unroll
-  for (int qb = 0; qb < NQ; ++qb) {
-#pragma unroll
-    for (int r = 0; r < 16; ++r) acc_o[qb][r] = 0.0f;
-    m_run[qb] = -INFINITY;
-    l_run[qb] = 0.0f;
-  }
+  for (int r = 0; r < 16; ++r) { acc_o[r] = 0.0f; acc_l[r] = 0.0f; }
+  float m_run = -INFINITY;        // running max, natural units
+  float nml = 0.0f;               // -m_run * log2(e)
 
   fetch(0);
   fetch_bias(0);
@@ -150,13 +155,11 @@ __global__ __launch_bounds__(256) void triattn_fwd_kernel(
 
   for (int tile = 0; tile < n_tiles; ++tile) {
     const int buf = tile & 1;
-    V8 bias_cur[NQ][2][2];
+    V8 bias_cur[2][2];
 #pragma unroll
-    for (int qb = 0; qb < NQ; ++qb)
+    for (int u = 0; u < 2; ++u)
 #pragma unroll
-      for (int u = 0; u < 2; ++u)
-#pragma unroll
-        for (int c = 0; c < 2; ++c) bias_cur[qb][u][c] = bias_nxt[qb][u][c];
+      for (int c = 0; c < 2; ++c) bias_cur[u][c] = bias_nxt[u][c];
     if (tile + 1 < n_tiles) {
       fetch(tile + 1);
       fetch_bias(tile + 1);
@@ -166,102 +169,90 @@ __global__ __launch_bounds__(256) void triattn_fwd_kernel(
     const float mb_lane = lds_mb[buf][lane];
     const bool masked_tile = __ballot(mb_lane != 0.0f) != 0ull;
 
-    V8 kf[2][2];
+    f32x16 s[2];
 #pragma unroll
-    for (int u = 0; u < 2; ++u)
+    for (int u = 0; u < 2; ++u) {
 #pragma unroll
-      for (int kk = 0; kk < 2; ++kk) kf[u][kk] = lds_kv[buf][u * 2 + kk][lane];
+      for (int r = 0; r < 16; ++r) s[u][r] = 0.0f;
+#pragma unroll
+      for (int kk = 0; kk < 2; ++kk) mma32(s[u], lds_kv[buf][u * 2 + kk][lane], qf[kk]);
+    }
 
-    f32x16 s[NQ][2];
+    V8 pf[2][2];
     if (!masked_tile) {
+      // bias on the matrix pipe: S^T += Sel * Bias
 #pragma unroll
-      for (int qb = 0; qb < NQ; ++qb)
+      for (int u = 0; u < 2; ++u)
 #pragma unroll
-        for (int u = 0; u < 2; ++u) {
+        for (int c = 0; c < 2; ++c) mma32(s[u], sel[c], bias_cur[u][c]);
+      float mx = fmaxf(s[0][0], s[1][0]);
 #pragma unroll
-          for (int c = 0; c < 2; ++c) {
-            const f32x8 b = to_f32(bias_cur[qb][u][c]);
+      for (int r = 1; r < 16; ++r) mx = fmaxf(mx, fmaxf(s[0][r], s[1][r]));
+      mx = fmaxf(mx, swap32(mx));
+      if (__any(mx > m_run)) {
+        const float m_new = fmaxf(m_run, mx);
+        const float alpha = fast_exp2((m_run - m_new) * kLog2e);
+        m_run = m_new;
+        nml = -m_new * kLog2e;
 #pragma unroll
-            for (int t = 0; t < 8; ++t) s[qb][u][8 * c + t] = b[t];
-          }
+        for (int r = 0; r < 16; ++r) acc_o[r] *= alpha;
+        acc_l[0] *= alpha;
+      }
 #pragma unroll
-          for (int kk = 0; kk < 2; ++kk) mma32(s[qb][u], kf[u][kk], qf[qb][kk]);
+      for (int u = 0; u < 2; ++u)
+#pragma unroll
+        for (int c = 0; c < 2; ++c) {
+          f32x8 p8;
+#pragma unroll
+          for (int t = 0; t < 8; ++t) p8[t] = fast_exp2(fmaf(s[u][8 * c + t], kLog2e, nml));
+          pf[u][c] = from_f32<T>(p8);
         }
     } else {
       // exact reference order in fp32: (q.k + mask_bias) + triangle_bias
-      float mb[2][16];
 #pragma unroll
       for (int u = 0; u < 2; ++u)
 #pragma unroll
-        for (int c = 0; c < 4; ++c) {
-          const f32x4 m4 = *reinterpret_cast<const f32x4*>(&lds_mb[buf][32 * g + 16 * u + 4 * c]);
+        for (int c = 0; c < 2; ++c) {
+          const f32x8 b = to_f32(bias_cur[u][c]);
+          const f32x4 m0 = *reinterpret_cast<const f32x4*>(&lds_mb[buf][32 * g + 16 * u + 8 * c]);
+          const f32x4 m1 = *reinterpret_cast<const f32x4*>(&lds_mb[buf][32 * g + 16 * u + 8 * c + 4]);
 #pragma unroll
-          for (int t = 0; t < 4; ++t) mb[u][4 * c + t] = m4[t];
-        }
-#pragma unroll
-      for (int qb = 0; qb < NQ; ++qb)
-#pragma unroll
-        for (int u = 0; u < 2; ++u) {
-#pragma unroll
-          for (int r = 0; r < 16; ++r) s[qb][u][r] = 0.0f;
-#pragma unroll
-          for (int kk = 0; kk < 2; ++kk) mma32(s[qb][u], kf[u][kk], qf[qb][kk]);
-#pragma unroll
-          for (int c = 0; c < 2; ++c) {
-            const f32x8 b = to_f32(bias_cur[qb][u][c]);
-#pragma unroll
-            for (int t = 0; t < 8; ++t) {
-              const int r = 8 * c + t;
-              const float v = (s[qb][u][r] + mb[u][r]) + b[t];
-              s[qb][u][r] = mb[u][r] == -INFINITY ? -INFINITY : v;   // key beyond n
-            }
+          for (int t = 0; t < 8; ++t) {
+            const float mbv = t < 4 ? m0[t & 3] : m1[t & 3];
+            const float v = (s[u][8 * c + t] + mbv) + b[t];
+            s[u][8 * c + t] = mbv == -INFINITY ? -INFINITY : v;   // key beyond n
           }
         }
-    }
-
-    // ---- online softmax over this tile's 64 keys, per query (= per lane pair) ----
-    V8 pf[NQ][2][2];
+      float mx = fmaxf(s[0][0], s[1][0]);
 #pragma unroll
-    for (int qb = 0; qb < NQ; ++qb) {
-      float mx = s[qb][0][0];
+      for (int r = 1; r < 16; ++r) mx = fmaxf(mx, fmaxf(s[0][r], s[1][r]));
+      mx = fmaxf(mx, swap32(mx));
+      const float m_new = fmaxf(m_run, mx);          // finite: key0 < n is never excluded
+      const float alpha = fast_exp2((m_run - m_new) * kLog2e);
+      m_run = m_new;
+      nml = -m_new * kLog2e;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc_o[r] *= alpha;
+      acc_l[0] *= alpha;
 #pragma unroll
       for (int u = 0; u < 2; ++u)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[qb][u][r]);
-      mx = fmaxf(mx, swap32(mx));
-      const float m_new = fmaxf(m_run[qb], mx);          // finite: key0 < n is never excluded
-      const float alpha = fast_exp2((m_run[qb] - m_new) * kLog2e);
-      m_run[qb] = m_new;
-      float psum = 0.0f;
-#pragma unroll
-      for (int u = 0; u < 2; ++u) {
-        f32x16 p;
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          p[r] = fast_exp2((s[qb][u][r] - m_new) * kLog2e);
-          psum += p[r];
-        }
-#pragma unroll
-        for (int sgrp = 0; sgrp < 2; ++sgrp) {
+        for (int c = 0; c < 2; ++c) {
           f32x8 p8;
+          // (s - m) first: exact when both sit near -1e9
 #pragma unroll
-          for (int t = 0; t < 8; ++t) p8[t] = p[8 * sgrp + t];
-          pf[qb][u][sgrp] = from_f32<T>(p8);
+          for (int t = 0; t < 8; ++t) p8[t] = fast_exp2((s[u][8 * c + t] - m_new) * kLog2e);
+          pf[u][c] = from_f32<T>(p8);
         }
-      }
-      l_run[qb] = l_run[qb] * alpha + psum;
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc_o[qb][r] *= alpha;
     }
 
-    // ---- O^T += V^T P^T ----
+    // ---- O^T += V^T P^T ; l += 1^T P^T ----
 #pragma unroll
     for (int u = 0; u < 2; ++u)
 #pragma unroll
-      for (int sgrp = 0; sgrp < 2; ++sgrp) {
-        const V8 vf = lds_kv[buf][4 + u * 2 + sgrp][lane];
-#pragma unroll
-        for (int qb = 0; qb < NQ; ++qb) mma32(acc_o[qb], vf, pf[qb][u][sgrp]);
+      for (int c = 0; c < 2; ++c) {
+        mma32(acc_o, lds_kv[buf][4 + u * 2 + c][lane], pf[u][c]);
+        mma32(acc_l, ones, pf[u][c]);
       }
 
     if (tile + 1 < n_tiles) stash(buf ^ 1);
@@ -270,31 +261,21 @@ __global__ __launch_bounds__(256) void triattn_fwd_kernel(
 
   // ---- normalise, gate, store: lane <-> query, register r <-> d = acc_row(r, g) ----
   // o may alias gate: every gate load is issued before the first store.
-  f32x4 gv[NQ][4];
+  const int64_t base = ((int64_t)i * n + qi) * C + h * kD + 4 * g;
+  f32x4 gv[4];
 #pragma unroll
-  for (int qb = 0; qb < NQ; ++qb) {
-    const int qi = q0 + qb * 32 + ln;
-    const int64_t base = ((int64_t)i * n + (qi < n ? qi : 0)) * C + h * kD + 4 * g;
+  for (int c = 0; c < 4; ++c) gv[c] = to_f32(*reinterpret_cast<const V4*>(gate + base + 8 * c));
+  const float inv = 1.0f / acc_l[0];
+  if (q0 + ln < n) {
 #pragma unroll
-    for (int c = 0; c < 4; ++c) gv[qb][c] = to_f32(*reinterpret_cast<const V4*>(gate + base + 8 * c));
-  }
+    for (int c = 0; c < 4; ++c) {
+      f32x4 ov;
 #pragma unroll
-  for (int qb = 0; qb < NQ; ++qb) {
-    const int qi = q0 + qb * 32 + ln;
-    const float l_tot = l_run[qb] + swap32(l_run[qb]);
-    const float inv = 1.0f / l_tot;
-    if (qi < n) {
-      const int64_t base = ((int64_t)i * n + qi) * C + h * kD + 4 * g;
-#pragma unroll
-      for (int c = 0; c < 4; ++c) {
-        f32x4 ov;
-#pragma unroll
-        for (int t = 0; t < 4; ++t) {
-          // attention output rounded to T before the gate multiply, as the reference does
-          ov[t] = to_f32(from_f32<T>(acc_o[qb][4 * c + t] * inv)) * gv[qb][c][t];
-        }
-        *reinterpret_cast<V4*>(o + base + 8 * c) = from_f32<T>(ov);
+      for (int t = 0; t < 4; ++t) {
+        // attention output rounded to T before the gate multiply, as the reference does
+        ov[t] = to_f32(from_f32<T>(acc_o[4 * c + t] * inv)) * gv[c][t];
       }
+      *reinterpret_cast<V4*>(o + base + 8 * c) = from_f32<T>(ov);
     }
   }
 }
@@ -304,25 +285,11 @@ int triattn_fwd(const T* q, const T* k, const T* vt, const T* g, const T* tri_bi
                 T* o, int n, int heads, int key_pitch, int mask_transposed, float inf,
                 hipStream_t stream) {
   if (n == 0) return 0;
-  // fp32 fragments are twice as wide: one query block per wave keeps registers in check;
-  // bf16 uses two when the query count fills them.
-  const bool two = sizeof(T) == 2 && n >= 256;
-  const int q_per_wg = 4 * 32 * (two ? 2 : 1);
-  const int n_qtiles = (n + q_per_wg - 1) / q_per_wg;
+  const int n_qtiles = (n + 127) / 128;
   const int64_t total = (int64_t)heads * n * n_qtiles;
   const int64_t per_xcd = (total + 7) / 8;
-  const dim3 grid((unsigned)(per_xcd * 8)), block(256);
-  if constexpr (sizeof(T) == 2) {
-    if (two) {
-      triattn_fwd_kernel<T, 2><<<grid, block, 0, stream>>>(q, k, vt, g, tri_bias, mask, o, n, heads,
-                                                           key_pitch, mask_transposed, inf,
-                                                           n_qtiles, total);
-      return 0;
-    }
-  }
-  triattn_fwd_kernel<T, 1><<<grid, block, 0, stream>>>(q, k, vt, g, tri_bias, mask, o, n, heads,
-                                                       key_pitch, mask_transposed, inf, n_qtiles,
-                                                       total);
+  triattn_fwd_kernel<T><<<dim3((unsigned)(per_xcd * 8)), dim3(256), 0, stream>>>(
+      q, k, vt, g, tri_bias, mask, o, n, heads, key_pitch, mask_transposed, inf, n_qtiles, total);
   return 0;
 }
 
