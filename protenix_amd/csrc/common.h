@@ -108,4 +108,40 @@ struct RowMap {
   }
 };
 
+// ---------------------------------------------------------------------------
+// Operand layouts of the triangle-attention core (written by the projection
+// kernel, read by the attention kernel).  Keys are grouped in tiles of 64; one
+// operand tile is stored in MFMA fragment order, 4 fragments x 64 lanes x 8
+// elements, so that every fragment load of the attention kernel is one fully
+// contiguous 1 KB (bf16) read.  Within a key tile, key jj = 32*g + 16*u + r:
+//   K   fragment (u, kk): lane 32*gl + m holds d = 16*kk + 8*gl .. +7 of the key
+//       whose MFMA row is m = 8*(r>>2) + 4*g + (r&3)
+//   V^T fragment (u, s):  lane 32*g + d holds keys 32*g + 16*u + 8*s .. +7 of channel d
+//   bias fragment (u, c): lane 32*g + q holds keys 32*g + 16*u + 8*c .. +7 of query q
+//       (queries in blocks of 32)
+// q, the gate and the output are head-major: [head][i][j][32].
+// ---------------------------------------------------------------------------
+constexpr int kAttnTileElems = 2048;   // 4 fragments x 64 lanes x 8
+
+__host__ __device__ __forceinline__ int64_t attn_k_offset(int h, int i, int j, int d, int n,
+                                                          int key_tiles) {
+  const int jj = j & 63, g = jj >> 5, u = (jj >> 4) & 1, r = jj & 15;
+  const int m = 8 * (r >> 2) + 4 * g + (r & 3);
+  const int c8 = d >> 3, kk = c8 >> 1, gl = c8 & 1;
+  return ((((int64_t)h * n + i) * key_tiles + (j >> 6)) * 4 + (u * 2 + kk)) * 512 +
+         (32 * gl + m) * 8 + (d & 7);
+}
+__host__ __device__ __forceinline__ int64_t attn_v_offset(int h, int i, int j, int d, int n,
+                                                          int key_tiles) {
+  const int jj = j & 63, g = jj >> 5, u = (jj >> 4) & 1, sg = (jj >> 3) & 1;
+  return ((((int64_t)h * n + i) * key_tiles + (j >> 6)) * 4 + (u * 2 + sg)) * 512 +
+         (32 * g + d) * 8 + (j & 7);
+}
+__host__ __device__ __forceinline__ int64_t attn_b_offset(int h, int q, int j, int q_blocks,
+                                                          int key_tiles) {
+  const int jj = j & 63, g = jj >> 5, u = (jj >> 4) & 1, c = (jj >> 3) & 1;
+  return ((((int64_t)h * q_blocks + (q >> 5)) * key_tiles + (j >> 6)) * 4 + (u * 2 + c)) * 512 +
+         (32 * g + (q & 31)) * 8 + (j & 7);
+}
+
 }  // namespace ptx

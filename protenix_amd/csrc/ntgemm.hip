@@ -105,7 +105,7 @@ __global__ __launch_bounds__(256) void nt_gemm_batched_kernel(const T* __restric
     for (int rb = 0; rb < 2; ++rb)
 #pragma unroll
       for (int kk = 0; kk < KK; ++kk) a_cur[rb][kk] = a_nxt[rb][kk];
-    if (stage + 1 < n_stages) fetch(stage + 1);
+    fetch(min(stage + 1, n_stages - 1));   // unconditional: static outstanding-load count
 
 #pragma unroll
     for (int kk = 0; kk < KK; ++kk) {
@@ -116,7 +116,7 @@ __global__ __launch_bounds__(256) void nt_gemm_batched_kernel(const T* __restric
         for (int rb = 0; rb < 2; ++rb) mma32(acc[rb][jb], a_cur[rb][kk], bf);
       }
     }
-    if (stage + 1 < n_stages) stash(buf ^ 1);
+    stash(buf ^ 1);
     __syncthreads();
   }
 

@@ -417,7 +417,7 @@ __global__ __launch_bounds__(256) void rowgemm_in_kernel(RowGemmInParams p) {
 
   for (int ch = 0; ch < nch; ++ch) {
     const int buf = C::NBUF == 2 ? (ch & 1) : 0;
-    if (ch + 1 < nch) fetch(ch + 1);
+    fetch(min(ch + 1, nch - 1));   // unconditional: keeps the outstanding-load count static
 
     // Orientation: channel-major outputs want lane <-> channel (x as A operand).
     bool chan_on_lanes;
@@ -487,10 +487,12 @@ __global__ __launch_bounds__(256) void rowgemm_in_kernel(RowGemmInParams p) {
         store_channel_major(outp, (int64_t)p.n * p.pitch, p.pitch, c0, kC, rb);
       }
     } else if constexpr (MODE == kTriAttnIn) {
+      // Outputs in the attention core's layouts (common.h): q and the gate head-major
+      // [h][p][32], K / V^T / bias in fragment-ordered key tiles.
       const int which = ch >> 1;
-      if (which < 3) {
-        // q (rounded, then scaled), k, sigmoid(g): row-major [p][128]
-        T* outp = (T*)p.out[which];
+      const int key_tiles = p.pitch >> 6;
+      if (which == 0 || which == 2) {
+        // q (rounded, then scaled) and sigmoid(g): one 32 x 32 tile = one head
 #pragma unroll
         for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
@@ -500,17 +502,19 @@ __global__ __launch_bounds__(256) void rowgemm_in_kernel(RowGemmInParams p) {
             for (int r = 0; r < 16; ++r) {
               float v = acc[rb][t][r];
               if (which == 0) v = to_f32(from_f32<T>(v)) * p.q_scale;
-              if (which == 2) v = sigmoidf_fast(v);
+              else v = sigmoidf_fast(v);
               vals[r] = v;
             }
             wave_lds_sync();
             stage_put<T>(st, vals, lane);
             wave_lds_sync();
-            store_row_major(outp, kC, ((ch & 1) * 2 + t) * 32, rb, nullptr);
+            const int h = (ch & 1) * 2 + t;
+            store_row_major((T*)p.out[which] + (int64_t)h * p.n_rows * 32, 32, 0, rb, nullptr);
           }
-      } else if (which == 3) {
-        // v^T[i][c][key]: lane <-> channel, register <-> row p = i*n + key.  Channel c of
-        // row i starts at i*128*pitch + c*pitch: planes `pitch` apart, plane rows 128*pitch.
+      } else if (which == 1) {
+        // K: staged row-major (major = key row, minor = d); each 16-byte d-chunk goes to
+        // its fragment slot
+        T* outp = (T*)p.out[1];
 #pragma unroll
         for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
@@ -521,21 +525,64 @@ __global__ __launch_bounds__(256) void rowgemm_in_kernel(RowGemmInParams p) {
             wave_lds_sync();
             stage_put<T>(st, vals, lane);
             wave_lds_sync();
-            store_channel_major((T*)p.out[3], (int64_t)p.pitch, (int64_t)p.pitch * kC,
-                                ((ch & 1) * 2 + t) * 32, kC, rb);
+            const int h = (ch & 1) * 2 + t;
+#pragma unroll
+            for (int ps = 0; ps < C::NPASS; ++ps) {
+              int mj, m0;
+              stage_coord<T>(ps, lane, mj, m0);
+              if (rrow[rb][ps] >= 0) {
+                const uint32_t pr = (uint32_t)rrow[rb][ps];
+                const uint32_t i = pr / (uint32_t)p.n, j = pr - i * (uint32_t)p.n;
+                *reinterpret_cast<VE_t*>(outp + attn_k_offset(h, i, j, m0, p.n, key_tiles)) =
+                    stage_get_vec<T>(st, mj, m0);
+              }
+            }
           }
       } else {
-        // triangle bias [h][i][pitch]
+        // V^T (which == 3, major = channel d of head h) and the triangle bias (which == 4,
+        // major = head, logical row = (query i, key j)): vectors of VE consecutive keys
+        const int q_blocks = (p.n + 31) >> 5;
 #pragma unroll
-        for (int rb = 0; rb < RB; ++rb) {
-          float vals[16];
+        for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
-          for (int r = 0; r < 16; ++r) vals[r] = acc[rb][0][r];
-          wave_lds_sync();
-          stage_put<T>(st, vals, lane);
-          wave_lds_sync();
-          store_channel_major((T*)p.out[4], (int64_t)p.n * p.pitch, p.pitch, 0, p.aux, rb);
-        }
+          for (int t = 0; t < 2; ++t) {
+            if (which == 4 && t == 1) continue;
+            float vals[16];
+#pragma unroll
+            for (int r = 0; r < 16; ++r) vals[r] = acc[rb][t][r];
+            wave_lds_sync();
+            stage_put<T>(st, vals, lane);
+            wave_lds_sync();
+            const int h = (ch & 1) * 2 + t;
+#pragma unroll
+            for (int ps = 0; ps < C::NPASS; ++ps) {
+              int chn, r0;
+              stage_coord<T>(ps, lane, chn, r0);
+              const int64_t pr = row0 + rb * 32 + r0;
+              if (which == 4 && chn >= p.aux) continue;
+              const VE_t v = stage_get_vec<T>(st, chn, r0);
+              T* outp = (T*)p.out[which];
+              if (vec_ok) {
+                if (pr < p.n_rows) {
+                  const uint32_t i = (uint32_t)pr / (uint32_t)p.n, j = (uint32_t)pr - i * (uint32_t)p.n;
+                  const int64_t off = which == 3 ? attn_v_offset(h, i, j, chn, p.n, key_tiles)
+                                                 : attn_b_offset(chn, i, j, q_blocks, key_tiles);
+                  *reinterpret_cast<VE_t*>(outp + off) = v;
+                }
+              } else {
+#pragma unroll
+                for (int e = 0; e < C::VE; ++e) {
+                  if (pr + e < p.n_rows) {
+                    const uint32_t pe = (uint32_t)(pr + e);
+                    const uint32_t i = pe / (uint32_t)p.n, j = pe - i * (uint32_t)p.n;
+                    const int64_t off = which == 3 ? attn_v_offset(h, i, j, chn, p.n, key_tiles)
+                                                   : attn_b_offset(chn, i, j, q_blocks, key_tiles);
+                    outp[off] = v[e];
+                  }
+                }
+              }
+            }
+          }
       }
     } else if constexpr (MODE == kTransitionIn) {
       // hidden[p][col] = silu(a) * b, row-major with leading dimension 128 * n_factor
@@ -605,7 +652,7 @@ __global__ __launch_bounds__(256) void rowgemm_in_kernel(RowGemmInParams p) {
     }
 
     if (C::NBUF == 1) __syncthreads();      // everyone is done reading the single buffer
-    if (ch + 1 < nch) stash(C::NBUF == 2 ? (buf ^ 1) : 0);
+    stash(C::NBUF == 2 ? (buf ^ 1) : 0);
     __syncthreads();
   }
 }
@@ -627,6 +674,7 @@ int launch_rowgemm_in(const RowGemmInParams& p, hipStream_t stream) {
 // ---------------------------------------------------------------------------
 struct RowGemmOutParams {
   const void* a;
+  int a_head_major;     // A is [4][n_rows][32] (attention output) instead of [n_rows][K]
   int n_slab;
   const void* w;        // [128][128*n_slab]
   const void* res;      // residual source (same addressing as out) or null
@@ -678,13 +726,27 @@ __global__ __launch_bounds__(256) void rowgemm_out_kernel(RowGemmOutParams p) {
   const int nch = 2 * p.n_slab;
   for (int slab = 0; slab < p.n_slab; ++slab) {
     RowFrags<T, RB> af;
-    load_rows<T, RB, false>(af, (const T*)p.a + slab * kC, amap, row0, p.n_rows, nullptr, nullptr,
-                            0.0f, lane);
+    if (p.a_head_major) {
+      // channel 16*kk + 8*g + t = head kk/2, d = 16*(kk%2) + 8*g + t
+      const int ln_ = lane & 31, g_ = lane >> 5;
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb) {
+        int64_t pr = row0 + rb * 32 + ln_;
+        pr = pr < p.n_rows ? pr : p.n_rows - 1;
+#pragma unroll
+        for (int kk = 0; kk < kKSteps; ++kk)
+          af.f[rb][kk] = load8<T>((const T*)p.a + ((int64_t)(kk >> 1) * p.n_rows + pr) * 32 +
+                                  16 * (kk & 1) + 8 * g_);
+      }
+    } else {
+      load_rows<T, RB, false>(af, (const T*)p.a + slab * kC, amap, row0, p.n_rows, nullptr,
+                              nullptr, 0.0f, lane);
+    }
 #pragma unroll
     for (int half = 0; half < 2; ++half) {
       const int ch = 2 * slab + half;
       const int buf = C::NBUF == 2 ? half : 0;
-      if (ch + 1 < nch) fetch(ch + 1);
+      fetch(min(ch + 1, nch - 1));
 #pragma unroll
       for (int kk = 0; kk < kKSteps; ++kk) {
         const V8 w0 = lds_w[buf][kk][lane];
@@ -697,7 +759,7 @@ __global__ __launch_bounds__(256) void rowgemm_out_kernel(RowGemmOutParams p) {
         }
       }
       if (C::NBUF == 1) __syncthreads();
-      if (ch + 1 < nch) stash(C::NBUF == 2 ? (buf ^ 1) : 0);
+      stash(C::NBUF == 2 ? (buf ^ 1) : 0);
       __syncthreads();
     }
   }
@@ -826,6 +888,7 @@ int triattn_output(const void* o, const void* w_o, const void* z, void* out, int
                    int add_residual, hipStream_t stream) {
   RowGemmOutParams p = {};
   p.a = o;
+  p.a_head_major = 1;
   p.n_slab = 1;
   p.w = w_o;
   p.res = add_residual ? z : nullptr;

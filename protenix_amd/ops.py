@@ -139,21 +139,23 @@ def triangle_attention(z: torch.Tensor, mask: Optional[torch.Tensor], w: dict, h
     dt, st = _dt(z), _stream()
     pitch = key_pitch(n)
     mask = _mask_for(mask, z)
-    hd = heads * d
     dev = z.device
-    q = torch.empty((n, n, hd), dtype=z.dtype, device=dev)
-    k = torch.empty((n, n, hd), dtype=z.dtype, device=dev)
-    g = torch.empty((n, n, hd), dtype=z.dtype, device=dev)
-    vt = torch.empty((n, hd, pitch), dtype=z.dtype, device=dev)
-    tb = torch.empty((heads, n, pitch), dtype=z.dtype, device=dev)
+    kt, qb = pitch // 64, (n + 31) // 32
+    # attention-core layouts (csrc/common.h): q, gate, output head-major; K, V^T and the
+    # triangle bias in fragment-ordered key tiles of 2048 elements
+    q = torch.empty((heads, n, n, d), dtype=z.dtype, device=dev)
+    g = torch.empty((heads, n, n, d), dtype=z.dtype, device=dev)
+    k = torch.empty((heads, n, kt, 2048), dtype=z.dtype, device=dev)
+    vt = torch.empty((heads, n, kt, 2048), dtype=z.dtype, device=dev)
+    tb = torch.empty((heads, qb, kt, 2048), dtype=z.dtype, device=dev)
     with torch.cuda.device(dev):
-        _call("triattn_project", lib.ptx_triattn_project, _ptr(z), _ptr(w["ln_w"]), _ptr(w["ln_b"]), _ptr(w["w_q"]), _ptr(w["w_k"]), _ptr(w["w_v"]),
-            _ptr(w["w_g"]), _ptr(w["w_b"]), _ptr(q), _ptr(k), _ptr(vt), _ptr(g), _ptr(tb), n, c,
-            heads, d, pitch, int(transposed), eps, dt, st)
+        _call("triattn_project", lib.ptx_triattn_project, _ptr(z), _ptr(w["ln_w"]),
+              _ptr(w["ln_b"]), _ptr(w["w_q"]), _ptr(w["w_k"]), _ptr(w["w_v"]), _ptr(w["w_g"]),
+              _ptr(w["w_b"]), _ptr(q), _ptr(k), _ptr(vt), _ptr(g), _ptr(tb), n, c, heads, d, pitch,
+              int(transposed), eps, dt, st)
         # o overwrites g: each element of g is read once, by the thread that then writes o there
-        _call("triattn_fwd", lib.ptx_triattn_fwd, _ptr(q), _ptr(k), _ptr(vt), _ptr(g), _ptr(tb), _ptr(mask),
-                                       _ptr(g), n, heads, d, pitch, int(transposed), float(inf), dt,
-                                       st)
+        _call("triattn_fwd", lib.ptx_triattn_fwd, _ptr(q), _ptr(k), _ptr(vt), _ptr(g), _ptr(tb),
+              _ptr(mask), _ptr(g), n, heads, d, pitch, int(transposed), float(inf), dt, st)
         del q, k, vt, tb
         if out is None:
             out = torch.empty_like(z)
