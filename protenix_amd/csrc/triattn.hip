@@ -25,6 +25,8 @@
 // bias in that order on the vector ALU, so -1e9 absorbs small logits and a fully
 // masked row averages v over all keys; tiles whose keys are all unmasked take
 // the matrix-pipe path above.
+#include <type_traits>
+
 #include "common.h"
 #include "kernels.h"
 
@@ -34,51 +36,60 @@ constexpr int kD = 32;          // head dim
 constexpr int kKeyTile = 64;
 constexpr float kLog2e = 1.4426950408889634f;
 
-template <typename T>
+// Rows of the pair tensor handled by one wave (the bias tile is then loaded once per key
+// tile and reused).  More than one row does not fit the register budget of 2 waves/SIMD.
+#ifndef PTX_ATTN_ROWS
+#define PTX_ATTN_ROWS 1
+#endif
+
+template <typename T, int R>
 __global__ __launch_bounds__(256, 2) void triattn_fwd_kernel(
     const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ vt,
     const T* gate, const T* __restrict__ bias, const T* __restrict__ mask,
     T* o, int n, int heads, int key_pitch, int mask_transposed, float inf,
-    int n_qtiles, int64_t total_items) {
+    int n_qtiles, int n_rowgroups, int64_t total_items) {
   typedef typename Vec8<T>::type V8;
   typedef typename Vec4<T>::type V4;
-  // ring of 3 key tiles: iteration t reads V^T(t) and K(t+1) while tile t+2 is written
-  __shared__ V8 lds_kv[3][8][kWave];     // fragments 0-3: K (u,kk); 4-7: V^T (u,s)
-  __shared__ __attribute__((aligned(16))) float lds_mb[3][kKeyTile];  // mask bias of the tile's keys
+  // ring of 3 key tiles x R rows: iteration t reads tile t while tile t+2 is written
+  __shared__ V8 lds_kv[3][R][8][kWave];     // fragments 0-3: K (u,kk); 4-7: V^T (u,s)
+  __shared__ __attribute__((aligned(16))) float lds_mb[3][R][kKeyTile];  // mask bias per key
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int ln = lane & 31, g = lane >> 5;
 
-  // Work item -> (h, i, query tile), h-major, one contiguous span per XCD
+  // Work item -> (h, row group, query tile), h-major, one contiguous span per XCD
   // (workgroups are dealt round-robin to the 8 XCDs).
   const int64_t per_xcd = (total_items + 7) / 8;
   const int64_t item = (int64_t)(blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
   if (item >= total_items) return;
   const int qt = (int)(item % n_qtiles);
-  const int i = (int)((item / n_qtiles) % n);
-  const int h = (int)(item / ((int64_t)n_qtiles * n));
+  const int i0 = (int)((item / n_qtiles) % n_rowgroups) * R;   // first of this workgroup's R rows
+  const int h = (int)(item / ((int64_t)n_qtiles * n_rowgroups));
 
   const int q0 = (qt * 4 + wave) * 32;   // first query of this wave
   const int key_tiles = key_pitch >> 6;
   const int q_blocks = (n + 31) >> 5;
-  // operand tiles in fragment order (common.h): 2048 elements per key tile, this lane's
-  // 8 elements of fragment f at f*512 + lane*8
-  const T* k_tiles = k + ((int64_t)h * n + i) * key_tiles * kAttnTileElems + lane * 8;
-  const T* v_tiles = vt + ((int64_t)h * n + i) * key_tiles * kAttnTileElems + lane * 8;
-  // (a wave whose queries all lie beyond n re-reads the last block; nothing of it is stored)
+  const int n_tiles = (n + kKeyTile - 1) / kKeyTile;
+  const bool has_mask = mask != nullptr;
+  const T* mask_or_dummy = has_mask ? mask : q;   // any valid address: the value is discarded
+  // Operand tiles in fragment order (common.h): 2048 elements per key tile, this lane's
+  // 8 elements of fragment f at f*512 + lane*8.  Rows beyond n re-read row n-1, a wave whose
+  // queries all lie beyond n re-reads the last query block; nothing of either is stored.
   const T* b_tiles = bias + ((int64_t)h * q_blocks + min(q0 >> 5, q_blocks - 1)) * key_tiles * kAttnTileElems + lane * 8;
-  // queries beyond n re-read the last one; their results are never stored
   const int qi = min(q0 + ln, n - 1);
-  const int64_t qrow = (((int64_t)h * n + i) * n + qi) * kD;   // head-major q / gate / o row
 
   // Q fragments (B operand): lane <-> query, slots <-> d = 16*kk + 8*g + t
-  V8 qf[2];
+  V8 qf[R][2];
+  int64_t qrow[R];                       // head-major q / gate / o row of this lane's query
 #pragma unroll
-  for (int kk = 0; kk < 2; ++kk)
-    qf[kk] = load8<T>(q + qrow + 16 * kk + 8 * g);
+  for (int r = 0; r < R; ++r) {
+    qrow[r] = (((int64_t)h * n + min(i0 + r, n - 1)) * n + qi) * kD;
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk) qf[r][kk] = load8<T>(q + qrow[r] + 16 * kk + 8 * g);
+  }
 
-  // Constant operands.  sel[s]: A operand with sel[m][slot (g,t)] = 1 iff key(m) is the key
-  // behind slot (g,t) of step s, i.e. g == (m>>2)&1 and 8s+t == 4*(m>>3) + (m&3).
+  // Constant operand sel[s]: A matrix with sel[m][slot (g,t)] = 1 iff key(m) is the key behind
+  // slot (g,t) of step s, i.e. g == (m>>2)&1 and 8s+t == 4*(m>>3) + (m&3).
   V8 sel[2];
   {
     const int g_m = (ln >> 2) & 1, r_m = 4 * (ln >> 3) + (ln & 3);
@@ -88,57 +99,53 @@ __global__ __launch_bounds__(256, 2) void triattn_fwd_kernel(
       for (int t = 0; t < 8; ++t) sel[sgrp][t] = (T)((g == g_m && 8 * sgrp + t == r_m) ? 1.0f : 0.0f);
   }
 
-  const int n_tiles = (n + kKeyTile - 1) / kKeyTile;
-  const bool has_mask = mask != nullptr;
-  const T* mask_or_dummy = has_mask ? mask : q;   // any valid address: the value is discarded
-
-  // ---- cooperative tile loader: wave w fetches fragments 2w and 2w+1 ----
-  // All loads are unconditional (indices clamped): keys beyond n get a -inf mask
-  // bias below, which removes them from the softmax whatever K holds; V^T is zeroed
-  // for them because 0 * garbage must stay 0.
-  V8 pre[2];
-  float pre_mb = 0.0f;
+  // ---- cooperative tile loader: 8*R fragments per key tile, 2*R per wave ----
+  // `tile` may run past the last tile: the pipeline below never branches around a load, so
+  // that the compiler can count the outstanding loads exactly.  Addresses use the clamped
+  // tile; the mask bias and the V^T zeroing use the real key index, which makes a phantom
+  // tile contribute exactly nothing.  Keys beyond n hold garbage in K (removed by the -inf
+  // mask bias) and are zeroed in V^T (0 * garbage must stay 0).
+  // fetch() only issues loads; everything that consumes a loaded value (mask -> additive
+  // bias, zeroing of V^T beyond n) happens in stash(), one tile of work later, so no wait
+  // for memory sits in the issue path.
+  V8 pre[2 * R];
+  T pre_mv;
   auto fetch = [&](int tile) {
-    // `tile` may run past the last tile (the pipeline below never branches around a load, so
-    // that the compiler can count outstanding loads exactly): addresses use the clamped tile,
-    // the mask bias and the V^T zeroing use the real key index, which makes a phantom tile
-    // contribute exactly nothing.
+    const int64_t atile = min(tile, n_tiles - 1);
+#pragma unroll
+    for (int j = 0; j < 2 * R; ++j) {
+      const int fid = wave * 2 * R + j;            // row = fid / 8, fragment = fid % 8
+      const int r = fid >> 3, f = fid & 7;
+      const int64_t rowtiles = ((int64_t)h * n + min(i0 + r, n - 1)) * key_tiles + atile;
+      pre[j] = load8<T>((f < 4 ? k : vt) + rowtiles * kAttnTileElems + (f & 3) * 512 + lane * 8);
+    }
+    // wave w < R publishes the mask bias of row i0 + w; all waves load (uniform load count)
+    const int kc = min(tile * kKeyTile + lane, n - 1);
+    const int row = min(i0 + min(wave, R - 1), n - 1);
+    const int64_t mi = mask_transposed ? (int64_t)kc * n + row : (int64_t)row * n + kc;
+    pre_mv = mask_or_dummy[has_mask ? mi : 0];
+  };
+  auto stash = [&](int tile) {
+    const int buf = tile % 3;
     const int key0 = tile * kKeyTile;
-    const int akey0 = min(tile, n_tiles - 1) * kKeyTile;
     const bool tail = key0 + kKeyTile > n;   // uniform
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const int fid = wave * 2 + j;
-      const int u = (fid >> 1) & 1, sub = fid & 1;
-      if (fid < 4) {
-        // K (A operand): MFMA row m <-> key 32*((m>>2)&1) + 16u + 4*(m>>3) + (m&3); slots <-> d.
-        // Keys beyond n hold garbage; the -inf mask bias removes them.
-        pre[j] = load8<T>(k_tiles + (int64_t)(akey0 >> 6) * kAttnTileElems + fid * 512);
-      } else {
-        // V^T (A operand): MFMA row <-> d = ln; slots <-> keys 32g + 16u + 8s + t
-        const int koff = 32 * g + 16 * u + 8 * sub;
-        V8 v = load8<T>(v_tiles + (int64_t)(akey0 >> 6) * kAttnTileElems + (fid - 4) * 512);
-        if (tail) {
+    for (int j = 0; j < 2 * R; ++j) {
+      const int fid = wave * 2 * R + j;
+      const int f = fid & 7;
+      V8 v = pre[j];
+      if (tail && f >= 4) {
+        // V^T fragment (u, s): slots <-> keys 32g + 16u + 8s + t
+        const int koff = key0 + 32 * g + 16 * ((f >> 1) & 1) + 8 * (f & 1);
 #pragma unroll
-          for (int t = 0; t < 8; ++t) v[t] = key0 + koff + t < n ? v[t] : (T)0.0f;
-        }
-        pre[j] = v;
+        for (int t = 0; t < 8; ++t) v[t] = koff + t < n ? v[t] : (T)0.0f;
       }
+      lds_kv[buf][fid >> 3][f][lane] = v;
     }
-    {
-      // every wave loads (keeps the load count uniform); wave 0 publishes it
-      const int key = key0 + lane;
-      const int kc = min(key, n - 1);
-      const int64_t mi = mask_transposed ? (int64_t)kc * n + i : (int64_t)i * n + kc;
-      const float mv = to_f32(mask_or_dummy[has_mask ? mi : 0]);
-      const float mb = has_mask ? inf * (mv - 1.0f) : 0.0f;
-      pre_mb = key < n ? mb : -INFINITY;
+    if (wave < R) {
+      const float mb = has_mask ? inf * (to_f32(pre_mv) - 1.0f) : 0.0f;
+      lds_mb[buf][wave][lane] = key0 + lane < n ? mb : -INFINITY;
     }
-  };
-  auto stash = [&](int buf) {
-#pragma unroll
-    for (int j = 0; j < 2; ++j) lds_kv[buf][wave * 2 + j][lane] = pre[j];
-    if (wave == 0) lds_mb[buf][lane] = pre_mb;
   };
 
   // ---- per-wave bias tile: lane <-> query, [u][c] = keys key0 + 32g + 16u + 8c .. +7 ----
@@ -150,27 +157,35 @@ __global__ __launch_bounds__(256, 2) void triattn_fwd_kernel(
       for (int c = 0; c < 2; ++c) dst[u][c] = load8<T>(bp + (u * 2 + c) * 512);
   };
 
-  f32x16 acc_o;                   // O^T
+  f32x16 acc_o[R];                // O^T per row
+  float m_run[R], l_run[R];       // running max (natural units) and denominator (this lane's keys)
 #pragma unroll
-  for (int r = 0; r < 16; ++r) acc_o[r] = 0.0f;
-  float m_run = -INFINITY;        // running max, natural units
-  float l_run = 0.0f;             // running denominator over this lane's keys (halves add up at the end)
+  for (int r = 0; r < R; ++r) {
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc_o[r][e] = 0.0f;
+    m_run[r] = -INFINITY;
+    l_run[r] = 0.0f;
+  }
 
-  // One key tile: logits, online softmax, P.V.  `tb` was fetched one tile ago.
-  auto process_tile = [&](int tile, V8 (&tb)[2][2]) {
-    const int buf = tile % 3;
-    const float mb_lane = lds_mb[buf][lane];
-    // Does this tile hold a masked or out-of-range key?  Same answer in all waves.
-    const bool masked_tile = __ballot(mb_lane != 0.0f) != 0ull;
+  // One key tile of one row: logits, online softmax, P.V.  `tb` was fetched one tile ago.
+  // Two complete instantiations, so that the (rare) masked path shares no code with - and
+  // cannot be speculated into - the fast path.
+  auto tile_row = [&](auto masked_tag, int buf, int r, V8 (&tb)[2][2]) {
+    constexpr bool MASKED = decltype(masked_tag)::value;
+    // all 8 operand fragments of the tile are requested from LDS up front, so their
+    // latency is paid once per tile instead of once per MFMA
+    V8 kvf[8];
+#pragma unroll
+    for (int f = 0; f < 8; ++f) kvf[f] = lds_kv[buf][r][f][lane];
     f32x16 s[2];
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
 #pragma unroll
-      for (int r = 0; r < 16; ++r) s[u][r] = 0.0f;
+      for (int e = 0; e < 16; ++e) s[u][e] = 0.0f;
 #pragma unroll
-      for (int kk = 0; kk < 2; ++kk) mma32(s[u], lds_kv[buf][u * 2 + kk][lane], qf[kk]);
+      for (int kk = 0; kk < 2; ++kk) mma32(s[u], kvf[u * 2 + kk], qf[r][kk]);
     }
-    if (!masked_tile) {
+    if constexpr (!MASKED) {
       // bias on the matrix pipe: S^T += Sel * Bias
 #pragma unroll
       for (int u = 0; u < 2; ++u)
@@ -183,8 +198,8 @@ __global__ __launch_bounds__(256, 2) void triattn_fwd_kernel(
 #pragma unroll
         for (int c = 0; c < 2; ++c) {
           const f32x8 b = to_f32(tb[u][c]);
-          const f32x4 m0 = *reinterpret_cast<const f32x4*>(&lds_mb[buf][32 * g + 16 * u + 8 * c]);
-          const f32x4 m1 = *reinterpret_cast<const f32x4*>(&lds_mb[buf][32 * g + 16 * u + 8 * c + 4]);
+          const f32x4 m0 = *reinterpret_cast<const f32x4*>(&lds_mb[buf][r][32 * g + 16 * u + 8 * c]);
+          const f32x4 m1 = *reinterpret_cast<const f32x4*>(&lds_mb[buf][r][32 * g + 16 * u + 8 * c + 4]);
 #pragma unroll
           for (int t = 0; t < 8; ++t) {
             const float mbv = t < 4 ? m0[t & 3] : m1[t & 3];
@@ -201,34 +216,33 @@ __global__ __launch_bounds__(256, 2) void triattn_fwd_kernel(
     float mt = fmaxf(fmaxf(fmaxf(mx[0], mx[1]), fmaxf(mx[2], mx[3])),
                      fmaxf(fmaxf(mx[4], mx[5]), fmaxf(mx[6], mx[7])));
     mt = fmaxf(mt, swap32(mt));
-    const float m_new = fmaxf(m_run, mt);          // finite: key0 < n is never excluded
-    const float alpha = fast_exp2((m_run - m_new) * kLog2e);   // 1 when the max did not move
-    m_run = m_new;
+    const float m_new = fmaxf(m_run[r], mt);        // finite: key0 < n is never excluded
+    const float alpha = fast_exp2((m_run[r] - m_new) * kLog2e);   // 1 when the max did not move
+    m_run[r] = m_new;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) acc_o[r] *= alpha;
+    for (int e = 0; e < 16; ++e) acc_o[r][e] *= alpha;
 
-    if (!masked_tile) {
+    float psum = 0.0f;
+    if constexpr (!MASKED) {
       const float nml = -m_new * kLog2e;
 #pragma unroll
       for (int u = 0; u < 2; ++u)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) s[u][r] = fmaf(s[u][r], kLog2e, nml);
+        for (int e = 0; e < 16; ++e) {
+          s[u][e] = fast_exp2(fmaf(s[u][e], kLog2e, nml));
+          psum += s[u][e];
+        }
     } else {
       // (s - m) first: exact when both sit near -1e9
 #pragma unroll
       for (int u = 0; u < 2; ++u)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) s[u][r] = (s[u][r] - m_new) * kLog2e;
+        for (int e = 0; e < 16; ++e) {
+          s[u][e] = fast_exp2((s[u][e] - m_new) * kLog2e);
+          psum += s[u][e];
+        }
     }
-    float psum = 0.0f;
-#pragma unroll
-    for (int u = 0; u < 2; ++u)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        s[u][r] = fast_exp2(s[u][r]);
-        psum += s[u][r];
-      }
-    l_run = l_run * alpha + psum;
+    l_run[r] = l_run[r] * alpha + psum;
 
     // O^T += V^T P^T
 #pragma unroll
@@ -238,19 +252,28 @@ __global__ __launch_bounds__(256, 2) void triattn_fwd_kernel(
         f32x8 p8;
 #pragma unroll
         for (int t = 0; t < 8; ++t) p8[t] = s[u][8 * c + t];
-        mma32(acc_o, lds_kv[buf][4 + u * 2 + c][lane], from_f32<T>(p8));
+        mma32(acc_o[r], kvf[4 + u * 2 + c], from_f32<T>(p8));
       }
+  };
+  auto process_tile = [&](int tile, V8 (&tb)[2][2]) {
+    const int buf = tile % 3;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      // Does this tile hold a masked or out-of-range key?  Same answer in all waves.
+      const float mb_lane = lds_mb[buf][r][lane];
+      if (__ballot(mb_lane != 0.0f) != 0ull) tile_row(std::true_type{}, buf, r, tb);
+      else tile_row(std::false_type{}, buf, r, tb);
+    }
   };
 
   // Tile t+2 travels global -> registers -> LDS while tile t is processed; the bias tile of
-  // t+1 is in flight to registers.  No load sits under a branch, so the compiler counts the
-  // outstanding loads exactly.
+  // t+1 is in flight to registers.  No load sits under a branch.
   V8 bias_a[2][2], bias_b[2][2];
   auto step = [&](int tile, V8 (&tb_cur)[2][2], V8 (&tb_nxt)[2][2]) {
     fetch(tile + 2);
     fetch_bias(tile + 1, tb_nxt);
     process_tile(tile, tb_cur);
-    stash((tile + 2) % 3);
+    stash(tile + 2);
     __syncthreads();
   };
 
@@ -266,23 +289,28 @@ __global__ __launch_bounds__(256, 2) void triattn_fwd_kernel(
     step(tile + 1, bias_b, bias_a);
   }
 
-  // ---- normalise, gate, store: lane <-> query, register r <-> d = acc_row(r, g) ----
+  // ---- normalise, gate, store: lane <-> query, register e <-> d = acc_row(e, g) ----
   // o may alias gate: every gate load is issued before the first store.
-  const int64_t base = qrow + 4 * g;
-  f32x4 gv[4];
+  f32x4 gv[R][4];
 #pragma unroll
-  for (int c = 0; c < 4; ++c) gv[c] = to_f32(*reinterpret_cast<const V4*>(gate + base + 8 * c));
-  const float inv = fast_rcp(l_run + swap32(l_run));
-  if (q0 + ln < n) {
+  for (int r = 0; r < R; ++r)
 #pragma unroll
-    for (int c = 0; c < 4; ++c) {
-      f32x4 ov;
+    for (int c = 0; c < 4; ++c)
+      gv[r][c] = to_f32(*reinterpret_cast<const V4*>(gate + qrow[r] + 4 * g + 8 * c));
 #pragma unroll
-      for (int t = 0; t < 4; ++t) {
-        // attention output rounded to T before the gate multiply, as the reference does
-        ov[t] = to_f32(from_f32<T>(acc_o[4 * c + t] * inv)) * gv[c][t];
+  for (int r = 0; r < R; ++r) {
+    const float inv = fast_rcp(l_run[r] + swap32(l_run[r]));
+    if (q0 + ln < n && i0 + r < n) {
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        f32x4 ov;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          // attention output rounded to T before the gate multiply, as the reference does
+          ov[t] = to_f32(from_f32<T>(acc_o[r][4 * c + t] * inv)) * gv[r][c][t];
+        }
+        *reinterpret_cast<V4*>(o + qrow[r] + 4 * g + 8 * c) = from_f32<T>(ov);
       }
-      *reinterpret_cast<V4*>(o + base + 8 * c) = from_f32<T>(ov);
     }
   }
 }
@@ -292,11 +320,14 @@ int triattn_fwd(const T* q, const T* k, const T* vt, const T* g, const T* tri_bi
                 T* o, int n, int heads, int key_pitch, int mask_transposed, float inf,
                 hipStream_t stream) {
   if (n == 0) return 0;
+  constexpr int R = PTX_ATTN_ROWS;
   const int n_qtiles = (n + 127) / 128;
-  const int64_t total = (int64_t)heads * n * n_qtiles;
+  const int n_rowgroups = (n + R - 1) / R;
+  const int64_t total = (int64_t)heads * n_rowgroups * n_qtiles;
   const int64_t per_xcd = (total + 7) / 8;
-  triattn_fwd_kernel<T><<<dim3((unsigned)(per_xcd * 8)), dim3(256), 0, stream>>>(
-      q, k, vt, g, tri_bias, mask, o, n, heads, key_pitch, mask_transposed, inf, n_qtiles, total);
+  triattn_fwd_kernel<T, R><<<dim3((unsigned)(per_xcd * 8)), dim3(256), 0, stream>>>(
+      q, k, vt, g, tri_bias, mask, o, n, heads, key_pitch, mask_transposed, inf, n_qtiles,
+      n_rowgroups, total);
   return 0;
 }
 
