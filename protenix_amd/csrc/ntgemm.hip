@@ -18,7 +18,7 @@
 namespace ptx {
 
 template <typename T>
-__global__ __launch_bounds__(256) void nt_gemm_batched_kernel(const T* __restrict__ a,
+__global__ __launch_bounds__(256, 2) void nt_gemm_batched_kernel(const T* __restrict__ a,
                                                               const T* __restrict__ b,
                                                               T* __restrict__ x, int n, int k_pitch,
                                                               int batch, int tiles_i, int tiles_j) {

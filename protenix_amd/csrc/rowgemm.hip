@@ -263,7 +263,7 @@ __device__ __forceinline__ int64_t plane_offset(int64_t p, int64_t n_rows, int n
 }
 
 template <typename T, int RB, int MODE>
-__global__ __launch_bounds__(256) void rowgemm_in_kernel(RowGemmInParams p) {
+__global__ __launch_bounds__(256, (MODE == kTriAttnIn ? 1 : 2)) void rowgemm_in_kernel(RowGemmInParams p) {
   typedef typename Vec8<T>::type V8;
   typedef typename VecE<T>::type VE_t;
   typedef Cfg<T> C;
@@ -684,7 +684,7 @@ struct RowGemmOutParams {
 };
 
 template <typename T, int RB>
-__global__ __launch_bounds__(256) void rowgemm_out_kernel(RowGemmOutParams p) {
+__global__ __launch_bounds__(256, 2) void rowgemm_out_kernel(RowGemmOutParams p) {
   typedef typename Vec8<T>::type V8;
   typedef typename VecE<T>::type VE_t;
   typedef Cfg<T> C;
