@@ -183,10 +183,12 @@ __device__ __forceinline__ typename VecE<T>::type add_vec(typename VecE<T>::type
 }
 
 // LDS traffic inside one wave: make the stores visible before the loads.
+// (LDS operations of one wave execute in order, so no hardware wait is needed; the fences
+// only keep the compiler from reordering the accesses.)
 __device__ __forceinline__ void wave_lds_sync() {
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
   __builtin_amdgcn_wave_barrier();
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
 // ---------------------------------------------------------------------------
@@ -344,6 +346,7 @@ __global__ __launch_bounds__(256, (MODE == kTriAttnIn ? 1 : 2)) void rowgemm_in_
   // Row-major destinations (kTriAttnIn q/k/g, kTransitionIn hidden, kTriMulOut out): the
   // logical row this lane stores in each read-back pass, or -1.
   int64_t rrow[RB][C::NPASS];
+  int rm_i[RB][C::NPASS], rm_j[RB][C::NPASS];   // the same rows as (outer, inner) of the pair tensor
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
@@ -352,7 +355,23 @@ __global__ __launch_bounds__(256, (MODE == kTriAttnIn ? 1 : 2)) void rowgemm_in_
       stage_coord<T>(ps, lane, mj, m0);
       const int64_t pr = row0 + rb * 32 + mj;
       rrow[rb][ps] = pr < p.n_rows ? pr : -1;
+      const uint32_t pc = (uint32_t)(pr < p.n_rows ? pr : 0);
+      rm_i[rb][ps] = pc / (uint32_t)p.n;
+      rm_j[rb][ps] = pc - rm_i[rb][ps] * (uint32_t)p.n;
     }
+  // Channel-major destinations: the VE consecutive logical rows this lane stores (the same
+  // in every read-back pass), as (outer, inner) of the pair tensor; all address divisions
+  // happen here, once, outside the chunk loop.
+  int cm_i[RB], cm_j[RB];
+  bool cm_ok[RB];
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
+    const int64_t pr = row0 + rb * 32 + (lane % C::LPM) * C::VE;
+    cm_ok[rb] = pr < p.n_rows;
+    const uint32_t pc = (uint32_t)(cm_ok[rb] ? pr : 0);
+    cm_i[rb] = pc / (uint32_t)p.n;
+    cm_j[rb] = pc - cm_i[rb] * (uint32_t)p.n;
+  }
 
   const int nch = n_chunks<MODE>(p);
   V8 pre[4];
@@ -402,8 +421,8 @@ __global__ __launch_bounds__(256, (MODE == kTriAttnIn ? 1 : 2)) void rowgemm_in_
         T* dst = plane0 + (int64_t)(c_first + chn) * plane_stride;
         const VE_t v = stage_get_vec<T>(st, chn, r0);
         if (vec_ok) {
-          const int64_t off = plane_offset(pr, p.n_rows, p.n, row_pitch);
-          if (off >= 0) *reinterpret_cast<VE_t*>(dst + off) = v;
+          if (cm_ok[rb])
+            *reinterpret_cast<VE_t*>(dst + (int64_t)cm_i[rb] * row_pitch + cm_j[rb]) = v;
         } else {
 #pragma unroll
           for (int e = 0; e < C::VE; ++e) {
@@ -461,6 +480,11 @@ __global__ __launch_bounds__(256, (MODE == kTriAttnIn ? 1 : 2)) void rowgemm_in_
         }
       }
     }
+
+    // The next chunk's weights go to the other LDS buffer now, before this chunk's stores
+    // are issued: waiting for those loads later would also wait for every store issued in
+    // between (memory operations retire in order).
+    if (C::NBUF == 2) stash(buf ^ 1);
 
     // ------------------------------ epilogues ------------------------------
     if constexpr (MODE == kTriMulIn) {
@@ -530,12 +554,10 @@ __global__ __launch_bounds__(256, (MODE == kTriAttnIn ? 1 : 2)) void rowgemm_in_
             for (int ps = 0; ps < C::NPASS; ++ps) {
               int mj, m0;
               stage_coord<T>(ps, lane, mj, m0);
-              if (rrow[rb][ps] >= 0) {
-                const uint32_t pr = (uint32_t)rrow[rb][ps];
-                const uint32_t i = pr / (uint32_t)p.n, j = pr - i * (uint32_t)p.n;
-                *reinterpret_cast<VE_t*>(outp + attn_k_offset(h, i, j, m0, p.n, key_tiles)) =
+              if (rrow[rb][ps] >= 0)
+                *reinterpret_cast<VE_t*>(
+                    outp + attn_k_offset(h, rm_i[rb][ps], rm_j[rb][ps], m0, p.n, key_tiles)) =
                     stage_get_vec<T>(st, mj, m0);
-              }
             }
           }
       } else {
@@ -563,10 +585,10 @@ __global__ __launch_bounds__(256, (MODE == kTriAttnIn ? 1 : 2)) void rowgemm_in_
               const VE_t v = stage_get_vec<T>(st, chn, r0);
               T* outp = (T*)p.out[which];
               if (vec_ok) {
-                if (pr < p.n_rows) {
-                  const uint32_t i = (uint32_t)pr / (uint32_t)p.n, j = (uint32_t)pr - i * (uint32_t)p.n;
-                  const int64_t off = which == 3 ? attn_v_offset(h, i, j, chn, p.n, key_tiles)
-                                                 : attn_b_offset(chn, i, j, q_blocks, key_tiles);
+                if (cm_ok[rb]) {
+                  const int64_t off =
+                      which == 3 ? attn_v_offset(h, cm_i[rb], cm_j[rb], chn, p.n, key_tiles)
+                                 : attn_b_offset(chn, cm_i[rb], cm_j[rb], q_blocks, key_tiles);
                   *reinterpret_cast<VE_t*>(outp + off) = v;
                 }
               } else {
@@ -651,8 +673,10 @@ __global__ __launch_bounds__(256, (MODE == kTriAttnIn ? 1 : 2)) void rowgemm_in_
       }
     }
 
-    if (C::NBUF == 1) __syncthreads();      // everyone is done reading the single buffer
-    stash(C::NBUF == 2 ? (buf ^ 1) : 0);
+    if (C::NBUF == 1) {
+      __syncthreads();      // everyone is done reading the single buffer
+      stash(0);
+    }
     __syncthreads();
   }
 }

@@ -61,7 +61,13 @@ class PairformerBlock(nn.Module):
         assert triangle_attention in ("torch", "deepspeed", "triattention", "cuequivariance")
         if not inplace_safe or not z.is_contiguous():
             z = z.clone(memory_format=torch.contiguous_format)
-        # every update below is "z += f(z)" fused into the kernel epilogues
+        self._pair_track(z, pair_mask)
+        if self.c_s > 0:
+            s = self._single_track(s, self.attention_pair_bias.pair_bias(z))
+        return s, z
+
+    def _pair_track(self, z: torch.Tensor, pair_mask: Optional[torch.Tensor]) -> None:
+        """The five pair updates, each "z += f(z)" fused into a kernel epilogue."""
         self.tri_mul_out(z, mask=pair_mask, inplace_safe=True, _add_with_inplace=True)
         self.tri_mul_in(z, mask=pair_mask, inplace_safe=True, _add_with_inplace=True)
         self.tri_att_start._run(z, pair_mask, transposed=False, residual_inplace=True)
@@ -69,10 +75,12 @@ class PairformerBlock(nn.Module):
         # mask^T, expressed through transposed addressing of z and mask
         self.tri_att_end._run(z, pair_mask, transposed=True, residual_inplace=True)
         self.pair_transition(z, _residual_out=z)
-        if self.c_s > 0:
-            s = s + self.attention_pair_bias(a=s, s=None, z=z)
-            s = s + self.single_transition(s)
-        return s, z
+
+    def _single_track(self, s: torch.Tensor, bias: torch.Tensor) -> torch.Tensor:
+        """s += attention(s; bias from z); s += transition(s).  Needs nothing of z but
+        `bias`, and z never depends on s."""
+        s = s + self.attention_pair_bias.forward_with_bias(s, bias)
+        return s + self.single_transition(s)
 
 
 class PairformerStack(nn.Module):
@@ -98,8 +106,41 @@ class PairformerStack(nn.Module):
         if not inplace_safe and len(self.blocks) > 0:
             # one private copy for the whole stack; the blocks then work in place
             z = z.clone(memory_format=torch.contiguous_format)
+        if not z.is_contiguous():
+            z = z.contiguous()
         for blk in self.blocks:
-            s, z = blk(s, z, pair_mask, triangle_multiplicative=triangle_multiplicative,
-                       triangle_attention=triangle_attention, inplace_safe=True,
-                       chunk_size=chunk_size)
+            if blk.training:
+                raise RuntimeError("protenix_amd.PairformerStack is inference-only: call .eval()")
+        if triangle_multiplicative not in ("torch", "cuequivariance"):
+            raise ValueError(
+                "triangle_multiplicative must be 'cuequivariance' or 'torch', but got "
+                f"{triangle_multiplicative}")
+        assert triangle_attention in ("torch", "deepspeed", "triattention", "cuequivariance")
+        if not z.is_cuda or s is None or any(b.c_s == 0 for b in self.blocks):
+            for blk in self.blocks:
+                s, z = blk(s, z, pair_mask, inplace_safe=True)
+            return s, z
+        # The pair track never reads s, and the single track reads z only through the pair
+        # bias: the small single-track kernels of block b run on a second stream (default
+        # priority) underneath the pair kernels of block b + 1.
+        main = torch.cuda.current_stream(z.device)
+        side = self._side_stream(z.device)
+        side.wait_stream(main)
+        for blk in self.blocks:
+            blk._pair_track(z, pair_mask)
+            bias = blk.attention_pair_bias.pair_bias(z)   # reads z before the next block writes it
+            ready = main.record_event()
+            with torch.cuda.stream(side):
+                side.wait_event(ready)
+                s = blk._single_track(s, bias)
+            bias.record_stream(side)
+        main.wait_stream(side)
+        s.record_stream(main)
         return s, z
+
+    def _side_stream(self, device: torch.device) -> "torch.cuda.Stream":
+        streams = self.__dict__.setdefault("_streams", {})
+        key = (device.type, device.index)
+        if key not in streams:
+            streams[key] = torch.cuda.Stream(device=device)
+        return streams[key]

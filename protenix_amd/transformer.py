@@ -110,6 +110,11 @@ class AttentionPairBias(nn.Module):
                 enable_efficient_fusion: bool = False) -> torch.Tensor:
         if n_queries or n_keys:
             raise NotImplementedError("local attention belongs to the diffusion module")
-        _forward_only(a, z, *self.parameters())
+        return self.forward_with_bias(a, self.pair_bias(z))
+
+    def forward_with_bias(self, a: torch.Tensor, bias: torch.Tensor) -> torch.Tensor:
+        """The single-track part, given bias = pair_bias(z).  Split off so that a
+        caller can run it on another stream once the pass over z is done."""
+        _forward_only(a, bias, *self.parameters())
         a = self.layernorm_a(a)
-        return self.attention(q_x=a, kv_x=a, attn_bias=self.pair_bias(z))
+        return self.attention(q_x=a, kv_x=a, attn_bias=bias)
