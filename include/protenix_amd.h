@@ -60,6 +60,25 @@ PTX_API const char* ptx_last_error_string(void);
 PTX_API int ptx_key_pitch(int n);
 
 /*
+ * Element counts of the workspaces that travel between the stages of one
+ * triangle update.  Their layouts are the library's own (MFMA operand order, so
+ * that the consuming kernel reads them in contiguous 1 KB runs); the caller
+ * only allocates them, uninitialised, and passes them from stage to stage.
+ *   ptx_trimul_operand_elems: one of a, b.  Per channel, rows in blocks of 32 and
+ *     K in steps of 16; fragment (c, rb, ks) holds 64 lanes x 8 elements, lane
+ *     32*g + r = row 32*rb + r, K = 16*ks + 8*g .. +7:
+ *     c_hidden * 32*ceil(n/32) * ptx_key_pitch(n).
+ *   ptx_triattn_kv_elems: one of k, vt.  Per (head, row i), keys in tiles of 64, a
+ *     tile = 4 fragments of 64 lanes x 8 elements: heads * n * ptx_key_pitch(n) * 32.
+ *   ptx_triattn_bias_elems: the triangle bias.  Per head, queries in blocks of 32
+ *     and keys in tiles of 64: heads * 32*ceil(n/32) * ptx_key_pitch(n).
+ * q, g and o of the attention are head-major, [heads][n][n][d].
+ */
+PTX_API int64_t ptx_trimul_operand_elems(int n, int c_hidden);
+PTX_API int64_t ptx_triattn_kv_elems(int n, int heads);
+PTX_API int64_t ptx_triattn_bias_elems(int n, int heads);
+
+/*
  * LayerNorm forward over the last dimension.
  * Replaces fast_layer_norm_cuda_v2.forward_{none,with_bias,with_weight,
  * with_both}_affine (layer_norm_cuda.cpp:142-157; kernel
@@ -78,8 +97,9 @@ PTX_API int ptx_layernorm_fwd(const void* x, const void* gamma, const void* beta
  *   outgoing (incoming = 0):  a[c][i][k] = a(z[i][k])[c]
  *   incoming (incoming = 1):  a[c][i][k] = a(z[k][i])[c]      (same for b)
  *   z [n][n][c_z], mask [n][n] in `dtype` or NULL (= ones),
- *   w_* [c_hidden][c_z], a, b [c_hidden][n][k_pitch], k_pitch = ptx_key_pitch(n).
- *   c_z = c_hidden = 128.
+ *   w_* [c_hidden][c_z]; a, b: workspaces of ptx_trimul_operand_elems(n, c_hidden)
+ *   elements each, written in the contraction's operand order (rows i beyond n and
+ *   K beyond n stay unwritten); k_pitch = ptx_key_pitch(n).  c_z = c_hidden = 128.
  */
 PTX_API int ptx_trimul_project(const void* z, const void* mask, const void* ln_w, const void* ln_b,
                        const void* w_ap, const void* w_ag, const void* w_bp, const void* w_bg,
@@ -90,7 +110,7 @@ PTX_API int ptx_trimul_project(const void* z, const void* mask, const void* ln_w
  * Triangle multiplication, stage 2 (triangular.py:123-150): for every channel
  *   x[c][i][j] = sum_k a[c][i][k] * b[c][j][k]
  * which with the stage-1 layouts is 'ikc,jkc->ijc' (outgoing) or
- * 'kic,kjc->ijc' (incoming).  a, b [c][n][k_pitch]; x [c][n][n] dense.
+ * 'kic,kjc->ijc' (incoming).  a, b as written by stage 1; x [c][n][n] dense.
  */
 PTX_API int ptx_trimul_contract(const void* a, const void* b, void* x, int n, int c, int k_pitch,
                         int dtype, void* stream);
@@ -111,9 +131,9 @@ PTX_API int ptx_trimul_output(const void* x, const void* z, const void* ln_in_w,
  *   xn = LN(x);  q = W_q xn / sqrt(d);  k = W_k xn;  v = W_v xn;
  *   g = sigmoid(W_g xn);  tri_bias = W_b xn
  * over logical rows p = i*n + j of x = z (transposed = 0) or z^T (transposed = 1).
- *   q, k, g [n][n][heads*d];  vt [n][heads*d][key_pitch] (v transposed per row i);
- *   tri_bias [heads][n][key_pitch];  key_pitch = ptx_key_pitch(n).
- *   c_in = heads*d = 128, d = 32.
+ *   q, g [heads][n][n][d] (logical row p = i*n + j);  k, vt: workspaces of
+ *   ptx_triattn_kv_elems(n, heads) elements;  tri_bias: ptx_triattn_bias_elems(n, heads)
+ *   elements;  key_pitch = ptx_key_pitch(n).   c_in = heads*d = 128, d = 32.
  */
 PTX_API int ptx_triattn_project(const void* z, const void* ln_w, const void* ln_b, const void* w_q,
                         const void* w_k, const void* w_v, const void* w_g, const void* w_b,
@@ -130,7 +150,8 @@ PTX_API int ptx_triattn_project(const void* z, const void* ln_w, const void* ln_
  * reference's order in fp32, so a fully masked row gives the mean of v, as
  * layers.py:286-291 does.
  *   mask [n][n] in `dtype` or NULL; mask(i,k) = mask[i][k], or mask[k][i] when
- *   mask_transposed = 1.   o [n][n][heads*d] (may alias g, not q/k/vt).
+ *   mask_transposed = 1.   q, k, vt, g, tri_bias as written by stage 1;
+ *   o [heads][n][n][d] (may alias g, not q/k/vt).
  */
 PTX_API int ptx_triattn_fwd(const void* q, const void* k, const void* vt, const void* g,
                     const void* tri_bias, const void* mask, void* o, int n, int heads, int d,
@@ -139,7 +160,8 @@ PTX_API int ptx_triattn_fwd(const void* q, const void* k, const void* vt, const 
 /*
  * Triangle attention, stage 3 (layers.py:392-396 + the caller's residual add,
  * pairformer.py:189-213):  out(p) = [z(p) +] W_o o[p], where logical row p maps
- * to z[i][j] or, transposed = 1, z[j][i].  out may alias z.
+ * to z[i][j] or, transposed = 1, z[j][i].  o [heads][n][n][d] as written by
+ * stage 2; out may alias z.
  */
 PTX_API int ptx_triattn_output(const void* o, const void* w_o, const void* z, void* out, int n,
                        int c_in, int transposed, int add_residual, int dtype, void* stream);

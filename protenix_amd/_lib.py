@@ -26,6 +26,9 @@ SIGNATURES = {
     "ptx_version": (_i, []),
     "ptx_last_error_string": (ctypes.c_char_p, []),
     "ptx_key_pitch": (_i, [_i]),
+    "ptx_trimul_operand_elems": (_l, [_i, _i]),
+    "ptx_triattn_kv_elems": (_l, [_i, _i]),
+    "ptx_triattn_bias_elems": (_l, [_i, _i]),
     "ptx_layernorm_fwd": (_i, [_p, _p, _p, _p, _p, _p, _l, _i, _f, _i, _p]),
     "ptx_trimul_project": (_i, [_p] * 10 + [_i, _i, _i, _i, _i, _f, _i, _p]),
     "ptx_trimul_contract": (_i, [_p, _p, _p, _i, _i, _i, _i, _p]),

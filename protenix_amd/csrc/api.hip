@@ -57,6 +57,18 @@ PTX_API int ptx_version(void) { return PTX_ABI_VERSION; }
 PTX_API const char* ptx_last_error_string(void) { return g_err; }
 
 PTX_API int ptx_key_pitch(int n) { return n <= 0 ? 0 : ((n + 63) / 64) * 64; }
+PTX_API int64_t ptx_trimul_operand_elems(int n, int c_hidden) {
+  if (n <= 0 || c_hidden <= 0) return 0;
+  return (int64_t)c_hidden * (((n + 31) / 32) * 32) * ptx_key_pitch(n);
+}
+PTX_API int64_t ptx_triattn_kv_elems(int n, int heads) {
+  if (n <= 0 || heads <= 0) return 0;
+  return (int64_t)heads * n * ptx_key_pitch(n) * 32;
+}
+PTX_API int64_t ptx_triattn_bias_elems(int n, int heads) {
+  if (n <= 0 || heads <= 0) return 0;
+  return (int64_t)heads * (((n + 31) / 32) * 32) * ptx_key_pitch(n);
+}
 
 PTX_API int ptx_layernorm_fwd(const void* x, const void* gamma, const void* beta, void* y, float* mean,
                       float* rstd, int64_t rows, int cols, float eps, int dtype, void* stream) {

@@ -109,6 +109,22 @@ struct RowMap {
 };
 
 // ---------------------------------------------------------------------------
+// Operand layout of the triangle-multiplication contraction (written by the
+// projection kernel, read by the contraction): per channel, rows in blocks of 32
+// and K in steps of 16; one (row block, K step) fragment is stored in MFMA
+// operand order, 64 lanes x 8 elements = 512 contiguous elements: lane
+// 32*g + r holds K = 16*ks + 8*g .. +7 of row 32*rb + r.  A channel has
+// ceil(n/32) row blocks (rows beyond n are never written) and k_pitch/16 K steps
+// (K beyond n is never written; the contraction zeroes it on the way in).
+// ---------------------------------------------------------------------------
+constexpr int kFragElems = 512;
+
+__host__ __device__ __forceinline__ int64_t trimul_frag_offset(int c, int rb, int ks, int n_rb,
+                                                               int n_ks) {
+  return (((int64_t)c * n_rb + rb) * n_ks + ks) * kFragElems;
+}
+
+// ---------------------------------------------------------------------------
 // Operand layouts of the triangle-attention core (written by the projection
 // kernel, read by the attention kernel).  Keys are grouped in tiles of 64; one
 // operand tile is stored in MFMA fragment order, 4 fragments x 64 lanes x 8

@@ -87,19 +87,16 @@ __device__ __forceinline__ void normalize_row(f32x8 (&v)[kKSteps], const T* __re
   }
 }
 
-// Load RB*32 rows starting at row0 (rows >= n_rows re-read the last valid row;
-// their results are never stored) and, if LN, normalise them.
+// Load RB row blocks whose lane rows start at element offsets off[rb] (+ 8*g added here)
+// and, if LN, normalise them.
 template <typename T, int RB, bool LN>
-__device__ __forceinline__ void load_rows(RowFrags<T, RB>& out, const T* __restrict__ x,
-                                          const RowMap& map, int64_t row0, int64_t n_rows,
-                                          const T* __restrict__ gamma, const T* __restrict__ beta,
-                                          float eps, int lane) {
-  const int n = lane & 31, g = lane >> 5;
+__device__ __forceinline__ void load_rows_at(RowFrags<T, RB>& out, const T* __restrict__ x,
+                                             const int64_t (&off)[RB], const T* __restrict__ gamma,
+                                             const T* __restrict__ beta, float eps, int lane) {
+  const int g = lane >> 5;
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
-    int64_t p = row0 + rb * 32 + n;
-    p = p < n_rows ? p : n_rows - 1;
-    const T* rp = x + map(p) + 8 * g;
+    const T* rp = x + off[rb] + 8 * g;
     if (!LN) {
 #pragma unroll
       for (int kk = 0; kk < kKSteps; ++kk) out.f[rb][kk] = load8<T>(rp + 16 * kk);
@@ -110,6 +107,23 @@ __device__ __forceinline__ void load_rows(RowFrags<T, RB>& out, const T* __restr
       normalize_row<T>(v, gamma, beta, eps, g, out.f[rb]);
     }
   }
+}
+
+// Load RB*32 consecutive logical rows starting at row0 (rows >= n_rows re-read the last
+// valid row; their results are never stored).
+template <typename T, int RB, bool LN>
+__device__ __forceinline__ void load_rows(RowFrags<T, RB>& out, const T* __restrict__ x,
+                                          const RowMap& map, int64_t row0, int64_t n_rows,
+                                          const T* __restrict__ gamma, const T* __restrict__ beta,
+                                          float eps, int lane) {
+  int64_t off[RB];
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
+    int64_t p = row0 + rb * 32 + (lane & 31);
+    p = p < n_rows ? p : n_rows - 1;
+    off[rb] = map(p);
+  }
+  load_rows_at<T, RB, LN>(out, x, off, gamma, beta, eps, lane);
 }
 
 // One weight fragment: 32 output columns x 16 K values, lane -> (column l%32,
@@ -255,15 +269,6 @@ __device__ __forceinline__ void chunk_tile(const RowGemmInParams& p, int ch, int
   }
 }
 
-// Element offset of logical row p inside one channel plane [n][pitch], or -1 if p
-// is out of range.  With n % VE == 0, VE rows starting at a multiple of VE share
-// one plane row and are contiguous.
-__device__ __forceinline__ int64_t plane_offset(int64_t p, int64_t n_rows, int n, int64_t pitch) {
-  if (p >= n_rows) return -1;
-  const uint32_t i = (uint32_t)p / (uint32_t)n;
-  return (int64_t)i * pitch + ((uint32_t)p - i * (uint32_t)n);
-}
-
 template <typename T, int RB, int MODE>
 __global__ __launch_bounds__(256, (MODE == kTriAttnIn ? 1 : 2)) void rowgemm_in_kernel(RowGemmInParams p) {
   typedef typename Vec8<T>::type V8;
@@ -278,9 +283,32 @@ __global__ __launch_bounds__(256, (MODE == kTriAttnIn ? 1 : 2)) void rowgemm_in_
   T* st = lds_stage[wave];
   const bool vec_ok = (p.n % C::VE) == 0;   // channel-major vectors stay inside one plane row
 
+  // kTriMulIn works on 2-D patches of the pair tensor instead of runs of logical rows: a
+  // workgroup covers 16*RB outer indices x 8 inner indices, a row block 4 x 8 (MFMA row r <->
+  // outer pi0 + 4*rb + r/8, inner pk0 + r%8), which makes a row block's 32 values of one
+  // channel 64 contiguous bytes of the contraction's fragment-ordered operands.
+  int pi0 = 0, pk0 = 0;
+  if constexpr (MODE == kTriMulIn) {
+    const uint32_t n_kb = (uint32_t)(p.n + 7) >> 3;
+    const uint32_t ip = blockIdx.x / n_kb;
+    pk0 = (int)(blockIdx.x - ip * n_kb) * 8;
+    pi0 = (int)ip * (16 * RB) + wave * (4 * RB);
+  }
+
   RowFrags<T, RB> xf;
-  load_rows<T, RB, true>(xf, (const T*)p.x, p.xmap, row0, p.n_rows, (const T*)p.gamma,
-                         (const T*)p.beta, p.eps, lane);
+  if constexpr (MODE == kTriMulIn) {
+    int64_t off[RB];
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) {
+      const int i = min(pi0 + 4 * rb + (n >> 3), p.n - 1), k = min(pk0 + (n & 7), p.n - 1);
+      off[rb] = (int64_t)i * p.xmap.stride_outer + (int64_t)k * p.xmap.stride_inner;
+    }
+    load_rows_at<T, RB, true>(xf, (const T*)p.x, off, (const T*)p.gamma, (const T*)p.beta, p.eps,
+                              lane);
+  } else {
+    load_rows<T, RB, true>(xf, (const T*)p.x, p.xmap, row0, p.n_rows, (const T*)p.gamma,
+                           (const T*)p.beta, p.eps, lane);
+  }
 
   // kTriMulOut: second fragment set = LayerNorm_out of the channel-major triangle product,
   // transposed through the staging tile 32 channels at a time.
@@ -334,9 +362,9 @@ __global__ __launch_bounds__(256, (MODE == kTriAttnIn ? 1 : 2)) void rowgemm_in_
     if (p.mask) {
 #pragma unroll
       for (int rb = 0; rb < RB; ++rb) {
-        int64_t pr = row0 + rb * 32 + n;
-        pr = pr < p.n_rows ? pr : p.n_rows - 1;
-        const float mv = to_f32(((const T*)p.mask)[p.mmap(pr)]);
+        const int i = min(pi0 + 4 * rb + (n >> 3), p.n - 1), k = min(pk0 + (n & 7), p.n - 1);
+        const float mv = to_f32(((const T*)p.mask)[(int64_t)i * p.mmap.stride_outer +
+                                                   (int64_t)k * p.mmap.stride_inner]);
         if (g == 0) lds_mask[wave][rb * 32 + n] = mv;
       }
       wave_lds_sync();
@@ -407,33 +435,6 @@ __global__ __launch_bounds__(256, (MODE == kTriAttnIn ? 1 : 2)) void rowgemm_in_
       }
     }
   };
-  // Channel-major store of the staged tile: major = channel (first = c_first, only
-  // channels < c_lim exist), minor = the 32 logical rows of row block rb; a channel's
-  // plane is [n][row_pitch] and planes are plane_stride apart.
-  auto store_channel_major = [&](T* plane0, int64_t plane_stride, int64_t row_pitch, int c_first,
-                                 int c_lim, int rb) {
-#pragma unroll
-    for (int ps = 0; ps < C::NPASS; ++ps) {
-      int chn, r0;
-      stage_coord<T>(ps, lane, chn, r0);
-      const int64_t pr = row0 + rb * 32 + r0;
-      if (c_first + chn < c_lim) {
-        T* dst = plane0 + (int64_t)(c_first + chn) * plane_stride;
-        const VE_t v = stage_get_vec<T>(st, chn, r0);
-        if (vec_ok) {
-          if (cm_ok[rb])
-            *reinterpret_cast<VE_t*>(dst + (int64_t)cm_i[rb] * row_pitch + cm_j[rb]) = v;
-        } else {
-#pragma unroll
-          for (int e = 0; e < C::VE; ++e) {
-            const int64_t off = plane_offset(pr + e, p.n_rows, p.n, row_pitch);
-            if (off >= 0) dst[off] = v[e];
-          }
-        }
-      }
-    }
-  };
-
   for (int ch = 0; ch < nch; ++ch) {
     const int buf = C::NBUF == 2 ? (ch & 1) : 0;
     fetch(min(ch + 1, nch - 1));   // unconditional: keeps the outstanding-load count static
@@ -508,7 +509,18 @@ __global__ __launch_bounds__(256, (MODE == kTriAttnIn ? 1 : 2)) void rowgemm_in_
         wave_lds_sync();
         stage_put<T>(st, vals, lane);
         wave_lds_sync();
-        store_channel_major(outp, (int64_t)p.n * p.pitch, p.pitch, c0, kC, rb);
+        // fragment-ordered store: 8 consecutive inner indices of one outer index = the 16
+        // bytes of one operand lane (half-wave (pk0/8)%2, row outer%32)
+        const int n_rb = (p.n + 31) >> 5, n_ks = p.pitch >> 4;
+#pragma unroll
+        for (int ps = 0; ps < C::NPASS; ++ps) {
+          int chn, r0;
+          stage_coord<T>(ps, lane, chn, r0);
+          const int i = pi0 + 4 * rb + (r0 >> 3);
+          const int64_t off = trimul_frag_offset(c0 + chn, i >> 5, pk0 >> 4, n_rb, n_ks) +
+                              ((pk0 >> 3) & 1) * 256 + (i & 31) * 8 + (r0 & 7);
+          *reinterpret_cast<VE_t*>(outp + off) = stage_get_vec<T>(st, chn, r0);
+        }
       }
     } else if constexpr (MODE == kTriAttnIn) {
       // Outputs in the attention core's layouts (common.h): q and the gate head-major
@@ -685,7 +697,9 @@ template <typename T, int MODE>
 int launch_rowgemm_in(const RowGemmInParams& p, hipStream_t stream) {
   constexpr int RB = (sizeof(T) == 2 && MODE != kTriMulOut) ? 2 : 1;
   const int64_t rows_per_block = 4 * RB * 32;
-  const int64_t blocks = (p.n_rows + rows_per_block - 1) / rows_per_block;
+  int64_t blocks = (p.n_rows + rows_per_block - 1) / rows_per_block;
+  if (MODE == kTriMulIn)   // 2-D patches: 16*RB outer x 8 inner indices per workgroup
+    blocks = (int64_t)((p.n + 16 * RB - 1) / (16 * RB)) * ((p.n + 7) / 8);
   if (blocks == 0) return 0;
   rowgemm_in_kernel<T, RB, MODE><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(p);
   return 0;

@@ -109,8 +109,10 @@ def triangle_multiplication(z: torch.Tensor, mask: Optional[torch.Tensor], w: di
     dt, st = _dt(z), _stream()
     pitch = key_pitch(n)
     mask = _mask_for(mask, z)
-    a = torch.empty((c_h, n, pitch), dtype=z.dtype, device=z.device)
-    b = torch.empty((c_h, n, pitch), dtype=z.dtype, device=z.device)
+    # contraction operands in the library's fragment order (see include/protenix_amd.h)
+    n_op = lib.ptx_trimul_operand_elems(n, c_h)
+    a = torch.empty((n_op,), dtype=z.dtype, device=z.device)
+    b = torch.empty((n_op,), dtype=z.dtype, device=z.device)
     with torch.cuda.device(z.device):
         _call("trimul_project", lib.ptx_trimul_project, _ptr(z), _ptr(mask), _ptr(w["ln_in_w"]), _ptr(w["ln_in_b"]), _ptr(w["w_ap"]),
             _ptr(w["w_ag"]), _ptr(w["w_bp"]), _ptr(w["w_bg"]), _ptr(a), _ptr(b), n, c_z, c_h, pitch,
@@ -140,14 +142,14 @@ def triangle_attention(z: torch.Tensor, mask: Optional[torch.Tensor], w: dict, h
     pitch = key_pitch(n)
     mask = _mask_for(mask, z)
     dev = z.device
-    kt, qb = pitch // 64, (n + 31) // 32
-    # attention-core layouts (csrc/common.h): q, gate, output head-major; K, V^T and the
-    # triangle bias in fragment-ordered key tiles of 2048 elements
+    # attention-core layouts (see include/protenix_amd.h): q, gate, output head-major; K, V^T
+    # and the triangle bias in fragment-ordered key tiles
+    n_kv, n_tb = lib.ptx_triattn_kv_elems(n, heads), lib.ptx_triattn_bias_elems(n, heads)
     q = torch.empty((heads, n, n, d), dtype=z.dtype, device=dev)
     g = torch.empty((heads, n, n, d), dtype=z.dtype, device=dev)
-    k = torch.empty((heads, n, kt, 2048), dtype=z.dtype, device=dev)
-    vt = torch.empty((heads, n, kt, 2048), dtype=z.dtype, device=dev)
-    tb = torch.empty((heads, qb, kt, 2048), dtype=z.dtype, device=dev)
+    k = torch.empty((n_kv,), dtype=z.dtype, device=dev)
+    vt = torch.empty((n_kv,), dtype=z.dtype, device=dev)
+    tb = torch.empty((n_tb,), dtype=z.dtype, device=dev)
     with torch.cuda.device(dev):
         _call("triattn_project", lib.ptx_triattn_project, _ptr(z), _ptr(w["ln_w"]),
               _ptr(w["ln_b"]), _ptr(w["w_q"]), _ptr(w["w_k"]), _ptr(w["w_v"]), _ptr(w["w_g"]),
