@@ -98,8 +98,9 @@ PTX_API int ptx_layernorm_fwd(const void* x, const void* gamma, const void* beta
  *   incoming (incoming = 1):  a[c][i][k] = a(z[k][i])[c]      (same for b)
  *   z [n][n][c_z], mask [n][n] in `dtype` or NULL (= ones),
  *   w_* [c_hidden][c_z]; a, b: workspaces of ptx_trimul_operand_elems(n, c_hidden)
- *   elements each, written in the contraction's operand order (rows i beyond n and
- *   K beyond n stay unwritten); k_pitch = ptx_key_pitch(n).  c_z = c_hidden = 128.
+ *   elements each, written in the contraction's operand order (K between n and
+ *   k_pitch is written as zeros, rows beyond n stay unwritten);
+ *   k_pitch = ptx_key_pitch(n).  c_z = c_hidden = 128.
  */
 PTX_API int ptx_trimul_project(const void* z, const void* mask, const void* ln_w, const void* ln_b,
                        const void* w_ap, const void* w_ag, const void* w_bp, const void* w_bg,
@@ -110,7 +111,8 @@ PTX_API int ptx_trimul_project(const void* z, const void* mask, const void* ln_w
  * Triangle multiplication, stage 2 (triangular.py:123-150): for every channel
  *   x[c][i][j] = sum_k a[c][i][k] * b[c][j][k]
  * which with the stage-1 layouts is 'ikc,jkc->ijc' (outgoing) or
- * 'kic,kjc->ijc' (incoming).  a, b as written by stage 1; x [c][n][n] dense.
+ * 'kic,kjc->ijc' (incoming).  a, b as written by stage 1 (K between n and k_pitch
+ * must hold zeros); x [c][n][n] dense.
  */
 PTX_API int ptx_trimul_contract(const void* a, const void* b, void* x, int n, int c, int k_pitch,
                         int dtype, void* stream);

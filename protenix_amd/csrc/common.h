@@ -115,7 +115,7 @@ struct RowMap {
 // operand order, 64 lanes x 8 elements = 512 contiguous elements: lane
 // 32*g + r holds K = 16*ks + 8*g .. +7 of row 32*rb + r.  A channel has
 // ceil(n/32) row blocks (rows beyond n are never written) and k_pitch/16 K steps
-// (K beyond n is never written; the contraction zeroes it on the way in).
+// (K between n and k_pitch is written as zeros: the contraction runs over it).
 // ---------------------------------------------------------------------------
 constexpr int kFragElems = 512;
 

@@ -13,15 +13,14 @@
 // SIMD), so each fragment read from LDS feeds 4 MFMAs.  A K stage (KK steps of
 // 16) of both operand panels is staged through LDS, double-buffered.  The wave
 // is software-pipelined by hand, because with one wave per SIMD nothing else
-// hides latency: the fragments of K step t+1 are read from LDS between the two
-// halves of step t's MFMAs, the next stage's global loads are issued a whole
-// stage before they are written to LDS, and the LDS write + workgroup barrier
-// sit in the middle of a step's MFMAs as well.
+// hides latency: the fragments of K step t+1 are read from LDS under step t's
+// MFMAs, global loads are issued two stages before they are written to LDS, and
+// loads, LDS writes and LDS reads are spread evenly between the MFMAs.
 //
 // MFMA operands are ordered so that a lane ends up holding 4 consecutive j per
 // register quad of one row i: results leave through a per-wave LDS tile as
-// 16-byte stores along j.  No load sits under a branch (indices are clamped, K
-// beyond n is zeroed on the way into LDS).  Workgroups are numbered so that all
+// 16-byte stores along j.  No load sits under a branch (indices are clamped;
+// K between n and k_pitch must hold zeros, which the projection kernel writes).  Workgroups are numbered so that all
 // tiles of one channel land on one XCD (round-robin dispatch: id % 8), keeping
 // that channel's panels in its L2.
 #include "common.h"
@@ -32,7 +31,6 @@ namespace ptx {
 template <typename T> struct GemmCfg {
   static constexpr int KK = sizeof(T) == 2 ? 4 : 1;   // 16-deep K steps per stage
   static constexpr int BK = 16 * KK;
-  static constexpr int U = KK == 1 ? 2 : KK;          // K steps per loop trip (even: register sets alternate)
   static constexpr int NF = 16 * KK;                  // fragments per stage (a: 8 row blocks, b: 8)
   static constexpr int FPW = NF / 4;                  // fragments each wave moves per stage
   static constexpr int VE = 16 / (int)sizeof(T);      // elements per 16-byte vector
@@ -50,7 +48,7 @@ __global__ __launch_bounds__(256) void nt_gemm_batched_kernel(const T* __restric
   typedef typename Vec8<T>::type V8;
   typedef typename Vec4<T>::type V4;
   typedef GemmCfg<T> G;
-  constexpr int KK = G::KK, BK = G::BK, U = G::U, FPW = G::FPW;
+  constexpr int KK = G::KK, BK = G::BK, FPW = G::FPW;
   __shared__ V8 lds_f[2][G::NF][kWave];   // [buffer][operand*8*KK + row block*KK + kk][lane]
   __shared__ __attribute__((aligned(16))) T lds_stage[4][32 * G::PITCH];
 
@@ -67,7 +65,7 @@ __global__ __launch_bounds__(256) void nt_gemm_batched_kernel(const T* __restric
 
   const int n_rb = (n + 31) >> 5;          // row blocks per channel
   const int n_ks = k_pitch >> 4;           // K steps per row block
-  const int n_stages = (n + BK - 1) / BK;
+  const int n_stages = k_pitch / BK;        // K padding up to k_pitch holds zeros
 
   // The fragments this wave moves global -> LDS each stage: ids wave*FPW .. +FPW-1, in
   // runs of KK consecutive K steps of one row block (consecutive in memory).
@@ -80,26 +78,25 @@ __global__ __launch_bounds__(256) void nt_gemm_batched_kernel(const T* __restric
     src[q] = (op ? b : a) + trimul_frag_offset(c, rb, 0, n_rb, n_ks) + lane * 8;
   }
 
-  V8 pre[FPW];
-  auto fetch = [&](int stage) {   // issues loads only; the stage index is clamped for the address
-    const int ks0 = min(stage, n_stages - 1) * KK;
+  // Loads are issued two stages ahead of their LDS write (HBM latency under load exceeds one
+  // stage of MFMA work) into two register sets that alternate by stage parity.  Everything
+  // is spread evenly over the K steps of a stage so that no queue sees a burst: step kk
+  // issues the loads of K step kk of stage + 2, and steps 0 .. KK-2 each write a share of
+  // stage + 1 into the LDS buffer that the barrier of the previous stage's last step freed.
+  V8 pre0[FPW], pre1[FPW];
+  auto fetch_part = [&](int stage, int kk, V8 (&pre)[FPW]) {   // stage clamped for the address
+    const int ks = min(stage, n_stages - 1) * KK + kk;
 #pragma unroll
-    for (int q = 0; q < FPW / KK; ++q)
-#pragma unroll
-      for (int kk = 0; kk < KK; ++kk) pre[q * KK + kk] = load8<T>(src[q] + (int64_t)(ks0 + kk) * 512);
+    for (int q = 0; q < FPW / KK; ++q) pre[q * KK + kk] = load8<T>(src[q] + (int64_t)ks * 512);
   };
-  auto stash = [&](int stage) {   // K slots beyond n (row padding, phantom stages) become zero
-    const int buf = stage & 1;
-    if (stage * BK + BK > n) {    // uniform
+  // share `part` of `parts`: fragments in the order their loads were issued (K step major),
+  // so every fragment has been in flight for at least KK - 1 steps when it is written
+  auto stash_part = [&](int stage, int part, int parts, V8 (&pre)[FPW]) {
 #pragma unroll
-      for (int f = 0; f < FPW; ++f) {
-        const int kbase = stage * BK + 16 * (f % KK) + 8 * g;
-#pragma unroll
-        for (int t = 0; t < 8; ++t) pre[f][t] = kbase + t < n ? pre[f][t] : (T)0.0f;
-      }
+    for (int f = 0; f < FPW; ++f) {
+      const int order = (f % KK) * (FPW / KK) + f / KK;
+      if (order * parts / FPW == part) lds_f[stage & 1][wave * FPW + f][lane] = pre[f];
     }
-#pragma unroll
-    for (int f = 0; f < FPW; ++f) lds_f[buf][wave * FPW + f][lane] = pre[f];
   };
   // fragments of one K step: this wave's 4 row blocks of a and 4 of b
   auto read_frags = [&](int buf, int kk, V8 (&af)[4], V8 (&bf)[4]) {
@@ -117,46 +114,66 @@ __global__ __launch_bounds__(256) void nt_gemm_batched_kernel(const T* __restric
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[rb][jb][r] = 0.0f;
 
-  // A operand = b rows (register <-> j), B operand = a rows (lane <-> i)
-  auto mma_half = [&](int half, V8 (&af)[4], V8 (&bf)[4]) {
-#pragma unroll
-    for (int rb = 2 * half; rb < 2 * half + 2; ++rb)
-#pragma unroll
-      for (int jb = 0; jb < 4; ++jb) mma32(acc[rb][jb], bf[jb], af[rb]);
-  };
-
-  // One K step.  `cur` holds its fragments; `nxt` receives the following step's.
+  // One K step.  `cur` holds its fragments; `nxt` receives the following step's.  `p_in` takes
+  // the loads of stage + 2, `p_out` holds stage + 1.
   auto k_step = [&](int stage, int kk, V8 (&a_cur)[4], V8 (&b_cur)[4], V8 (&a_nxt)[4],
-                    V8 (&b_nxt)[4]) {
-    if (kk == 0) fetch(stage + 1);
-    mma_half(0, a_cur, b_cur);
-    __builtin_amdgcn_sched_barrier(0);
-    if (kk == KK - 1) {
-      // every wave finished reading buffer (stage+1)&1 before the previous barrier
-      stash(stage + 1);
-      __syncthreads();
-      read_frags((stage + 1) & 1, 0, a_nxt, b_nxt);
-    } else {
-      read_frags(stage & 1, kk + 1, a_nxt, b_nxt);
+                    V8 (&b_nxt)[4], V8 (&p_in)[FPW], V8 (&p_out)[FPW]) {
+    if (KK == 1) stash_part(stage + 1, 0, 1, p_out);
+    // all shares of stage + 1 are in LDS once every wave passes here; nobody still reads
+    // the other buffer's previous contents after the barrier one stage earlier
+    if (kk == KK - 1) __syncthreads();
+    if (kk == KK - 1) read_frags((stage + 1) & 1, 0, a_nxt, b_nxt);
+    else read_frags(stage & 1, kk + 1, a_nxt, b_nxt);
+    fetch_part(stage + 2, kk, p_in);
+    if (KK > 1 && kk < KK - 1) stash_part(stage + 1, kk, KK - 1, p_out);
+    // A operand = b rows (register <-> j), B operand = a rows (lane <-> i)
+#pragma unroll
+    for (int rb = 0; rb < 4; ++rb)
+#pragma unroll
+      for (int jb = 0; jb < 4; ++jb) mma32(acc[rb][jb], b_cur[jb], a_cur[rb]);
+    if constexpr (sizeof(T) == 2) {
+      // issue order: 2 MFMAs, then one LDS read, one global load (first 4 groups) and one
+      // LDS write (first 6 groups)
+#pragma unroll
+      for (int grp = 0; grp < 8; ++grp) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        if (grp < 4) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+        if (grp < 6) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+      }
     }
-    __builtin_amdgcn_sched_barrier(0);
-    mma_half(1, a_cur, b_cur);
+  };
+  auto stage_steps = [&](int stage, V8 (&p_in)[FPW], V8 (&p_out)[FPW], V8 (&a_c)[4], V8 (&b_c)[4],
+                         V8 (&a_n)[4], V8 (&b_n)[4]) {
+    // KK is 1 or even: with KK even a stage starts and ends on the same fragment set
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+      if ((kk & 1) == 0) k_step(stage, kk, a_c, b_c, a_n, b_n, p_in, p_out);
+      else k_step(stage, kk, a_n, b_n, a_c, b_c, p_in, p_out);
+    }
   };
 
   V8 a0[4], b0[4], a1[4], b1[4];
-  fetch(0);
-  stash(0);
+#pragma unroll
+  for (int kk = 0; kk < KK; ++kk) fetch_part(0, kk, pre0);
+#pragma unroll
+  for (int kk = 0; kk < KK; ++kk) fetch_part(1, kk, pre1);
+  stash_part(0, 0, 1, pre0);
   __syncthreads();
   read_frags(0, 0, a0, b0);
-  // U K steps per trip; stages past the end (when KK == 1 and n_stages is odd) add zeros
-  const int n_steps = n_stages * KK;
-  for (int t0 = 0; t0 < n_steps; t0 += U) {
-#pragma unroll
-    for (int u = 0; u < U; u += 2) {
-      k_step(t0 / KK + u / KK, u % KK, a0, b0, a1, b1);
-      k_step(t0 / KK + (u + 1) / KK, (u + 1) % KK, a1, b1, a0, b0);
+  // Two stages per trip (prefetch sets alternate by parity), then a last single stage.  The
+  // last stage's writes and reads for "stage + 1" move valid but unused data.
+  int s0 = 0;
+  for (; s0 + 1 < n_stages; s0 += 2) {
+    if (KK == 1) {
+      stage_steps(s0, pre0, pre1, a0, b0, a1, b1);
+      stage_steps(s0 + 1, pre1, pre0, a1, b1, a0, b0);
+    } else {
+      stage_steps(s0, pre0, pre1, a0, b0, a1, b1);
+      stage_steps(s0 + 1, pre1, pre0, a0, b0, a1, b1);
     }
   }
+  if (s0 < n_stages) stage_steps(s0, pre0, pre1, a0, b0, a1, b1);
 
   // ---- epilogue: lane <-> row i, register quads <-> 4 consecutive j ----
   T* x_c = x + (int64_t)c * n * n;

@@ -289,7 +289,7 @@ __global__ __launch_bounds__(256, (MODE == kTriAttnIn ? 1 : 2)) void rowgemm_in_
   // channel 64 contiguous bytes of the contraction's fragment-ordered operands.
   int pi0 = 0, pk0 = 0;
   if constexpr (MODE == kTriMulIn) {
-    const uint32_t n_kb = (uint32_t)(p.n + 7) >> 3;
+    const uint32_t n_kb = (uint32_t)p.pitch >> 3;   // the K padding is written too (as zeros)
     const uint32_t ip = blockIdx.x / n_kb;
     pk0 = (int)(blockIdx.x - ip * n_kb) * 8;
     pi0 = (int)ip * (16 * RB) + wave * (4 * RB);
@@ -358,17 +358,19 @@ __global__ __launch_bounds__(256, (MODE == kTriAttnIn ? 1 : 2)) void rowgemm_in_
   }
 
   // TriMulIn: the 32 mask values of each row block, shared through LDS
+  // (inner indices between n and the pitch get factor 0: the contraction relies on zeros there)
   if constexpr (MODE == kTriMulIn) {
-    if (p.mask) {
 #pragma unroll
-      for (int rb = 0; rb < RB; ++rb) {
-        const int i = min(pi0 + 4 * rb + (n >> 3), p.n - 1), k = min(pk0 + (n & 7), p.n - 1);
-        const float mv = to_f32(((const T*)p.mask)[(int64_t)i * p.mmap.stride_outer +
-                                                   (int64_t)k * p.mmap.stride_inner]);
-        if (g == 0) lds_mask[wave][rb * 32 + n] = mv;
-      }
-      wave_lds_sync();
+    for (int rb = 0; rb < RB; ++rb) {
+      const int i = min(pi0 + 4 * rb + (n >> 3), p.n - 1), k = min(pk0 + (n & 7), p.n - 1);
+      float mv = 1.0f;
+      if (p.mask)
+        mv = to_f32(((const T*)p.mask)[(int64_t)i * p.mmap.stride_outer +
+                                       (int64_t)k * p.mmap.stride_inner]);
+      if (pk0 + (n & 7) >= p.n) mv = 0.0f;
+      if (g == 0) lds_mask[wave][rb * 32 + n] = mv;
     }
+    wave_lds_sync();
   }
 
   // Row-major destinations (kTriAttnIn q/k/g, kTransitionIn hidden, kTriMulOut out): the
@@ -497,9 +499,7 @@ __global__ __launch_bounds__(256, (MODE == kTriAttnIn ? 1 : 2)) void rowgemm_in_
         float vals[16];
 #pragma unroll
         for (int qd = 0; qd < 4; ++qd) {
-          f32x4 m4 = {1.0f, 1.0f, 1.0f, 1.0f};
-          if (p.mask)
-            m4 = *reinterpret_cast<const f32x4*>(&lds_mask[wave][rb * 32 + 8 * qd + 4 * g]);
+          const f32x4 m4 = *reinterpret_cast<const f32x4*>(&lds_mask[wave][rb * 32 + 8 * qd + 4 * g]);
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
             const int r = 4 * qd + e;
@@ -699,7 +699,7 @@ int launch_rowgemm_in(const RowGemmInParams& p, hipStream_t stream) {
   const int64_t rows_per_block = 4 * RB * 32;
   int64_t blocks = (p.n_rows + rows_per_block - 1) / rows_per_block;
   if (MODE == kTriMulIn)   // 2-D patches: 16*RB outer x 8 inner indices per workgroup
-    blocks = (int64_t)((p.n + 16 * RB - 1) / (16 * RB)) * ((p.n + 7) / 8);
+    blocks = (int64_t)((p.n + 16 * RB - 1) / (16 * RB)) * (p.pitch / 8);
   if (blocks == 0) return 0;
   rowgemm_in_kernel<T, RB, MODE><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(p);
   return 0;
