@@ -10,12 +10,14 @@
 //
 // Workgroup = 4 waves (2 x 2), tile 256 (i) x 256 (j); a wave owns 128 x 128:
 // 4 x 4 accumulator tiles of 32 x 32 (256 accumulator registers, one wave per
-// SIMD), so each fragment read from LDS feeds 4 MFMAs.  A K stage (KK steps of
-// 16) of both operand panels is staged through LDS, double-buffered.  The wave
-// is software-pipelined by hand, because with one wave per SIMD nothing else
-// hides latency: the fragments of K step t+1 are read from LDS under step t's
-// MFMAs, global loads are issued two stages before they are written to LDS, and
-// loads, LDS writes and LDS reads are spread evenly between the MFMAs.
+// SIMD), so each fragment read from LDS feeds 4 MFMAs.  K stages (KK steps of
+// 16) of both operand panels travel global -> LDS with direct-to-LDS loads
+// (global_load_lds_dwordx4: no registers, no LDS write instructions) into a
+// ring of 4 stage buffers, issued three stages ahead of their use: concurrent
+// tiles of one channel walk K in lockstep, so every load sees HBM latency.
+// With one wave per SIMD nothing else hides latency, so the wave is pipelined by
+// hand: the fragments of K step t+1 are read from LDS under step t's MFMAs, and
+// loads and LDS reads are spread evenly between the MFMAs.
 //
 // MFMA operands are ordered so that a lane ends up holding 4 consecutive j per
 // register quad of one row i: results leave through a per-wave LDS tile as
@@ -29,16 +31,46 @@
 namespace ptx {
 
 template <typename T> struct GemmCfg {
-  static constexpr int KK = sizeof(T) == 2 ? 4 : 1;   // 16-deep K steps per stage
+  static constexpr int KK = sizeof(T) == 2 ? 2 : 1;   // 16-deep K steps per stage
   static constexpr int BK = 16 * KK;
+  static constexpr int NBUF = 4;                      // LDS stage buffers (loads run 3 stages ahead)
+  static constexpr int PIECES = (int)sizeof(T) / 2;   // 16-byte pieces per lane and fragment
   static constexpr int NF = 16 * KK;                  // fragments per stage (a: 8 row blocks, b: 8)
-  static constexpr int FPW = NF / 4;                  // fragments each wave moves per stage
+  static constexpr int RUNS = 4;                      // (operand, row block) runs each wave moves
+  static constexpr int DMA_PER_STEP = RUNS * PIECES;  // direct-to-LDS loads a wave issues per K step
   static constexpr int VE = 16 / (int)sizeof(T);      // elements per 16-byte vector
   static constexpr int LPM = 32 / VE;                 // lanes per 32-long row of the staging tile
   static constexpr int MPP = kWave / LPM;             // rows per read-back pass
   static constexpr int NPASS = 32 / MPP;
   static constexpr int PITCH = 32 + 8 / (int)sizeof(T);   // staging row pitch, 8-byte aligned rows
 };
+
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;
+
+// Direct-to-LDS load: every lane moves 16 bytes from its own global address to LDS address
+// lds_base + 16 * lane (M0 carries the base).  Issued as inline asm on purpose: for
+// direct-to-LDS loads it knows about, the compiler waits for ALL of them (vmcnt(0)) before
+// any later LDS read, which would serialise a ring whose loads run stages ahead.  The
+// waits are placed by hand in ring_barrier() instead.
+__device__ __forceinline__ void load_to_lds16(const void* gptr, uint32_t lds_base) {
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+               :
+               : "v"(gptr), "s"(lds_base)
+               : "m0");
+}
+// LDS byte address of p, which must be the same for all lanes (it goes to a scalar register)
+__device__ __forceinline__ uint32_t lds_address(const void* p) {
+  return __builtin_amdgcn_readfirstlane(
+      (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void*)p);
+}
+
+// Workgroup barrier for the stage ring: wait until all but the N youngest direct-to-LDS
+// loads of this wave have landed and all its LDS reads have returned, then s_barrier.
+// The memory clobbers keep the compiler from moving LDS accesses across the barrier.
+template <int N> __device__ __forceinline__ void ring_barrier() {
+  static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+  asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(N) : "memory");
+}
 
 template <typename T>
 __global__ __launch_bounds__(256) void nt_gemm_batched_kernel(const T* __restrict__ a,
@@ -48,8 +80,9 @@ __global__ __launch_bounds__(256) void nt_gemm_batched_kernel(const T* __restric
   typedef typename Vec8<T>::type V8;
   typedef typename Vec4<T>::type V4;
   typedef GemmCfg<T> G;
-  constexpr int KK = G::KK, BK = G::BK, FPW = G::FPW;
-  __shared__ V8 lds_f[2][G::NF][kWave];   // [buffer][operand*8*KK + row block*KK + kk][lane]
+  constexpr int KK = G::KK, BK = G::BK, NBUF = G::NBUF, PIECES = G::PIECES, RUNS = G::RUNS;
+  // [buffer][operand*8*KK + row block*KK + kk][16-byte piece][lane]
+  __shared__ u32x4_t lds_f[NBUF][G::NF][PIECES][kWave];
   __shared__ __attribute__((aligned(16))) T lds_stage[4][32 * G::PITCH];
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -65,45 +98,45 @@ __global__ __launch_bounds__(256) void nt_gemm_batched_kernel(const T* __restric
 
   const int n_rb = (n + 31) >> 5;          // row blocks per channel
   const int n_ks = k_pitch >> 4;           // K steps per row block
-  const int n_stages = k_pitch / BK;        // K padding up to k_pitch holds zeros
+  const int n_stages = k_pitch / BK;       // K padding up to k_pitch holds zeros
 
-  // The fragments this wave moves global -> LDS each stage: ids wave*FPW .. +FPW-1, in
-  // runs of KK consecutive K steps of one row block (consecutive in memory).
-  const T* src[FPW / KK];
+  // The fragments this wave moves global -> LDS each stage: RUNS runs of KK consecutive K
+  // steps of one (operand, row block), consecutive in memory.  Lane address of piece 0.
+  const T* src[RUNS];
 #pragma unroll
-  for (int q = 0; q < FPW / KK; ++q) {
-    const int run = wave * (FPW / KK) + q;        // 0..15: operand = run / 8, row block = run % 8
+  for (int q = 0; q < RUNS; ++q) {
+    const int run = wave * RUNS + q;              // 0..15: operand = run / 8, row block = run % 8
     const int op = run >> 3;
     const int rb = min((op ? tj : ti) * 8 + (run & 7), n_rb - 1);   // blocks past the end re-read the last
     src[q] = (op ? b : a) + trimul_frag_offset(c, rb, 0, n_rb, n_ks) + lane * 8;
   }
 
-  // Loads are issued two stages ahead of their LDS write (HBM latency under load exceeds one
-  // stage of MFMA work) into two register sets that alternate by stage parity.  Everything
-  // is spread evenly over the K steps of a stage so that no queue sees a burst: step kk
-  // issues the loads of K step kk of stage + 2, and steps 0 .. KK-2 each write a share of
-  // stage + 1 into the LDS buffer that the barrier of the previous stage's last step freed.
-  V8 pre0[FPW], pre1[FPW];
-  auto fetch_part = [&](int stage, int kk, V8 (&pre)[FPW]) {   // stage clamped for the address
+  // Direct-to-LDS loads of K step kk of `stage` (clamped for the address): each moves 16
+  // bytes per lane to consecutive LDS slots, which is the fragment image itself.
+  auto dma_part = [&](int stage, int kk) {
     const int ks = min(stage, n_stages - 1) * KK + kk;
+    const int buf = stage & (NBUF - 1);
 #pragma unroll
-    for (int q = 0; q < FPW / KK; ++q) pre[q * KK + kk] = load8<T>(src[q] + (int64_t)ks * 512);
+    for (int q = 0; q < RUNS; ++q)
+#pragma unroll
+      for (int pc = 0; pc < PIECES; ++pc)
+        load_to_lds16(src[q] + (int64_t)ks * 512 + pc * G::VE,
+                      lds_address(&lds_f[buf][(wave * RUNS + q) * KK + kk][pc][0]));
   };
-  // share `part` of `parts`: fragments in the order their loads were issued (K step major),
-  // so every fragment has been in flight for at least KK - 1 steps when it is written
-  auto stash_part = [&](int stage, int part, int parts, V8 (&pre)[FPW]) {
+  auto read_one = [&](int buf, int frag) {
+    V8 v;
+    u32x4_t* d = reinterpret_cast<u32x4_t*>(&v);
 #pragma unroll
-    for (int f = 0; f < FPW; ++f) {
-      const int order = (f % KK) * (FPW / KK) + f / KK;
-      if (order * parts / FPW == part) lds_f[stage & 1][wave * FPW + f][lane] = pre[f];
-    }
+    for (int pc = 0; pc < PIECES; ++pc) d[pc] = lds_f[buf][frag][pc][lane];
+    return v;
   };
   // fragments of one K step: this wave's 4 row blocks of a and 4 of b
-  auto read_frags = [&](int buf, int kk, V8 (&af)[4], V8 (&bf)[4]) {
+  auto read_frags = [&](int stage, int kk, V8 (&af)[4], V8 (&bf)[4]) {
+    const int buf = stage & (NBUF - 1);
 #pragma unroll
-    for (int r = 0; r < 4; ++r) af[r] = lds_f[buf][(wi * 4 + r) * KK + kk][lane];
+    for (int r = 0; r < 4; ++r) af[r] = read_one(buf, (wi * 4 + r) * KK + kk);
 #pragma unroll
-    for (int r = 0; r < 4; ++r) bf[r] = lds_f[buf][(8 + wj * 4 + r) * KK + kk][lane];
+    for (int r = 0; r < 4; ++r) bf[r] = read_one(buf, (8 + wj * 4 + r) * KK + kk);
   };
 
   f32x16 acc[4][4];   // [row block of a][row block of b]
@@ -114,66 +147,52 @@ __global__ __launch_bounds__(256) void nt_gemm_batched_kernel(const T* __restric
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[rb][jb][r] = 0.0f;
 
-  // One K step.  `cur` holds its fragments; `nxt` receives the following step's.  `p_in` takes
-  // the loads of stage + 2, `p_out` holds stage + 1.
+  // One K step.  `cur` holds its fragments; `nxt` receives the following step's.
+  //   Buffer use: stage s is computed from buffer s % 4 while the loads of stage s + 3 land
+  // in buffer (s + 3) % 4, whose last readers (stage s - 1) finished before the barrier in
+  // stage s - 1's last step.  Before that barrier each wave waits until its own loads of the
+  // next stage have landed: loads complete in issue order, and the only younger ones are
+  // those of stage s + 2 and the part of stage s + 3 issued so far.
   auto k_step = [&](int stage, int kk, V8 (&a_cur)[4], V8 (&b_cur)[4], V8 (&a_nxt)[4],
-                    V8 (&b_nxt)[4], V8 (&p_in)[FPW], V8 (&p_out)[FPW]) {
-    if (KK == 1) stash_part(stage + 1, 0, 1, p_out);
-    // all shares of stage + 1 are in LDS once every wave passes here; nobody still reads
-    // the other buffer's previous contents after the barrier one stage earlier
-    if (kk == KK - 1) __syncthreads();
-    if (kk == KK - 1) read_frags((stage + 1) & 1, 0, a_nxt, b_nxt);
-    else read_frags(stage & 1, kk + 1, a_nxt, b_nxt);
-    fetch_part(stage + 2, kk, p_in);
-    if (KK > 1 && kk < KK - 1) stash_part(stage + 1, kk, KK - 1, p_out);
+                    V8 (&b_nxt)[4]) {
+    if (kk == KK - 1) {
+      ring_barrier<G::DMA_PER_STEP * (KK + KK - 1)>();
+      read_frags(stage + 1, 0, a_nxt, b_nxt);
+    } else {
+      read_frags(stage, kk + 1, a_nxt, b_nxt);
+    }
+    dma_part(stage + 3, kk);
     // A operand = b rows (register <-> j), B operand = a rows (lane <-> i)
 #pragma unroll
     for (int rb = 0; rb < 4; ++rb)
 #pragma unroll
       for (int jb = 0; jb < 4; ++jb) mma32(acc[rb][jb], b_cur[jb], a_cur[rb]);
     if constexpr (sizeof(T) == 2) {
-      // issue order: 2 MFMAs, then one LDS read, one global load (first 4 groups) and one
-      // LDS write (first 6 groups)
+      // issue order: 2 MFMAs, then one LDS read
 #pragma unroll
       for (int grp = 0; grp < 8; ++grp) {
         __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
         __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-        if (grp < 4) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
-        if (grp < 6) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
       }
-    }
-  };
-  auto stage_steps = [&](int stage, V8 (&p_in)[FPW], V8 (&p_out)[FPW], V8 (&a_c)[4], V8 (&b_c)[4],
-                         V8 (&a_n)[4], V8 (&b_n)[4]) {
-    // KK is 1 or even: with KK even a stage starts and ends on the same fragment set
-#pragma unroll
-    for (int kk = 0; kk < KK; ++kk) {
-      if ((kk & 1) == 0) k_step(stage, kk, a_c, b_c, a_n, b_n, p_in, p_out);
-      else k_step(stage, kk, a_n, b_n, a_c, b_c, p_in, p_out);
     }
   };
 
   V8 a0[4], b0[4], a1[4], b1[4];
 #pragma unroll
-  for (int kk = 0; kk < KK; ++kk) fetch_part(0, kk, pre0);
+  for (int st0 = 0; st0 < 3; ++st0)
 #pragma unroll
-  for (int kk = 0; kk < KK; ++kk) fetch_part(1, kk, pre1);
-  stash_part(0, 0, 1, pre0);
-  __syncthreads();
+    for (int kk = 0; kk < KK; ++kk) dma_part(st0, kk);
+  ring_barrier<G::DMA_PER_STEP * KK * 2>();
   read_frags(0, 0, a0, b0);
-  // Two stages per trip (prefetch sets alternate by parity), then a last single stage.  The
-  // last stage's writes and reads for "stage + 1" move valid but unused data.
-  int s0 = 0;
-  for (; s0 + 1 < n_stages; s0 += 2) {
-    if (KK == 1) {
-      stage_steps(s0, pre0, pre1, a0, b0, a1, b1);
-      stage_steps(s0 + 1, pre1, pre0, a1, b1, a0, b0);
-    } else {
-      stage_steps(s0, pre0, pre1, a0, b0, a1, b1);
-      stage_steps(s0 + 1, pre1, pre0, a0, b0, a1, b1);
-    }
+  // Two K steps per trip (the fragment sets alternate); the number of K steps is even.
+  const int n_steps = n_stages * KK;
+  for (int t0 = 0; t0 < n_steps; t0 += 2) {
+    k_step(t0 / KK, 0, a0, b0, a1, b1);
+    k_step((t0 + 1) / KK, (t0 + 1) % KK, a1, b1, a0, b0);
   }
-  if (s0 < n_stages) stage_steps(s0, pre0, pre1, a0, b0, a1, b1);
+
+  // the loads issued for stages past the end are still in flight: let them land
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
   // ---- epilogue: lane <-> row i, register quads <-> 4 consecutive j ----
   T* x_c = x + (int64_t)c * n * n;
