@@ -169,15 +169,23 @@ PTX_API int ptx_triattn_output(const void* o, const void* w_o, const void* z, vo
                        int c_in, int transposed, int add_residual, int dtype, void* stream);
 
 /*
- * Transition (primitives.py:190-230):
+ * Transition (primitives.py:190-230), one fused kernel:
  *   out = [x +] W_o ( silu(W_a LN(x)) * (W_b LN(x)) )
- *   x, out [rows][c] (out may alias x), w_a, w_b [n_factor*c][c], w_o [c][n_factor*c],
- *   hidden: caller-provided workspace [rows][n_factor*c].   c = 128.
+ * The hidden activations stay on chip, so there is no workspace; instead the three
+ * weight matrices are packed once per weight set into the kernel's streaming order
+ * (MFMA operand fragments, grouped in chunks of 32 hidden channels):
+ *   ptx_transition_pack:  w_a, w_b [n_factor*c][c], w_o [c][n_factor*c]  ->
+ *     packed, ptx_transition_packed_elems(c, n_factor) = 3*n_factor*c*c elements.
+ *   ptx_transition_fwd:   x, out [rows][c] (out may alias x), ln_w / ln_b may be NULL.
+ * a and b stay in fp32 through the activation (the reference rounds them to the
+ * storage dtype first); the product is rounded once.   c = 128.
  */
-PTX_API int ptx_transition_fwd(const void* x, const void* ln_w, const void* ln_b, const void* w_a,
-                       const void* w_b, const void* w_o, void* hidden, void* out, int64_t rows,
-                       int c, int n_factor, int add_residual, float eps, int dtype,
-                       void* stream);
+PTX_API int64_t ptx_transition_packed_elems(int c, int n_factor);
+PTX_API int ptx_transition_pack(const void* w_a, const void* w_b, const void* w_o, void* packed, int c,
+                        int n_factor, int dtype, void* stream);
+PTX_API int ptx_transition_fwd(const void* x, const void* ln_w, const void* ln_b, const void* packed,
+                       void* out, int64_t rows, int c, int n_factor, int add_residual, float eps,
+                       int dtype, void* stream);
 
 /*
  * Pair bias of the single-representation attention (transformer.py:191-194):

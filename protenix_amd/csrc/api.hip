@@ -212,25 +212,41 @@ PTX_API int ptx_triattn_output(const void* o, const void* w_o, const void* z, vo
   return after_launch("triattn_output");
 }
 
-PTX_API int ptx_transition_fwd(const void* x, const void* ln_w, const void* ln_b, const void* w_a,
-                       const void* w_b, const void* w_o, void* hidden, void* out, int64_t rows,
-                       int c, int n_factor, int add_residual, float eps, int dtype,
-                       void* stream) {
+PTX_API int64_t ptx_transition_packed_elems(int c, int n_factor) {
+  if (c <= 0 || n_factor <= 0) return 0;
+  return (int64_t)3 * n_factor * c * c;
+}
+
+PTX_API int ptx_transition_pack(const void* w_a, const void* w_b, const void* w_o, void* packed, int c,
+                        int n_factor, int dtype, void* stream) {
+  PTX_REQUIRE(dtype_ok(dtype), PTX_ERR_BAD_ARG, "transition_pack: unknown dtype %d", dtype);
+  PTX_REQUIRE(n_factor > 0, PTX_ERR_BAD_ARG, "transition_pack: n_factor=%d", n_factor);
+  PTX_REQUIRE(c == 128, PTX_ERR_UNSUPPORTED, "transition_pack: only c=128 is built (got %d)", c);
+  PTX_REQUIRE(n_factor <= 64, PTX_ERR_UNSUPPORTED, "transition_pack: n_factor=%d too large",
+              n_factor);
+  PTX_REQUIRE(w_a && w_b && w_o && packed, PTX_ERR_BAD_ARG, "transition_pack: null pointer");
+  PTX_REQUIRE(aligned16(packed), PTX_ERR_BAD_ARG, "transition_pack: packed must be 16-byte aligned");
+  PTX_DISPATCH(dtype, ptx::transition_pack<T>(w_a, w_b, w_o, packed, n_factor, (hipStream_t)stream));
+  return after_launch("transition_pack");
+}
+
+PTX_API int ptx_transition_fwd(const void* x, const void* ln_w, const void* ln_b, const void* packed,
+                       void* out, int64_t rows, int c, int n_factor, int add_residual, float eps,
+                       int dtype, void* stream) {
   PTX_REQUIRE(dtype_ok(dtype), PTX_ERR_BAD_ARG, "transition: unknown dtype %d", dtype);
   PTX_REQUIRE(rows >= 0 && n_factor > 0, PTX_ERR_BAD_ARG, "transition: rows=%lld n_factor=%d",
               (long long)rows, n_factor);
   PTX_REQUIRE(c == 128, PTX_ERR_UNSUPPORTED, "transition: only c=128 is built (got %d)", c);
+  PTX_REQUIRE(n_factor <= 64, PTX_ERR_UNSUPPORTED, "transition: n_factor=%d too large", n_factor);
   PTX_REQUIRE(rows < ((int64_t)1 << 30), PTX_ERR_UNSUPPORTED, "transition: rows=%lld too large",
               (long long)rows);
   if (rows == 0) return PTX_OK;
-  PTX_REQUIRE(x && w_a && w_b && w_o && hidden && out, PTX_ERR_BAD_ARG,
-              "transition: null pointer");
-  PTX_REQUIRE(aligned16(x) && aligned16(w_a) && aligned16(w_b) && aligned16(w_o) &&
-                  aligned16(hidden) && aligned16(out) && (!ln_w || aligned16(ln_w)) &&
+  PTX_REQUIRE(x && packed && out, PTX_ERR_BAD_ARG, "transition: null pointer");
+  PTX_REQUIRE(aligned16(x) && aligned16(packed) && aligned16(out) && (!ln_w || aligned16(ln_w)) &&
                   (!ln_b || aligned16(ln_b)),
               PTX_ERR_BAD_ARG, "transition: pointers must be 16-byte aligned");
-  PTX_DISPATCH(dtype, ptx::transition_fwd<T>(x, ln_w, ln_b, w_a, w_b, w_o, hidden, out, rows,
-                                             n_factor, add_residual, eps, (hipStream_t)stream));
+  PTX_DISPATCH(dtype, ptx::transition_fwd<T>(x, ln_w, ln_b, packed, out, rows, n_factor,
+                                             add_residual, eps, (hipStream_t)stream));
   return after_launch("transition");
 }
 

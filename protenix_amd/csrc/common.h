@@ -91,6 +91,38 @@ __device__ __forceinline__ typename Vec8<T>::type zero8() {
   return z;
 }
 
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;
+
+// Direct-to-LDS load: every lane moves 16 bytes from its own global address to LDS address
+// lds_base + 16 * lane (M0 carries the base).  Issued as inline asm on purpose: for
+// direct-to-LDS loads it knows about, the compiler waits for ALL of them (vmcnt(0)) before
+// any later LDS read, which would serialise a ring whose loads run stages ahead.  The
+// waits are placed by hand in ring_barrier() instead.
+// (M0 is a reserved register, which the compiler warns about in a clobber list; the
+// clobber is what tells it to re-initialise M0 before its own next use.)
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
+__device__ __forceinline__ void load_to_lds16(const void* gptr, uint32_t lds_base) {
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+               :
+               : "v"(gptr), "s"(lds_base)
+               : "m0");
+}
+#pragma clang diagnostic pop
+// LDS byte address of p, which must be the same for all lanes (it goes to a scalar register)
+__device__ __forceinline__ uint32_t lds_address(const void* p) {
+  return __builtin_amdgcn_readfirstlane(
+      (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void*)p);
+}
+
+// Workgroup barrier for the stage ring: wait until all but the N youngest direct-to-LDS
+// loads of this wave have landed and all its LDS reads have returned, then s_barrier.
+// The memory clobbers keep the compiler from moving LDS accesses across the barrier.
+template <int N> __device__ __forceinline__ void ring_barrier() {
+  static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+  asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(N) : "memory");
+}
+
 // Position of a logical pair-tensor row p = outer * n_inner + inner in a tensor
 // whose (outer, inner) axes have arbitrary element strides.  The ending-node
 // attention and the incoming triangle product read z[inner, outer] this way,

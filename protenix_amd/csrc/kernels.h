@@ -26,10 +26,14 @@ int triattn_project(const void* z, const void* ln_w, const void* ln_b, const voi
 template <typename T>
 int triattn_output(const void* o, const void* w_o, const void* z, void* out, int n, int transposed,
                    int add_residual, hipStream_t stream);
+// transition weights -> fragment-ordered chunks of 32 hidden (3 * n_factor*128 * 128 elements)
 template <typename T>
-int transition_fwd(const void* x, const void* ln_w, const void* ln_b, const void* w_a,
-                   const void* w_b, const void* w_o, void* hidden, void* out, int64_t rows,
-                   int n_factor, int add_residual, float eps, hipStream_t stream);
+int transition_pack(const void* w_a, const void* w_b, const void* w_o, void* packed, int n_factor,
+                    hipStream_t stream);
+template <typename T>
+int transition_fwd(const void* x, const void* ln_w, const void* ln_b, const void* packed,
+                   void* out, int64_t rows, int n_factor, int add_residual, float eps,
+                   hipStream_t stream);
 template <typename T>
 int pair_bias_fwd(const void* z, const void* ln_w, const void* ln_b, const void* w, void* bias,
                   int n, int heads, int out_f32, float eps, hipStream_t stream);

@@ -45,33 +45,6 @@ template <typename T> struct GemmCfg {
   static constexpr int PITCH = 32 + 8 / (int)sizeof(T);   // staging row pitch, 8-byte aligned rows
 };
 
-typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;
-
-// Direct-to-LDS load: every lane moves 16 bytes from its own global address to LDS address
-// lds_base + 16 * lane (M0 carries the base).  Issued as inline asm on purpose: for
-// direct-to-LDS loads it knows about, the compiler waits for ALL of them (vmcnt(0)) before
-// any later LDS read, which would serialise a ring whose loads run stages ahead.  The
-// waits are placed by hand in ring_barrier() instead.
-__device__ __forceinline__ void load_to_lds16(const void* gptr, uint32_t lds_base) {
-  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
-               :
-               : "v"(gptr), "s"(lds_base)
-               : "m0");
-}
-// LDS byte address of p, which must be the same for all lanes (it goes to a scalar register)
-__device__ __forceinline__ uint32_t lds_address(const void* p) {
-  return __builtin_amdgcn_readfirstlane(
-      (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void*)p);
-}
-
-// Workgroup barrier for the stage ring: wait until all but the N youngest direct-to-LDS
-// loads of this wave have landed and all its LDS reads have returned, then s_barrier.
-// The memory clobbers keep the compiler from moving LDS accesses across the barrier.
-template <int N> __device__ __forceinline__ void ring_barrier() {
-  static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
-  asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(N) : "memory");
-}
-
 template <typename T>
 __global__ __launch_bounds__(256) void nt_gemm_batched_kernel(const T* __restrict__ a,
                                                               const T* __restrict__ b,

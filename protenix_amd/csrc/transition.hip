@@ -1,0 +1,268 @@
+// Transition (SwiGLU feed-forward) on rows of 128 channels, one kernel:
+//   out = [x +] W_o ( silu(W_a LN(x)) * (W_b LN(x)) ),   W_a, W_b [128*n_factor][128]
+// The hidden activations (n_factor * 128 per row) never leave the chip: a wave
+// keeps its rows as MFMA operand fragments, walks the hidden dimension in chunks
+// of 32 and accumulates the output projection as it goes.
+//
+//   GEMM1 (per chunk): h^T[32 hidden x 32 rows] = W[32 x 128] * LN(x)^T, so a lane ends up
+//     with one row and 16 hidden values in its accumulator registers;
+//   activation in registers, rounded to T;
+//   GEMM2: out^T[128 x 32 rows] += W_o[:, chunk] * h^T.  Registers 8u .. 8u+7 of a lane are
+//     used directly as the K slots of K step u: which hidden index a slot stands for is
+//     free as long as both operands agree, and the packed W_o fragments follow the
+//     accumulator's register order (no shuffles, no LDS round trip).
+//
+// Weights are packed once (transition_pack) into MFMA fragment order, chunk by
+// chunk, and stream global -> LDS with direct-to-LDS loads into a ring of
+// chunk buffers shared by the workgroup's 4 waves.  One wave per SIMD (the
+// accumulators and the row fragments take ~370 registers), so the wave is
+// pipelined by hand: while the MFMAs of chunk j's GEMM1 run, the VALU computes
+// the activation of chunk j-1, whose GEMM2 follows.
+#include "common.h"
+#include "kernels.h"
+#include "rowtile.h"
+
+namespace ptx {
+
+constexpr int kTrFrags = 24;   // fragments per chunk of 32 hidden: W_a 8 K steps, W_b 8, W_o 4 x 2
+
+template <typename T> struct TrCfg {
+  static constexpr int RB = sizeof(T) == 2 ? 2 : 1;     // row blocks of 32 per wave
+  static constexpr int NBUF = sizeof(T) == 2 ? 4 : 3;   // chunk buffers in LDS
+  static constexpr int D = NBUF - 2;                    // chunks the loads run ahead (two are in use)
+  static constexpr int PIECES = (int)sizeof(T) / 2;     // 16-byte pieces per lane and fragment
+  static constexpr int FPW = kTrFrags / 4;              // fragments each wave moves per chunk
+  static constexpr int DMA_PER_CHUNK = FPW * PIECES;
+};
+
+// packed[chunk j][fragment f][lane][8]:
+//   f <  8: W_a, K step f:      lane (m, g) = W_a[32j + m][16f + 8g .. +7]
+//   f < 16: W_b, K step f - 8
+//   else:   W_o, output block ob = (f-16)/2, K step u = (f-16)%2:
+//           lane (m, g), slot t = W_o[32 ob + m][32j + 8(2u + t/4) + 4g + t%4]
+//           (slot t of K step u <-> accumulator register 8u + t of GEMM1)
+template <typename T>
+__global__ void transition_pack_kernel(const T* __restrict__ w_a, const T* __restrict__ w_b,
+                                       const T* __restrict__ w_o, T* __restrict__ packed,
+                                       int n_hidden) {
+  const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+  const int n_chunks = n_hidden / 32;
+  if (idx >= n_chunks * kTrFrags * kWave) return;
+  const int lane = idx & 63, f = (idx >> 6) % kTrFrags, j = idx / (kWave * kTrFrags);
+  const int m = lane & 31, g = lane >> 5;
+  typename Vec8<T>::type v;
+  if (f < 16) {
+    const T* w = f < 8 ? w_a : w_b;
+    const int kk = f & 7;
+#pragma unroll
+    for (int t = 0; t < 8; ++t) v[t] = w[(int64_t)(32 * j + m) * kC + 16 * kk + 8 * g + t];
+  } else {
+    const int ob = (f - 16) >> 1, u = (f - 16) & 1;
+#pragma unroll
+    for (int t = 0; t < 8; ++t) {
+      const int hidden = 32 * j + 8 * (2 * u + (t >> 2)) + 4 * g + (t & 3);
+      v[t] = w_o[(int64_t)(32 * ob + m) * n_hidden + hidden];
+    }
+  }
+  store8<T>(packed + (int64_t)idx * 8, v);
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void transition_fused_kernel(
+    const T* x, const T* __restrict__ gamma, const T* __restrict__ beta,
+    const T* __restrict__ packed, T* out, int64_t n_rows, int n_chunks, int add_residual,
+    float eps) {
+  typedef typename Vec8<T>::type V8;
+  typedef typename VecE<T>::type VE_t;
+  typedef TrCfg<T> G;
+  typedef Cfg<T> C;
+  constexpr int RB = G::RB, NBUF = G::NBUF, D = G::D, PIECES = G::PIECES, FPW = G::FPW;
+  __shared__ u32x4_t lds_w[NBUF][kTrFrags][PIECES][kWave];
+  static_assert(sizeof(T) * 4 * 32 * C::PITCH <= sizeof(u32x4_t) * kTrFrags * PIECES * kWave,
+                "the staging tiles reuse chunk buffer 0");
+
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t row0 = ((int64_t)blockIdx.x * 4 + wave) * (RB * 32);
+
+  // chunk j (clamped for the address) -> buffer j % NBUF; every wave moves FPW fragments
+  auto dma_chunk = [&](int j) {
+    const int jc = min(j, n_chunks - 1);
+    const int buf = j % NBUF;
+#pragma unroll
+    for (int q = 0; q < FPW; ++q) {
+      const int frag = wave * FPW + q;
+#pragma unroll
+      for (int pc = 0; pc < PIECES; ++pc)
+        load_to_lds16(packed + ((int64_t)jc * kTrFrags + frag) * kFragElems + lane * 8 + pc * C::VE,
+                      lds_address(&lds_w[buf][frag][pc][0]));
+    }
+  };
+  auto read_frag = [&](int buf, int frag) {
+    V8 v;
+    u32x4_t* d = reinterpret_cast<u32x4_t*>(&v);
+#pragma unroll
+    for (int pc = 0; pc < PIECES; ++pc) d[pc] = lds_w[buf][frag][pc][lane];
+    return v;
+  };
+
+  // start the weight ring, then fetch and normalise this wave's rows
+#pragma unroll
+  for (int j = 0; j < D; ++j) dma_chunk(j);
+  RowFrags<T, RB> xf;
+  load_rows<T, RB, true>(xf, x, RowMap{kC, 0, 1}, row0, n_rows, gamma, beta, eps, lane);
+
+  f32x16 acc_o[RB][4];   // [row block][output column block]: lane <-> row, register <-> column
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+    for (int ob = 0; ob < 4; ++ob)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc_o[rb][ob][r] = 0.0f;
+  f32x16 ab0[RB][2], ab1[RB][2];   // GEMM1 accumulators (a, b) of even / odd chunks
+  V8 hf[RB][2];                    // activated hidden values as GEMM2 operand fragments
+
+  auto zero_ab = [&](f32x16 (&ab)[RB][2]) {
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) ab[rb][t][r] = 0.0f;
+  };
+  // K step kk of GEMM1: lane <-> row, register <-> hidden
+  auto gemm1_step = [&](int buf, int kk, f32x16 (&ab)[RB][2]) {
+    const V8 wa = read_frag(buf, kk), wb = read_frag(buf, 8 + kk);
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) {
+      mma32(ab[rb][0], wa, xf.f[rb][kk]);
+      mma32(ab[rb][1], wb, xf.f[rb][kk]);
+    }
+  };
+  // One eighth of a chunk's activation: accumulator registers 2*part, 2*part + 1.
+  // a and b stay in fp32 through the activation; the product is rounded to T once.
+  auto act_part = [&](int part, f32x16 (&ab)[RB][2]) {
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+      for (int e = 0; e < 2; ++e) {
+        const int r = 2 * part + e;
+        const float a = ab[rb][0][r], b = ab[rb][1][r];
+        hf[rb][r >> 3][r & 7] = from_f32<T>(a * b * sigmoidf_fast(a));
+      }
+  };
+  auto gemm2 = [&](int buf) {
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+      for (int ob = 0; ob < 4; ++ob) {
+        const V8 wo = read_frag(buf, 16 + ob * 2 + u);
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) mma32(acc_o[rb][ob], wo, hf[rb][u]);
+      }
+  };
+  // Iteration j: chunk j has landed in every wave's share of buffer j % NBUF once all waves
+  // pass the barrier (loads complete in issue order; the only younger ones are chunks
+  // j+1 .. j+D-1), and every wave has finished reading buffer (j-2) % NBUF, which the loads
+  // of chunk j + D now refill.
+  auto iteration = [&](int j, f32x16 (&cur)[RB][2], f32x16 (&prev)[RB][2]) {
+    ring_barrier<(D - 1) * G::DMA_PER_CHUNK>();
+    dma_chunk(j + D);
+    zero_ab(cur);
+    const int buf = j % NBUF;
+#pragma unroll
+    for (int kk = 0; kk < kKSteps; ++kk) {
+      gemm1_step(buf, kk, cur);
+      act_part(kk, prev);
+    }
+    gemm2((j + NBUF - 1) % NBUF);
+  };
+
+  // chunk 0: GEMM1 only
+  ring_barrier<(D - 1) * G::DMA_PER_CHUNK>();
+  dma_chunk(D);
+  zero_ab(ab0);
+#pragma unroll
+  for (int kk = 0; kk < kKSteps; ++kk) gemm1_step(0, kk, ab0);
+  // chunks 1 .. n_chunks-1 (n_chunks is even): GEMM1(j), activation and GEMM2 of j-1
+  int j = 1;
+  for (; j + 1 < n_chunks; j += 2) {
+    iteration(j, ab1, ab0);
+    iteration(j + 1, ab0, ab1);
+  }
+  iteration(j, ab1, ab0);
+  // drain: activation and GEMM2 of the last chunk
+#pragma unroll
+  for (int kk = 0; kk < kKSteps; ++kk) act_part(kk, ab1);
+  gemm2((n_chunks - 1) % NBUF);
+
+  // ---- epilogue: out rows through the per-wave staging tile (reuses chunk buffer 0 once
+  // every wave is past its last fragment read and all loads have landed) ----
+  ring_barrier<0>();
+  T* st = reinterpret_cast<T*>(&lds_w[0][0][0][0]) + wave * (32 * C::PITCH);
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
+    int64_t obase[C::NPASS];
+#pragma unroll
+    for (int ps = 0; ps < C::NPASS; ++ps) {
+      int mj, m0;
+      stage_coord<T>(ps, lane, mj, m0);
+      const int64_t pr = row0 + rb * 32 + mj;
+      obase[ps] = pr < n_rows ? pr * kC + m0 : -1;
+    }
+#pragma unroll
+    for (int ob = 0; ob < 4; ++ob) {
+      float vals[16];
+#pragma unroll
+      for (int r = 0; r < 16; ++r) vals[r] = acc_o[rb][ob][r];
+      wave_lds_sync();
+      stage_put<T>(st, vals, lane);
+      wave_lds_sync();
+#pragma unroll
+      for (int ps = 0; ps < C::NPASS; ++ps) {
+        int mj, m0;
+        stage_coord<T>(ps, lane, mj, m0);
+        if (obase[ps] >= 0) {
+          const int64_t off = obase[ps] + ob * 32;
+          VE_t v = stage_get_vec<T>(st, mj, m0);
+          // out may alias x: a lane reads the residual vector it is about to overwrite
+          if (add_residual) v = add_vec<T>(v, *reinterpret_cast<const VE_t*>(x + off));
+          *reinterpret_cast<VE_t*>(out + off) = v;
+        }
+      }
+    }
+  }
+}
+
+template <typename T>
+int transition_pack(const void* w_a, const void* w_b, const void* w_o, void* packed, int n_factor,
+                    hipStream_t stream) {
+  const int n_hidden = kC * n_factor;
+  const int total = (n_hidden / 32) * kTrFrags * kWave;
+  if (total == 0) return 0;
+  transition_pack_kernel<T><<<dim3((total + 255) / 256), dim3(256), 0, stream>>>(
+      (const T*)w_a, (const T*)w_b, (const T*)w_o, (T*)packed, n_hidden);
+  return 0;
+}
+
+template <typename T>
+int transition_fwd(const void* x, const void* ln_w, const void* ln_b, const void* packed,
+                   void* out, int64_t rows, int n_factor, int add_residual, float eps,
+                   hipStream_t stream) {
+  if (rows == 0) return 0;
+  const int64_t rows_per_block = 4 * TrCfg<T>::RB * 32;
+  const int64_t blocks = (rows + rows_per_block - 1) / rows_per_block;
+  transition_fused_kernel<T><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(
+      (const T*)x, (const T*)ln_w, (const T*)ln_b, (const T*)packed, (T*)out, rows, 4 * n_factor,
+      add_residual, eps);
+  return 0;
+}
+
+template int transition_pack<float>(const void*, const void*, const void*, void*, int, hipStream_t);
+template int transition_pack<bf16_t>(const void*, const void*, const void*, void*, int,
+                                     hipStream_t);
+template int transition_fwd<float>(const void*, const void*, const void*, const void*, void*,
+                                   int64_t, int, int, float, hipStream_t);
+template int transition_fwd<bf16_t>(const void*, const void*, const void*, const void*, void*,
+                                    int64_t, int, int, float, hipStream_t);
+
+}  // namespace ptx

@@ -166,11 +166,25 @@ def triangle_attention(z: torch.Tensor, mask: Optional[torch.Tensor], w: dict, h
     return out
 
 
+def transition_pack(w_a: torch.Tensor, w_b: torch.Tensor, w_o: torch.Tensor) -> torch.Tensor:
+    """Packs the three Transition weights (c = 128) into the fused kernel's streaming order."""
+    _dev(w_a, "w_a")
+    lib = _lib.load()
+    c = w_a.shape[1]
+    n_factor = w_a.shape[0] // c
+    packed = torch.empty((lib.ptx_transition_packed_elems(c, n_factor),), dtype=w_a.dtype,
+                         device=w_a.device)
+    with torch.cuda.device(w_a.device):
+        _call("transition_pack", lib.ptx_transition_pack, _ptr(w_a.contiguous()),
+              _ptr(w_b.contiguous()), _ptr(w_o.contiguous()), _ptr(packed), c, n_factor, _dt(w_a),
+              _stream())
+    return packed
+
+
 def transition(x: torch.Tensor, w: dict, n_factor: int, add_residual: bool,
-               out: Optional[torch.Tensor] = None, eps: float = 1e-5,
-               max_rows: int = 1 << 21) -> torch.Tensor:
-    """x [..., 128] -> [x +] W_o(silu(W_a LN x) * W_b LN x), rows processed in
-    slabs of `max_rows` so the hidden workspace stays bounded."""
+               out: Optional[torch.Tensor] = None, eps: float = 1e-5) -> torch.Tensor:
+    """x [..., 128] -> [x +] W_o(silu(W_a LN x) * W_b LN x); `w["packed"]` comes from
+    transition_pack."""
     _dev(x, "x")
     lib = _lib.load()
     c = x.shape[-1]
@@ -182,14 +196,9 @@ def transition(x: torch.Tensor, w: dict, n_factor: int, add_residual: bool,
     if out is None:
         out = torch.empty_like(x2)
     o2 = out.view(-1, c)
-    slab = min(rows, max_rows)
-    hidden = torch.empty((slab, n_factor * c), dtype=x.dtype, device=x.device)
     with torch.cuda.device(x.device):
-        for r0 in range(0, rows, slab):
-            r1 = min(rows, r0 + slab)
-            _call("transition", lib.ptx_transition_fwd, _ptr(x2[r0:r1]), _ptr(w["ln_w"]), _ptr(w["ln_b"]), _ptr(w["w_a"]), _ptr(w["w_b"]),
-                _ptr(w["w_o"]), _ptr(hidden), _ptr(o2[r0:r1]), r1 - r0, c, n_factor,
-                int(add_residual), eps, dt, st)
+        _call("transition", lib.ptx_transition_fwd, _ptr(x2), _ptr(w["ln_w"]), _ptr(w["ln_b"]),
+              _ptr(w["packed"]), _ptr(o2), rows, c, n_factor, int(add_residual), eps, dt, st)
     return out.view(x.shape)
 
 

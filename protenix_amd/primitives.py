@@ -101,8 +101,10 @@ class Transition(nn.Module):
     def _weights(self, dtype, device) -> dict:
         ps = (self.layernorm1.weight, self.layernorm1.bias, self.linear_no_bias_a.weight,
               self.linear_no_bias_b.weight, self.linear_no_bias.weight)
-        return self._cache.get(ps, dtype, device, lambda: dict(
-            zip(("ln_w", "ln_b", "w_a", "w_b", "w_o"), (_cv(p, dtype, device) for p in ps))))
+        def make():
+            ln_w, ln_b, w_a, w_b, w_o = (_cv(p, dtype, device) for p in ps)
+            return {"ln_w": ln_w, "ln_b": ln_b, "packed": ops.transition_pack(w_a, w_b, w_o)}
+        return self._cache.get(ps, dtype, device, make)
 
     def forward(self, x: torch.Tensor, _residual_out: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Returns the update; with `_residual_out` (may be x itself) writes

@@ -50,7 +50,9 @@ def test_argument_validation_without_gpu():
     assert b"128" in lib.ptx_last_error_string()
     assert lib.ptx_triattn_fwd(*([None] * 7), 8, 4, 16, 64, 0, 1e9, 1, None) == 2
     assert lib.ptx_triattn_project(*([None] * 13), 8, 128, 8, 16, 64, 0, 1e-5, 1, None) == 2
-    assert lib.ptx_transition_fwd(*([None] * 8), 10, 384, 4, 0, 1e-5, 0, None) == 2
+    assert lib.ptx_transition_fwd(*([None] * 5), 10, 384, 4, 0, 1e-5, 0, None) == 2
+    assert lib.ptx_transition_pack(None, None, None, None, 384, 4, 0, None) == 2
+    assert lib.ptx_transition_packed_elems(128, 4) == 3 * 4 * 128 * 128
     assert lib.ptx_pair_bias_fwd(*([None] * 5), 8, 128, 33, 1, 1e-5, 0, None) == 2
     assert lib.ptx_triattn_output(None, None, None, None, 8, 128, 0, 1, 0, None) == 1
     with pytest.raises(RuntimeError, match="unsupported shape"):
