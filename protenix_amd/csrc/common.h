@@ -108,6 +108,15 @@ __device__ __forceinline__ void load_to_lds16(const void* gptr, uint32_t lds_bas
                : "v"(gptr), "s"(lds_base)
                : "m0");
 }
+// The 4-byte form, used to pull cache lines into L2 ahead of time: no register receives the
+// data (a register destination would have to stay reserved until the load returns), it
+// lands in a junk LDS area of 256 bytes at lds_base.
+__device__ __forceinline__ void touch_to_lds4(const void* gptr, uint32_t lds_base) {
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off"
+               :
+               : "v"(gptr), "s"(lds_base)
+               : "m0");
+}
 #pragma clang diagnostic pop
 // LDS byte address of p, which must be the same for all lanes (it goes to a scalar register)
 __device__ __forceinline__ uint32_t lds_address(const void* p) {

@@ -255,7 +255,6 @@ __global__ __launch_bounds__(256, (MODE == kTriAttnIn ? 1 : 2)) void rowgemm_in_
   for (int ch = 0; ch < nch; ++ch) {
     const int buf = C::NBUF == 2 ? (ch & 1) : 0;
     fetch(min(ch + 1, nch - 1));   // unconditional: keeps the outstanding-load count static
-
     // Orientation: channel-major outputs want lane <-> channel (x as A operand).
     bool chan_on_lanes;
     if (MODE == kTriMulIn || MODE == kPairBias) chan_on_lanes = true;
@@ -600,19 +599,34 @@ __global__ __launch_bounds__(256, 2) void rowgemm_out_kernel(RowGemmOutParams p)
     }
   }
 
-  // out may alias res: a lane reads the residual vector it is about to overwrite.
+  // out may alias res: a lane reads the residual vectors it is about to overwrite.  They
+  // are all requested up front: next to their stores each would cost a serialised memory
+  // round trip, since no load can move above the previous (possibly aliasing) store.
   T* outp = (T*)p.out;
   const T* resp = (const T*)p.res;
+  int64_t obase[RB][C::NPASS];
+  VE_t resv[RB][4][C::NPASS];
 #pragma unroll
-  for (int rb = 0; rb < RB; ++rb) {
-    int64_t obase[C::NPASS];
+  for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
     for (int ps = 0; ps < C::NPASS; ++ps) {
       int mj, m0;
       stage_coord<T>(ps, lane, mj, m0);
       const int64_t pr = row0 + rb * 32 + mj;
-      obase[ps] = pr < p.n_rows ? p.omap(pr) + m0 : -1;
+      obase[rb][ps] = pr < p.n_rows ? p.omap(pr) + m0 : -1;
     }
+  if (resp) {
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+      for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int ps = 0; ps < C::NPASS; ++ps)
+          if (obase[rb][ps] >= 0)
+            resv[rb][t][ps] = *reinterpret_cast<const VE_t*>(resp + obase[rb][ps] + t * 32);
+  }
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
       float vals[16];
@@ -625,11 +639,10 @@ __global__ __launch_bounds__(256, 2) void rowgemm_out_kernel(RowGemmOutParams p)
       for (int ps = 0; ps < C::NPASS; ++ps) {
         int mj, m0;
         stage_coord<T>(ps, lane, mj, m0);
-        if (obase[ps] >= 0) {
-          const int64_t off = obase[ps] + t * 32;
+        if (obase[rb][ps] >= 0) {
           VE_t v = stage_get_vec<T>(st, mj, m0);
-          if (resp) v = add_vec<T>(v, *reinterpret_cast<const VE_t*>(resp + off));
-          *reinterpret_cast<VE_t*>(outp + off) = v;
+          if (resp) v = add_vec<T>(v, resv[rb][t][ps]);
+          *reinterpret_cast<VE_t*>(outp + obase[rb][ps] + t * 32) = v;
         }
       }
     }

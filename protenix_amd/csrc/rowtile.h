@@ -27,6 +27,28 @@ struct RowFrags {
   typename Vec8<T>::type f[RB][kKSteps];
 };
 
+// gamma = 1 / beta = 0 stand-ins for a LayerNorm without weight / bias: the affine loads
+// below are unconditional (a load under a branch costs a full wait of its own), a missing
+// parameter just points here.
+#define PTX_REP8(x) x, x, x, x, x, x, x, x
+#define PTX_REP128(x)                                                                           \
+  PTX_REP8(x), PTX_REP8(x), PTX_REP8(x), PTX_REP8(x), PTX_REP8(x), PTX_REP8(x), PTX_REP8(x),   \
+      PTX_REP8(x), PTX_REP8(x), PTX_REP8(x), PTX_REP8(x), PTX_REP8(x), PTX_REP8(x), PTX_REP8(x), \
+      PTX_REP8(x), PTX_REP8(x)
+static __device__ const float kOnesF32[kC] = {PTX_REP128(1.0f)};
+static __device__ const uint16_t kOnesBf16[kC] = {PTX_REP128(0x3F80)};
+static __device__ const float kZerosAny[kC] = {PTX_REP128(0.0f)};
+#undef PTX_REP128
+#undef PTX_REP8
+template <typename T> __device__ __forceinline__ const T* default_gamma();
+template <> __device__ __forceinline__ const float* default_gamma<float>() { return kOnesF32; }
+template <> __device__ __forceinline__ const bf16_t* default_gamma<bf16_t>() {
+  return reinterpret_cast<const bf16_t*>(kOnesBf16);
+}
+template <typename T> __device__ __forceinline__ const T* default_beta() {
+  return reinterpret_cast<const T*>(kZerosAny);
+}
+
 // Mean / rstd of a 128-channel row spread over the two half-wave lanes that hold it,
 // then gamma/beta (either may be null); result rounded to T like the reference's
 // LayerNorm output.
@@ -34,6 +56,14 @@ template <typename T>
 __device__ __forceinline__ void normalize_row(f32x8 (&v)[kKSteps], const T* __restrict__ gamma,
                                               const T* __restrict__ beta, float eps, int g,
                                               typename Vec8<T>::type (&out)[kKSteps]) {
+  const T* gp = (gamma ? gamma : default_gamma<T>()) + 8 * g;
+  const T* bp = (beta ? beta : default_beta<T>()) + 8 * g;
+  typename Vec8<T>::type gm[kKSteps], bt[kKSteps];
+#pragma unroll
+  for (int kk = 0; kk < kKSteps; ++kk) {
+    gm[kk] = load8<T>(gp + 16 * kk);
+    bt[kk] = load8<T>(bp + 16 * kk);
+  }
   float s = 0.0f;
 #pragma unroll
   for (int kk = 0; kk < kKSteps; ++kk)
@@ -53,19 +83,51 @@ __device__ __forceinline__ void normalize_row(f32x8 (&v)[kKSteps], const T* __re
   const float rstd = rsqrtf(q * (1.0f / kC) + eps);
 #pragma unroll
   for (int kk = 0; kk < kKSteps; ++kk) {
+    const f32x8 gmf = to_f32(gm[kk]), btf = to_f32(bt[kk]);
     f32x8 o;
 #pragma unroll
-    for (int t = 0; t < 8; ++t) o[t] = (v[kk][t] - mean) * rstd;
-    if (gamma) {
-      const f32x8 gm = to_f32(load8<T>(gamma + 16 * kk + 8 * g));
+    for (int t = 0; t < 8; ++t) o[t] = (v[kk][t] - mean) * rstd * gmf[t] + btf[t];
+    out[kk] = from_f32<T>(o);
+  }
+}
+
+// The same LayerNorm straight from the stored fragments, converting on the fly in each of
+// its three passes: no fp32 copy of the row is kept, for callers short of registers.
+template <typename T>
+__device__ __forceinline__ void normalize_raw(const typename Vec8<T>::type (&raw)[kKSteps],
+                                              const T* __restrict__ gamma,
+                                              const T* __restrict__ beta, float eps, int g,
+                                              typename Vec8<T>::type (&out)[kKSteps]) {
+  const T* gp = (gamma ? gamma : default_gamma<T>()) + 8 * g;
+  const T* bp = (beta ? beta : default_beta<T>()) + 8 * g;
+  float s = 0.0f;
 #pragma unroll
-      for (int t = 0; t < 8; ++t) o[t] *= gm[t];
-    }
-    if (beta) {
-      const f32x8 bt = to_f32(load8<T>(beta + 16 * kk + 8 * g));
+  for (int kk = 0; kk < kKSteps; ++kk) {
+    const f32x8 v = to_f32(raw[kk]);
 #pragma unroll
-      for (int t = 0; t < 8; ++t) o[t] += bt[t];
+    for (int t = 0; t < 8; ++t) s += v[t];
+  }
+  s += swap32(s);
+  const float mean = s * (1.0f / kC);
+  float q = 0.0f;
+#pragma unroll
+  for (int kk = 0; kk < kKSteps; ++kk) {
+    const f32x8 v = to_f32(raw[kk]);
+#pragma unroll
+    for (int t = 0; t < 8; ++t) {
+      const float d = v[t] - mean;
+      q += d * d;
     }
+  }
+  q += swap32(q);
+  const float rstd = rsqrtf(q * (1.0f / kC) + eps);
+#pragma unroll
+  for (int kk = 0; kk < kKSteps; ++kk) {
+    const f32x8 v = to_f32(raw[kk]);
+    const f32x8 gmf = to_f32(load8<T>(gp + 16 * kk)), btf = to_f32(load8<T>(bp + 16 * kk));
+    f32x8 o;
+#pragma unroll
+    for (int t = 0; t < 8; ++t) o[t] = (v[t] - mean) * rstd * gmf[t] + btf[t];
     out[kk] = from_f32<T>(o);
   }
 }

@@ -17,10 +17,12 @@
 // chunk buffers shared by the workgroup's 4 waves.  One wave per SIMD (the
 // accumulators and the row fragments take ~370 registers), so the wave is
 // pipelined by hand: while the MFMAs of chunk j's GEMM1 run, the VALU computes
-// the activation of chunk j-1, whose GEMM2 follows.
+// the activation of chunk j-1, whose GEMM2 follows; LDS fragment reads are issued
+// one step ahead of their use.
 #include "common.h"
 #include "kernels.h"
 #include "rowtile.h"
+#include <type_traits>
 
 namespace ptx {
 
@@ -121,23 +123,6 @@ __global__ __launch_bounds__(256) void transition_fused_kernel(
   f32x16 ab0[RB][2], ab1[RB][2];   // GEMM1 accumulators (a, b) of even / odd chunks
   V8 hf[RB][2];                    // activated hidden values as GEMM2 operand fragments
 
-  auto zero_ab = [&](f32x16 (&ab)[RB][2]) {
-#pragma unroll
-    for (int rb = 0; rb < RB; ++rb)
-#pragma unroll
-      for (int t = 0; t < 2; ++t)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) ab[rb][t][r] = 0.0f;
-  };
-  // K step kk of GEMM1: lane <-> row, register <-> hidden
-  auto gemm1_step = [&](int buf, int kk, f32x16 (&ab)[RB][2]) {
-    const V8 wa = read_frag(buf, kk), wb = read_frag(buf, 8 + kk);
-#pragma unroll
-    for (int rb = 0; rb < RB; ++rb) {
-      mma32(ab[rb][0], wa, xf.f[rb][kk]);
-      mma32(ab[rb][1], wb, xf.f[rb][kk]);
-    }
-  };
   // One eighth of a chunk's activation: accumulator registers 2*part, 2*part + 1.
   // a and b stay in fp32 through the activation; the product is rounded to T once.
   auto act_part = [&](int part, f32x16 (&ab)[RB][2]) {
@@ -150,15 +135,50 @@ __global__ __launch_bounds__(256) void transition_fused_kernel(
         hf[rb][r >> 3][r & 7] = from_f32<T>(a * b * sigmoidf_fast(a));
       }
   };
-  auto gemm2 = [&](int buf) {
+  // GEMM1 of the chunk in buffer `buf` into `cur` (lane <-> row, register <-> hidden), with
+  // the activation of the previous chunk (`prev`) between its MFMAs when ACT.  Fragments
+  // are read from LDS one K step before they are used; the last step fetches the first
+  // W_o fragment of the GEMM2 that follows (buffer `tail_buf`) and returns it.
+  auto gemm1 = [&](auto act_tag, int buf, f32x16 (&cur)[RB][2], f32x16 (&prev)[RB][2],
+                   int tail_buf) {
+    constexpr bool ACT = decltype(act_tag)::value;
+    V8 wa = read_frag(buf, 0), wb = read_frag(buf, 8);
 #pragma unroll
-    for (int u = 0; u < 2; ++u)
-#pragma unroll
-      for (int ob = 0; ob < 4; ++ob) {
-        const V8 wo = read_frag(buf, 16 + ob * 2 + u);
-#pragma unroll
-        for (int rb = 0; rb < RB; ++rb) mma32(acc_o[rb][ob], wo, hf[rb][u]);
+    for (int kk = 0; kk < kKSteps; ++kk) {
+      V8 na, nb = wb;
+      if (kk + 1 < kKSteps) {
+        na = read_frag(buf, kk + 1);
+        nb = read_frag(buf, 8 + kk + 1);
+      } else {
+        na = read_frag(tail_buf, 16);
       }
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb) {
+        if (kk == 0) {   // first K step: accumulate onto a constant zero (no register clears)
+          const f32x16 z = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+          cur[rb][0] = z;
+          cur[rb][1] = z;
+        }
+        mma32(cur[rb][0], wa, xf.f[rb][kk]);
+        mma32(cur[rb][1], wb, xf.f[rb][kk]);
+      }
+      if (ACT) act_part(kk, prev);
+      wa = na;
+      wb = nb;
+    }
+    return wa;
+  };
+  // GEMM2 of the chunk whose W_o fragments sit in buffer `buf`; `wo` is its first fragment.
+  auto gemm2 = [&](int buf, V8 wo) {
+#pragma unroll
+    for (int s2 = 0; s2 < 8; ++s2) {
+      const int u = s2 >> 2, ob = s2 & 3;
+      V8 nw = wo;
+      if (s2 + 1 < 8) nw = read_frag(buf, 16 + ((s2 + 1) & 3) * 2 + ((s2 + 1) >> 2));
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb) mma32(acc_o[rb][ob], wo, hf[rb][u]);
+      wo = nw;
+    }
   };
   // Iteration j: chunk j has landed in every wave's share of buffer j % NBUF once all waves
   // pass the barrier (loads complete in issue order; the only younger ones are chunks
@@ -167,22 +187,15 @@ __global__ __launch_bounds__(256) void transition_fused_kernel(
   auto iteration = [&](int j, f32x16 (&cur)[RB][2], f32x16 (&prev)[RB][2]) {
     ring_barrier<(D - 1) * G::DMA_PER_CHUNK>();
     dma_chunk(j + D);
-    zero_ab(cur);
-    const int buf = j % NBUF;
-#pragma unroll
-    for (int kk = 0; kk < kKSteps; ++kk) {
-      gemm1_step(buf, kk, cur);
-      act_part(kk, prev);
-    }
-    gemm2((j + NBUF - 1) % NBUF);
+    const int pbuf = (j + NBUF - 1) % NBUF;
+    const V8 wo = gemm1(std::true_type{}, j % NBUF, cur, prev, pbuf);
+    gemm2(pbuf, wo);
   };
 
   // chunk 0: GEMM1 only
   ring_barrier<(D - 1) * G::DMA_PER_CHUNK>();
   dma_chunk(D);
-  zero_ab(ab0);
-#pragma unroll
-  for (int kk = 0; kk < kKSteps; ++kk) gemm1_step(0, kk, ab0);
+  gemm1(std::false_type{}, 0, ab0, ab1, 0);
   // chunks 1 .. n_chunks-1 (n_chunks is even): GEMM1(j), activation and GEMM2 of j-1
   int j = 1;
   for (; j + 1 < n_chunks; j += 2) {
@@ -190,10 +203,35 @@ __global__ __launch_bounds__(256) void transition_fused_kernel(
     iteration(j + 1, ab0, ab1);
   }
   iteration(j, ab1, ab0);
+  // The residual vectors this lane will add in the epilogue, requested now so that their
+  // latency passes under the drain (loading each one next to its store would serialise a
+  // full memory round trip per tile: out may alias x, so no load could move above the
+  // previous store).  Each lane reads exactly the vectors it later overwrites.
+  int64_t obase[RB][C::NPASS];
+  VE_t resv[RB][4][C::NPASS];
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+    for (int ps = 0; ps < C::NPASS; ++ps) {
+      int mj, m0;
+      stage_coord<T>(ps, lane, mj, m0);
+      const int64_t pr = row0 + rb * 32 + mj;
+      obase[rb][ps] = pr < n_rows ? pr * kC + m0 : -1;
+    }
+  if (add_residual) {
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+      for (int ob = 0; ob < 4; ++ob)
+#pragma unroll
+        for (int ps = 0; ps < C::NPASS; ++ps)
+          if (obase[rb][ps] >= 0)
+            resv[rb][ob][ps] = *reinterpret_cast<const VE_t*>(x + obase[rb][ps] + ob * 32);
+  }
   // drain: activation and GEMM2 of the last chunk
 #pragma unroll
   for (int kk = 0; kk < kKSteps; ++kk) act_part(kk, ab1);
-  gemm2((n_chunks - 1) % NBUF);
+  gemm2((n_chunks - 1) % NBUF, read_frag((n_chunks - 1) % NBUF, 16));
 
   // ---- epilogue: out rows through the per-wave staging tile (reuses chunk buffer 0 once
   // every wave is past its last fragment read and all loads have landed) ----
@@ -201,14 +239,6 @@ __global__ __launch_bounds__(256) void transition_fused_kernel(
   T* st = reinterpret_cast<T*>(&lds_w[0][0][0][0]) + wave * (32 * C::PITCH);
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
-    int64_t obase[C::NPASS];
-#pragma unroll
-    for (int ps = 0; ps < C::NPASS; ++ps) {
-      int mj, m0;
-      stage_coord<T>(ps, lane, mj, m0);
-      const int64_t pr = row0 + rb * 32 + mj;
-      obase[ps] = pr < n_rows ? pr * kC + m0 : -1;
-    }
 #pragma unroll
     for (int ob = 0; ob < 4; ++ob) {
       float vals[16];
@@ -221,12 +251,10 @@ __global__ __launch_bounds__(256) void transition_fused_kernel(
       for (int ps = 0; ps < C::NPASS; ++ps) {
         int mj, m0;
         stage_coord<T>(ps, lane, mj, m0);
-        if (obase[ps] >= 0) {
-          const int64_t off = obase[ps] + ob * 32;
+        if (obase[rb][ps] >= 0) {
           VE_t v = stage_get_vec<T>(st, mj, m0);
-          // out may alias x: a lane reads the residual vector it is about to overwrite
-          if (add_residual) v = add_vec<T>(v, *reinterpret_cast<const VE_t*>(x + off));
-          *reinterpret_cast<VE_t*>(out + off) = v;
+          if (add_residual) v = add_vec<T>(v, resv[rb][ob][ps]);
+          *reinterpret_cast<VE_t*>(out + obase[rb][ps] + ob * 32) = v;
         }
       }
     }
