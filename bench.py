@@ -29,6 +29,11 @@ N_BLOCKS = 48
 C_Z, C_S = 128, 384
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
+# HBM bytes per launch of the triangle-attention core at N_token = 768, bf16, measured with
+# rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on this benchmark and calibrated against a plain
+# elementwise kernel of known size (profiles/trunk_n768_bf16_hbm_traffic.txt):
+# 603780 KiB fetched + 147456 KiB written.  Algorithmic: 594432 + 147456 KiB.
+TRIATTN_FWD_TRAFFIC_BYTES_N768 = (603780 + 147456) * 1024
 
 # Algorithmic work per launch at N tokens, c = 128, bf16 (2 bytes):
 #   flops for the MFMA-bound kernels, bytes for the HBM-bound ones.
@@ -37,7 +42,7 @@ def _work(n: int) -> dict:
     return {
         "triattn_fwd":     ("mfma", 512.0 * n ** 3),              # QK^T + PV, 4*N^3*H*D
         "trimul_contract": ("mfma", 256.0 * n ** 3),              # 2*N^3*c
-        "transition":      ("mfma", 393216.0 * n * n),            # 3 GEMMs 128<->512
+        "transition":      ("mfma", 393216.0 * n * n),            # 3 GEMMs 128<->512, fused
         "trimul_project":  ("hbm", 3.0 * e),                      # read z, write a and b
         "trimul_output":   ("hbm", 3.0 * e),                      # read x and z, write z
         "triattn_project": ("hbm", 5.0 * e),                      # read z, write q k v g (+ bias)
@@ -146,7 +151,8 @@ def main() -> int:
         kernels.append(ent)
     dom = next(k for k in kernels if k["kernel"] == "triattn_fwd")
     roofline = {"kernel": "triattn_fwd_kernel", "bound": "mfma", "achieved": dom["achieved"],
-                "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": dom["frac"], "traffic": None,
+                "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": dom["frac"],
+                "traffic": TRIATTN_FWD_TRAFFIC_BYTES_N768 if n == N_TOKEN else None,
                 "avg_ms": dom["avg_ms"], "launches": dom["launches"],
                 "algorithmic": "512*N^3 flop per launch (QK^T + PV over 4 heads x 32)"}
 
