@@ -1,0 +1,159 @@
+"""The named benchmark shapes: oracle parity where the CPU oracle finishes in seconds
+(configurations 2 and 3), and size-independent properties of the HIP path at the sizes it
+cannot reach (N_token = 768 blocks, N_token = 2048).  Tolerances as in test_gpu_parity."""
+import pytest
+import torch
+
+import protenix_amd as P
+from oracle import pairformer_oracle as O
+from tests.util import TOL_BF16, oracle_and_product, pad_mask, rel_err
+
+pytestmark = pytest.mark.gpu
+BF16 = torch.bfloat16
+
+
+def _z(n, seed=1234, c=128):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randn(1, n, n, c, generator=g).to(BF16)
+
+
+def test_config2_triattn_start_n384_pad32():
+    """TriangleAttention starting node, bf16, N = 384, last 32 tokens padded."""
+    ref, prod = oracle_and_product(O.TriangleAttention, P.TriangleAttention, 128, 32, 4,
+                                   starting=True, dtype=BF16)
+    n = 384
+    z, mask = _z(n), pad_mask(n, 32, BF16)
+    with torch.no_grad():
+        want = ref(z.float(), mask.float(), chunk_size=64)
+        got = prod(z.cuda(), mask.cuda())
+    assert rel_err(got, want) <= TOL_BF16
+
+
+@pytest.mark.parametrize("cls", ["TriangleMultiplicationOutgoing", "TriangleMultiplicationIncoming"])
+def test_config3_trimul_n768_pad48(cls):
+    """TriangleMultiplication outgoing / incoming, bf16, N = 768, 48 trailing padded tokens."""
+    ref, prod = oracle_and_product(getattr(O, cls), getattr(P, cls), 128, 128, dtype=BF16)
+    n = 768
+    z, mask = _z(n), pad_mask(n, 48, BF16)
+    with torch.no_grad():
+        want = ref(z.float(), mask.float())
+        got = prod(z.cuda(), mask.cuda())
+    assert rel_err(got, want) <= TOL_BF16
+
+
+def _block(seed=4321):
+    ref = O.seed_parameters_(O.PairformerBlock(), seed=seed)
+    blk = P.PairformerBlock()
+    blk.load_state_dict(ref.state_dict())
+    return blk.to("cuda", BF16).eval()
+
+
+def test_block_n768_padding_is_token_deletion():
+    """At N = 768 with 48 padded tokens, the valid 720 x 720 corner of the block's output
+    equals the block run on the cropped inputs (padded keys are inert in both triangle
+    updates; every other operation on the pair tensor is local to a pair)."""
+    blk = _block()
+    n, n_pad = 768, 48
+    nv = n - n_pad
+    s, z, _ = O.make_inputs(n, dtype=BF16)
+    mask = pad_mask(n, n_pad, BF16)
+    with torch.no_grad():
+        s_full, z_full = blk(s.cuda(), z.cuda(), mask.cuda())
+        s_crop, z_crop = blk(s[:, :nv].contiguous().cuda(), z[:, :nv, :nv].contiguous().cuda(),
+                             pad_mask(nv, 0, BF16).cuda())
+    assert rel_err(z_full[:, :nv, :nv], z_crop) <= TOL_BF16
+    # (not so for s: like the reference, the single attention has no key mask, so padded
+    # tokens do take part in it)
+    assert torch.isfinite(s_full.float()).all() and torch.isfinite(s_crop.float()).all()
+
+
+def test_triattn_n768_ending_is_starting_on_transpose():
+    """Ending-node attention reads z through transposed addressing; it must equal the
+    starting-node attention of the same weights applied to an explicit transpose."""
+    ref = O.seed_parameters_(O.TriangleAttention(128, 32, 4, starting=False))
+    end = P.TriangleAttention(128, 32, 4, starting=False)
+    start = P.TriangleAttention(128, 32, 4, starting=True)
+    end.load_state_dict(ref.state_dict())
+    start.load_state_dict(ref.state_dict())
+    end, start = end.to("cuda", BF16).eval(), start.to("cuda", BF16).eval()
+    n = 768
+    z = _z(n).cuda()
+    mask = pad_mask(n, 48, BF16).cuda()
+    with torch.no_grad():
+        got = end(z, mask)
+        want = start(z.transpose(1, 2).contiguous(), mask.transpose(1, 2).contiguous())
+    # same arithmetic on the same values, only the addressing differs
+    assert rel_err(got, want.transpose(1, 2)) <= TOL_BF16 / 4
+
+
+def test_trimul_n768_incoming_is_outgoing_on_transpose():
+    """incoming(z)[i, j] = g(z[i, j]) f(sum_k a(z[k, i]) b(z[k, j])) is the outgoing update with
+    the roles of a and b exchanged, applied to z^T and transposed back."""
+    ref = O.seed_parameters_(O.TriangleMultiplicationIncoming(128, 128))
+    in_m = P.TriangleMultiplicationIncoming(128, 128)
+    in_m.load_state_dict(ref.state_dict())
+    swapped = {}
+    for k, v in ref.state_dict().items():
+        k2 = k.replace("linear_a_", "linear_X_").replace("linear_b_", "linear_a_").replace(
+            "linear_X_", "linear_b_")
+        swapped[k2] = v
+    out_m = P.TriangleMultiplicationOutgoing(128, 128)
+    out_m.load_state_dict(swapped)
+    out_m, in_m = out_m.to("cuda", BF16).eval(), in_m.to("cuda", BF16).eval()
+    n = 768
+    z = _z(n).cuda()
+    mask = pad_mask(n, 48, BF16).cuda()
+    with torch.no_grad():
+        got = in_m(z, mask)
+        want = out_m(z.transpose(1, 2).contiguous(), mask.transpose(1, 2).contiguous())
+    # same values in a different summation order
+    assert rel_err(got, want.transpose(1, 2)) <= TOL_BF16 / 4
+
+
+def test_stack_48_blocks_bf16_tracks_fp32():
+    """Error growth through the full depth: the 48-block stack in bf16 against the same
+    stack in fp32 (itself within 1e-4 of the oracle per block) at a size both finish fast."""
+    n = 128
+    ref = O.seed_parameters_(O.PairformerStack(n_blocks=48))
+    outs = {}
+    for dt in (torch.float32, BF16):
+        st = P.PairformerStack(n_blocks=48)
+        st.load_state_dict(ref.state_dict())
+        with torch.no_grad():
+            for p in st.parameters():
+                p.copy_(p.to(BF16).float())
+        st = st.to("cuda", dt).eval()
+        s, z, pm = O.make_inputs(n, dtype=BF16)
+        with torch.no_grad():
+            outs[dt] = st(s.to(dt).cuda(), z.to(dt).cuda(), pm.to(dt).cuda())
+    for a, b in zip(outs[BF16], outs[torch.float32]):
+        assert rel_err(a, b) <= 5e-2   # 48 blocks of bf16 rounding on the residual stream
+
+
+def test_config5_n2048_pad64_two_blocks():
+    """N_token = 2048 with 64 padded tokens: the N^3 logits are never materialised (peak HBM
+    stays a small multiple of the pair tensor) and padding is token deletion here too."""
+    n, n_pad = 2048, 64
+    nv = n - n_pad
+    ref = O.seed_parameters_(O.PairformerStack(n_blocks=2))
+    st = P.PairformerStack(n_blocks=2)
+    st.load_state_dict(ref.state_dict())
+    st = st.to("cuda", BF16).eval()
+    g = torch.Generator().manual_seed(7)
+    z = torch.randn(1, n, n, 128, generator=g).to(BF16)
+    s = torch.randn(1, n, 384, generator=g).to(BF16)
+    mask = pad_mask(n, n_pad, BF16)
+    torch.cuda.reset_peak_memory_stats()
+    base = torch.cuda.memory_allocated()
+    with torch.no_grad():
+        s_full, z_full = st(s.cuda(), z.cuda(), mask.cuda())
+        peak = torch.cuda.max_memory_allocated() - base
+        z_bytes = n * n * 128 * 2
+        assert peak <= 12 * z_bytes, f"peak {peak / 1e9:.2f} GB"   # N^3 logits would be 69 GB
+        z_full = z_full[:, :nv, :nv].clone()
+        s_full = s_full[:, :nv].clone()
+        s_crop, z_crop = st(s[:, :nv].contiguous().cuda(), z[:, :nv, :nv].contiguous().cuda(),
+                            pad_mask(nv, 0, BF16).cuda())
+    assert torch.isfinite(z_full.float()).all()
+    assert rel_err(z_full, z_crop) <= TOL_BF16
+    assert torch.isfinite(s_full.float()).all() and torch.isfinite(s_crop.float()).all()
