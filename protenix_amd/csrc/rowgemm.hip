@@ -22,6 +22,7 @@
 #include "common.h"
 #include "kernels.h"
 #include "rowtile.h"
+#include <type_traits>
 
 namespace ptx {
 
@@ -90,12 +91,16 @@ __global__ __launch_bounds__(256, (MODE == kTriAttnIn ? 1 : 2)) void rowgemm_in_
   typedef typename VecE<T>::type VE_t;
   typedef Cfg<T> C;
   __shared__ V8 lds_w[C::NBUF][2 * kKSteps][kWave];
-  __shared__ __attribute__((aligned(16))) T lds_stage[4][32 * C::PITCH];
+  // One staging tile per 32 x 32 result tile of a chunk: all tiles of a chunk are written,
+  // then all are read back and stored, so that a chunk pays one LDS round trip, not one per tile.
+  constexpr int NST = 2 * RB;
+  __shared__ __attribute__((aligned(16))) T lds_stage[4][NST][32 * C::PITCH];
   __shared__ __attribute__((aligned(16))) float lds_mask[4][RB * 32];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int n = lane & 31, g = lane >> 5;
   const int64_t row0 = ((int64_t)blockIdx.x * 4 + wave) * (RB * 32);
-  T* st = lds_stage[wave];
+  T* st = lds_stage[wave][0];
+  auto stile = [&](int k) { return lds_stage[wave][k]; };
   const bool vec_ok = (p.n % C::VE) == 0;   // channel-major vectors stay inside one plane row
 
   // kTriMulIn works on 2-D patches of the pair tensor instead of runs of logical rows: a
@@ -239,14 +244,14 @@ __global__ __launch_bounds__(256, (MODE == kTriAttnIn ? 1 : 2)) void rowgemm_in_
   __syncthreads();
 
   // Row-major store of the staged tile (major = row, minor = 32 output columns at col0).
-  auto store_row_major = [&](T* outp, int64_t ld, int col0, int rb, const T* resp) {
+  auto store_row_major = [&](const T* stg, T* outp, int64_t ld, int col0, int rb, const T* resp) {
 #pragma unroll
     for (int ps = 0; ps < C::NPASS; ++ps) {
       int mj, m0;
       stage_coord<T>(ps, lane, mj, m0);
       if (rrow[rb][ps] >= 0) {
         const int64_t off = rrow[rb][ps] * ld + col0 + m0;
-        VE_t v = stage_get_vec<T>(st, mj, m0);
+        VE_t v = stage_get_vec<T>(stg, mj, m0);
         if (resp) v = add_vec<T>(v, *reinterpret_cast<const VE_t*>(resp + off));
         *reinterpret_cast<VE_t*>(outp + off) = v;
       }
@@ -308,6 +313,7 @@ __global__ __launch_bounds__(256, (MODE == kTriAttnIn ? 1 : 2)) void rowgemm_in_
       // a/b[c][i][k] = mask * sigmoid(gate) * proj ; lane <-> channel, register <-> row
       T* outp = (T*)p.out[ch >> 2];
       const int c0 = (ch & 3) * 32;
+      wave_lds_sync();
 #pragma unroll
       for (int rb = 0; rb < RB; ++rb) {
         float vals[16];
@@ -320,12 +326,14 @@ __global__ __launch_bounds__(256, (MODE == kTriAttnIn ? 1 : 2)) void rowgemm_in_
             vals[r] = m4[e] * sigmoidf_fast(acc[rb][1][r]) * acc[rb][0][r];
           }
         }
-        wave_lds_sync();
-        stage_put<T>(st, vals, lane);
-        wave_lds_sync();
-        // fragment-ordered store: 8 consecutive inner indices of one outer index = the 16
-        // bytes of one operand lane (half-wave (pk0/8)%2, row outer%32)
-        const int n_rb = (p.n + 31) >> 5, n_ks = p.pitch >> 4;
+        stage_put<T>(stile(rb), vals, lane);
+      }
+      wave_lds_sync();
+      // fragment-ordered store: 8 consecutive inner indices of one outer index = the 16
+      // bytes of one operand lane (half-wave (pk0/8)%2, row outer%32)
+      const int n_rb = (p.n + 31) >> 5, n_ks = p.pitch >> 4;
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
         for (int ps = 0; ps < C::NPASS; ++ps) {
           int chn, r0;
@@ -333,16 +341,17 @@ __global__ __launch_bounds__(256, (MODE == kTriAttnIn ? 1 : 2)) void rowgemm_in_
           const int i = pi0 + 4 * rb + (r0 >> 3);
           const int64_t off = trimul_frag_offset(c0 + chn, i >> 5, pk0 >> 4, n_rb, n_ks) +
                               ((pk0 >> 3) & 1) * 256 + (i & 31) * 8 + (r0 & 7);
-          *reinterpret_cast<VE_t*>(outp + off) = stage_get_vec<T>(st, chn, r0);
+          *reinterpret_cast<VE_t*>(outp + off) = stage_get_vec<T>(stile(rb), chn, r0);
         }
-      }
     } else if constexpr (MODE == kTriAttnIn) {
       // Outputs in the attention core's layouts (common.h): q and the gate head-major
       // [h][p][32], K / V^T / bias in fragment-ordered key tiles.
       const int which = ch >> 1;
       const int key_tiles = p.pitch >> 6;
-      if (which == 0 || which == 2) {
-        // q (rounded, then scaled) and sigmoid(g): one 32 x 32 tile = one head
+      // all result tiles of the chunk go to their staging tiles first ...
+      wave_lds_sync();
+      auto put_all = [&](auto kind) {   // kind: 0 = q (rounded, then scaled), 2 = gate, 1 = as is
+        constexpr int KIND = decltype(kind)::value;
 #pragma unroll
         for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
@@ -351,15 +360,27 @@ __global__ __launch_bounds__(256, (MODE == kTriAttnIn ? 1 : 2)) void rowgemm_in_
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
               float v = acc[rb][t][r];
-              if (which == 0) v = to_f32(from_f32<T>(v)) * p.q_scale;
-              else v = sigmoidf_fast(v);
+              if (KIND == 0) v = to_f32(from_f32<T>(v)) * p.q_scale;
+              if (KIND == 2) v = sigmoidf_fast(v);
               vals[r] = v;
             }
-            wave_lds_sync();
-            stage_put<T>(st, vals, lane);
-            wave_lds_sync();
+            stage_put<T>(stile(rb * 2 + t), vals, lane);
+          }
+      };
+      if (which == 0) put_all(std::integral_constant<int, 0>{});
+      else if (which == 2) put_all(std::integral_constant<int, 2>{});
+      else put_all(std::integral_constant<int, 1>{});
+      wave_lds_sync();
+      // ... and are then read back as 16-byte vectors and stored
+      if (which == 0 || which == 2) {
+        // q and sigmoid(g): one 32 x 32 tile = one head, head-major rows
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+          for (int t = 0; t < 2; ++t) {
             const int h = (ch & 1) * 2 + t;
-            store_row_major((T*)p.out[which] + (int64_t)h * p.n_rows * 32, 32, 0, rb, nullptr);
+            store_row_major(stile(rb * 2 + t), (T*)p.out[which] + (int64_t)h * p.n_rows * 32, 32, 0,
+                            rb, nullptr);
           }
       } else if (which == 1) {
         // K: staged row-major (major = key row, minor = d); each 16-byte d-chunk goes to
@@ -369,12 +390,6 @@ __global__ __launch_bounds__(256, (MODE == kTriAttnIn ? 1 : 2)) void rowgemm_in_
         for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
           for (int t = 0; t < 2; ++t) {
-            float vals[16];
-#pragma unroll
-            for (int r = 0; r < 16; ++r) vals[r] = acc[rb][t][r];
-            wave_lds_sync();
-            stage_put<T>(st, vals, lane);
-            wave_lds_sync();
             const int h = (ch & 1) * 2 + t;
 #pragma unroll
             for (int ps = 0; ps < C::NPASS; ++ps) {
@@ -383,7 +398,7 @@ __global__ __launch_bounds__(256, (MODE == kTriAttnIn ? 1 : 2)) void rowgemm_in_
               if (rrow[rb][ps] >= 0)
                 *reinterpret_cast<VE_t*>(
                     outp + attn_k_offset(h, rm_i[rb][ps], rm_j[rb][ps], m0, p.n, key_tiles)) =
-                    stage_get_vec<T>(st, mj, m0);
+                    stage_get_vec<T>(stile(rb * 2 + t), mj, m0);
             }
           }
       } else {
@@ -395,12 +410,6 @@ __global__ __launch_bounds__(256, (MODE == kTriAttnIn ? 1 : 2)) void rowgemm_in_
 #pragma unroll
           for (int t = 0; t < 2; ++t) {
             if (which == 4 && t == 1) continue;
-            float vals[16];
-#pragma unroll
-            for (int r = 0; r < 16; ++r) vals[r] = acc[rb][t][r];
-            wave_lds_sync();
-            stage_put<T>(st, vals, lane);
-            wave_lds_sync();
             const int h = (ch & 1) * 2 + t;
 #pragma unroll
             for (int ps = 0; ps < C::NPASS; ++ps) {
@@ -408,7 +417,7 @@ __global__ __launch_bounds__(256, (MODE == kTriAttnIn ? 1 : 2)) void rowgemm_in_
               stage_coord<T>(ps, lane, chn, r0);
               const int64_t pr = row0 + rb * 32 + r0;
               if (which == 4 && chn >= p.aux) continue;
-              const VE_t v = stage_get_vec<T>(st, chn, r0);
+              const VE_t v = stage_get_vec<T>(stile(rb * 2 + t), chn, r0);
               T* outp = (T*)p.out[which];
               if (vec_ok) {
                 if (cm_ok[rb]) {
@@ -477,7 +486,7 @@ __global__ __launch_bounds__(256, (MODE == kTriAttnIn ? 1 : 2)) void rowgemm_in_
         wave_lds_sync();
         stage_put<T>(st, vals, lane);
         wave_lds_sync();
-        store_row_major((T*)p.out[0], kC, ch * 32, rb,
+        store_row_major(st, (T*)p.out[0], kC, ch * 32, rb,
                         p.add_residual ? (const T*)p.x : nullptr);
       }
     }
