@@ -35,6 +35,10 @@ namespace ptx {
 constexpr int kD = 32;          // head dim
 constexpr int kKeyTile = 64;
 constexpr float kLog2e = 1.4426950408889634f;
+// tile_row: code paths, and the largest per-lane probability sum of a tile (32 values) the
+// optimistic path accepts
+enum { kOptimistic = 0, kClassic = 1, kMasked = 2 };
+constexpr float kOptimisticLimit = 1.0e12f;
 
 // Rows of the pair tensor handled by one wave (the bias tile is then loaded once per key
 // tile and reused).  More than one row does not fit the register budget of 2 waves/SIMD.
@@ -168,15 +172,30 @@ __global__ __launch_bounds__(256, 2) void triattn_fwd_kernel(
   }
 
   // One key tile of one row: logits, online softmax, P.V.  `tb` was fetched one tile ago.
-  // Two complete instantiations, so that the (rare) masked path shares no code with - and
-  // cannot be speculated into - the fast path.
-  auto tile_row = [&](auto masked_tag, int buf, int r, V8 (&tb)[2][2]) {
-    constexpr bool MASKED = decltype(masked_tag)::value;
+  // Three complete instantiations, so that the rarer paths share no code with - and cannot
+  // be speculated into - the common one:
+  //   kOptimistic  the common path.  The softmax reference m_run only has to keep exp() in
+  //                range, so it is NOT updated: probabilities are taken against the reference
+  //                left by earlier tiles, no tile maximum is formed and O, l are not rescaled.
+  //                If a probability sum leaves the safe range (a logit ~28 above the
+  //                reference, or no reference yet), nothing has been committed and the tile
+  //                is redone by kClassic.  Returns false in that case (same in all lanes).
+  //   kClassic     running maximum, rescale of O and l (first tile, or redo).
+  //   kMasked      tiles with a masked or out-of-range key: the reference's exact fp32
+  //                order (q.k + mask_bias) + triangle_bias.
+  auto tile_row = [&](auto mode_tag, int buf, int r, V8 (&tb)[2][2], int next_tile) -> bool {
+    constexpr int MODE = decltype(mode_tag)::value;
+    constexpr bool MASKED = MODE == kMasked;
     // all 8 operand fragments of the tile are requested from LDS up front, so their
     // latency is paid once per tile instead of once per MFMA
     V8 kvf[8];
 #pragma unroll
     for (int f = 0; f < 8; ++f) kvf[f] = lds_kv[buf][r][f][lane];
+    // the bias registers are refilled with the next tile's bias as soon as this tile's has
+    // been consumed (after the last row that shares it, and only once the tile is committed)
+    auto refill_bias = [&]() {
+      if (r == R - 1) fetch_bias(next_tile, tb);
+    };
     f32x16 s[2];
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
@@ -209,42 +228,40 @@ __global__ __launch_bounds__(256, 2) void triattn_fwd_kernel(
         }
     }
 
-    float mx[8];
+    float alpha = 1.0f;
+    if constexpr (MODE != kOptimistic) {
+      refill_bias();
+      float mx[8];
 #pragma unroll
-    for (int j = 0; j < 8; ++j)
-      mx[j] = fmaxf(fmaxf(s[0][2 * j], s[0][2 * j + 1]), fmaxf(s[1][2 * j], s[1][2 * j + 1]));
-    float mt = fmaxf(fmaxf(fmaxf(mx[0], mx[1]), fmaxf(mx[2], mx[3])),
-                     fmaxf(fmaxf(mx[4], mx[5]), fmaxf(mx[6], mx[7])));
-    mt = fmaxf(mt, swap32(mt));
-    const float m_new = fmaxf(m_run[r], mt);        // finite: key0 < n is never excluded
-    const float alpha = fast_exp2((m_run[r] - m_new) * kLog2e);   // 1 when the max did not move
-    m_run[r] = m_new;
+      for (int j = 0; j < 8; ++j)
+        mx[j] = fmaxf(fmaxf(s[0][2 * j], s[0][2 * j + 1]), fmaxf(s[1][2 * j], s[1][2 * j + 1]));
+      float mt = fmaxf(fmaxf(fmaxf(mx[0], mx[1]), fmaxf(mx[2], mx[3])),
+                       fmaxf(fmaxf(mx[4], mx[5]), fmaxf(mx[6], mx[7])));
+      mt = fmaxf(mt, swap32(mt));
+      const float m_new = fmaxf(m_run[r], mt);        // finite: key0 < n is never excluded
+      alpha = fast_exp2((m_run[r] - m_new) * kLog2e);   // 1 when the max did not move
+      m_run[r] = m_new;
 #pragma unroll
-    for (int e = 0; e < 16; ++e) acc_o[r][e] *= alpha;
+      for (int e = 0; e < 16; ++e) acc_o[r][e] *= alpha;
+    }
 
-    float psum = 0.0f;
     if constexpr (!MASKED) {
-      const float nml = -m_new * kLog2e;
+      const float nml = -m_run[r] * kLog2e;
 #pragma unroll
       for (int u = 0; u < 2; ++u)
 #pragma unroll
-        for (int e = 0; e < 16; ++e) {
-          s[u][e] = fast_exp2(fmaf(s[u][e], kLog2e, nml));
-          psum += s[u][e];
-        }
+        for (int e = 0; e < 16; ++e) s[u][e] = fast_exp2(fmaf(s[u][e], kLog2e, nml));
     } else {
       // (s - m) first: exact when both sit near -1e9
 #pragma unroll
       for (int u = 0; u < 2; ++u)
 #pragma unroll
-        for (int e = 0; e < 16; ++e) {
-          s[u][e] = fast_exp2((s[u][e] - m_new) * kLog2e);
-          psum += s[u][e];
-        }
+        for (int e = 0; e < 16; ++e) s[u][e] = fast_exp2((s[u][e] - m_run[r]) * kLog2e);
     }
-    l_run[r] = l_run[r] * alpha + psum;
-
-    // O^T += V^T P^T
+    // P as the B operand of P.V; its row sums are taken from the rounded values the matrix
+    // pipe will see (bf16: two per v_dot2c_f32_bf16)
+    V8 pf[2][2];
+    float psum = 0.0f;
 #pragma unroll
     for (int u = 0; u < 2; ++u)
 #pragma unroll
@@ -252,42 +269,72 @@ __global__ __launch_bounds__(256, 2) void triattn_fwd_kernel(
         f32x8 p8;
 #pragma unroll
         for (int t = 0; t < 8; ++t) p8[t] = s[u][8 * c + t];
-        mma32(acc_o[r], kvf[4 + u * 2 + c], from_f32<T>(p8));
+        pf[u][c] = from_f32<T>(p8);
+        if constexpr (sizeof(T) == 2) {
+          typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
+          bf16x2_t ones;
+          ones[0] = (__bf16)1.0f;
+          ones[1] = (__bf16)1.0f;
+#pragma unroll
+          for (int t = 0; t < 4; ++t) {
+            bf16x2_t pr;
+            pr[0] = pf[u][c][2 * t];
+            pr[1] = pf[u][c][2 * t + 1];
+            psum = __builtin_amdgcn_fdot2_f32_bf16(pr, ones, psum, false);
+          }
+        } else {
+#pragma unroll
+          for (int t = 0; t < 8; ++t) psum += p8[t];
+        }
       }
+    if constexpr (MODE == kOptimistic) {
+      // out of the safe range (also catches inf and NaN)?  Nothing committed yet: redo.
+      if (__ballot(!(psum < kOptimisticLimit)) != 0ull) return false;
+      refill_bias();
+    }
+    l_run[r] = l_run[r] * alpha + psum;
+
+    // O^T += V^T P^T
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+      for (int c = 0; c < 2; ++c) mma32(acc_o[r], kvf[4 + u * 2 + c], pf[u][c]);
+    return true;
   };
   auto process_tile = [&](int tile, V8 (&tb)[2][2]) {
     const int buf = tile % 3;
+    const int nt = tile + 1;
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       // Does this tile hold a masked or out-of-range key?  Same answer in all waves.
       const float mb_lane = lds_mb[buf][r][lane];
-      if (__ballot(mb_lane != 0.0f) != 0ull) tile_row(std::true_type{}, buf, r, tb);
-      else tile_row(std::false_type{}, buf, r, tb);
+      if (__ballot(mb_lane != 0.0f) != 0ull) {
+        tile_row(std::integral_constant<int, kMasked>{}, buf, r, tb, nt);
+      } else {
+        bool done = false;
+        if (tile != 0) done = tile_row(std::integral_constant<int, kOptimistic>{}, buf, r, tb, nt);
+        if (!done) tile_row(std::integral_constant<int, kClassic>{}, buf, r, tb, nt);
+      }
     }
   };
 
   // Tile t+2 travels global -> registers -> LDS while tile t is processed; the bias tile of
-  // t+1 is in flight to registers.  No load sits under a branch.
-  V8 bias_a[2][2], bias_b[2][2];
-  auto step = [&](int tile, V8 (&tb_cur)[2][2], V8 (&tb_nxt)[2][2]) {
+  // t+1 is requested into the bias registers once tile t has consumed them.
+  V8 tbias[2][2];
+  auto step = [&](int tile) {
     fetch(tile + 2);
-    fetch_bias(tile + 1, tb_nxt);
-    process_tile(tile, tb_cur);
+    process_tile(tile, tbias);
     stash(tile + 2);
     __syncthreads();
   };
 
   fetch(0);
-  fetch_bias(0, bias_a);
+  fetch_bias(0, tbias);
   stash(0);
   fetch(1);
   stash(1);
   __syncthreads();
-  // tiles are processed in pairs; a phantom last tile (odd tile count) is all -inf logits
-  for (int tile = 0; tile < n_tiles; tile += 2) {
-    step(tile, bias_a, bias_b);
-    step(tile + 1, bias_b, bias_a);
-  }
+  for (int tile = 0; tile < n_tiles; ++tile) step(tile);
 
   // ---- normalise, gate, store: lane <-> query, register e <-> d = acc_row(e, g) ----
   // o may alias gate: every gate load is issued before the first store.
