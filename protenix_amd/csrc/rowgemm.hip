@@ -138,9 +138,10 @@ __global__ __launch_bounds__(256, (MODE == kTriAttnIn ? 1 : 2)) void rowgemm_in_
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb) {
       f32x8 v[kKSteps];
+      // all four channel groups are requested at once: one memory round trip, not four
+      VE_t vec[4][C::NPASS];
 #pragma unroll
-      for (int cg = 0; cg < 4; ++cg) {           // channels 32*cg .. +31
-        VE_t vec[C::NPASS];
+      for (int cg = 0; cg < 4; ++cg)
 #pragma unroll
         for (int ps = 0; ps < C::NPASS; ++ps) {
           int chn, r0;
@@ -149,21 +150,23 @@ __global__ __launch_bounds__(256, (MODE == kTriAttnIn ? 1 : 2)) void rowgemm_in_
           const T* src = x2 + (int64_t)(32 * cg + chn) * p.n_rows;
           if (vec_ok) {
             const int64_t pc = pr + C::VE <= p.n_rows ? pr : 0;
-            vec[ps] = *reinterpret_cast<const VE_t*>(src + pc);
+            vec[cg][ps] = *reinterpret_cast<const VE_t*>(src + pc);
           } else {
 #pragma unroll
             for (int e = 0; e < C::VE; ++e) {
               const int64_t pe = pr + e < p.n_rows ? pr + e : p.n_rows - 1;
-              vec[ps][e] = src[pe];
+              vec[cg][ps][e] = src[pe];
             }
           }
         }
+#pragma unroll
+      for (int cg = 0; cg < 4; ++cg) {           // channels 32*cg .. +31
         wave_lds_sync();
 #pragma unroll
         for (int ps = 0; ps < C::NPASS; ++ps) {
           int chn, r0;
           stage_coord<T>(ps, lane, chn, r0);
-          stage_put_vec<T>(st, chn, r0, vec[ps]);
+          stage_put_vec<T>(st, chn, r0, vec[cg][ps]);
         }
         wave_lds_sync();
         // lane (row n, half g) picks channels 16*kk + 8*g + t of this group
@@ -244,7 +247,7 @@ __global__ __launch_bounds__(256, (MODE == kTriAttnIn ? 1 : 2)) void rowgemm_in_
   __syncthreads();
 
   // Row-major store of the staged tile (major = row, minor = 32 output columns at col0).
-  auto store_row_major = [&](const T* stg, T* outp, int64_t ld, int col0, int rb, const T* resp) {
+  auto store_row_major = [&](const T* stg, T* outp, int64_t ld, int col0, int rb, const VE_t* resv) {
 #pragma unroll
     for (int ps = 0; ps < C::NPASS; ++ps) {
       int mj, m0;
@@ -252,14 +255,33 @@ __global__ __launch_bounds__(256, (MODE == kTriAttnIn ? 1 : 2)) void rowgemm_in_
       if (rrow[rb][ps] >= 0) {
         const int64_t off = rrow[rb][ps] * ld + col0 + m0;
         VE_t v = stage_get_vec<T>(stg, mj, m0);
-        if (resp) v = add_vec<T>(v, *reinterpret_cast<const VE_t*>(resp + off));
+        if (resv) v = add_vec<T>(v, resv[ps]);
         *reinterpret_cast<VE_t*>(outp + off) = v;
       }
     }
   };
+  // (not unrolled: unrolled, the compiler hoists every chunk's loads to the top and spills them)
+#pragma clang loop unroll(disable)
   for (int ch = 0; ch < nch; ++ch) {
     const int buf = C::NBUF == 2 ? (ch & 1) : 0;
     fetch(min(ch + 1, nch - 1));   // unconditional: keeps the outstanding-load count static
+    // kTriMulOut: the residual vectors of this chunk's columns, requested before the MFMAs
+    // (next to their stores they would cost a serialised memory round trip per chunk, since
+    // out may alias z and no load can move above the previous store)
+    VE_t resv[RB][C::NPASS];
+    if constexpr (MODE == kTriMulOut) {
+      if (p.add_residual) {
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+          for (int ps = 0; ps < C::NPASS; ++ps) {
+            int mj, m0;
+            stage_coord<T>(ps, lane, mj, m0);
+            const int64_t pr = rrow[rb][ps] >= 0 ? rrow[rb][ps] : 0;
+            resv[rb][ps] = *reinterpret_cast<const VE_t*>((const T*)p.x + pr * kC + ch * 32 + m0);
+          }
+      }
+    }
     // Orientation: channel-major outputs want lane <-> channel (x as A operand).
     bool chan_on_lanes;
     if (MODE == kTriMulIn || MODE == kPairBias) chan_on_lanes = true;
@@ -486,8 +508,7 @@ __global__ __launch_bounds__(256, (MODE == kTriAttnIn ? 1 : 2)) void rowgemm_in_
         wave_lds_sync();
         stage_put<T>(st, vals, lane);
         wave_lds_sync();
-        store_row_major(st, (T*)p.out[0], kC, ch * 32, rb,
-                        p.add_residual ? (const T*)p.x : nullptr);
+        store_row_major(st, (T*)p.out[0], kC, ch * 32, rb, p.add_residual ? resv[rb] : nullptr);
       }
     }
 

@@ -58,12 +58,6 @@ __device__ __forceinline__ void normalize_row(f32x8 (&v)[kKSteps], const T* __re
                                               typename Vec8<T>::type (&out)[kKSteps]) {
   const T* gp = (gamma ? gamma : default_gamma<T>()) + 8 * g;
   const T* bp = (beta ? beta : default_beta<T>()) + 8 * g;
-  typename Vec8<T>::type gm[kKSteps], bt[kKSteps];
-#pragma unroll
-  for (int kk = 0; kk < kKSteps; ++kk) {
-    gm[kk] = load8<T>(gp + 16 * kk);
-    bt[kk] = load8<T>(bp + 16 * kk);
-  }
   float s = 0.0f;
 #pragma unroll
   for (int kk = 0; kk < kKSteps; ++kk)
@@ -83,7 +77,8 @@ __device__ __forceinline__ void normalize_row(f32x8 (&v)[kKSteps], const T* __re
   const float rstd = rsqrtf(q * (1.0f / kC) + eps);
 #pragma unroll
   for (int kk = 0; kk < kKSteps; ++kk) {
-    const f32x8 gmf = to_f32(gm[kk]), btf = to_f32(bt[kk]);
+    // (no branch around these loads, so the compiler may issue them as early as registers allow)
+    const f32x8 gmf = to_f32(load8<T>(gp + 16 * kk)), btf = to_f32(load8<T>(bp + 16 * kk));
     f32x8 o;
 #pragma unroll
     for (int t = 0; t < 8; ++t) o[t] = (v[kk][t] - mean) * rstd * gmf[t] + btf[t];
