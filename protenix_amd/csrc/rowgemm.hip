@@ -93,7 +93,11 @@ __global__ __launch_bounds__(256, (MODE == kTriAttnIn ? 1 : 2)) void rowgemm_in_
   __shared__ V8 lds_w[C::NBUF][2 * kKSteps][kWave];
   // One staging tile per 32 x 32 result tile of a chunk: all tiles of a chunk are written,
   // then all are read back and stored, so that a chunk pays one LDS round trip, not one per tile.
-  constexpr int NST = 2 * RB;
+  constexpr int NST = MODE == kTriMulOut ? 1 : 2 * RB;
+  // kTriMulOut: the raw z rows of this wave, kept for the residual add (re-reading them from
+  // HBM at the end costs a full extra pass: by then they have left the L2)
+  constexpr int kResPitch = kC + 16 / (int)sizeof(T);
+  __shared__ __attribute__((aligned(16))) T lds_res[MODE == kTriMulOut ? 4 : 1][MODE == kTriMulOut ? RB * 32 : 1][kResPitch];
   __shared__ __attribute__((aligned(16))) T lds_stage[4][NST][32 * C::PITCH];
   __shared__ __attribute__((aligned(16))) float lds_mask[4][RB * 32];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -125,6 +129,17 @@ __global__ __launch_bounds__(256, (MODE == kTriAttnIn ? 1 : 2)) void rowgemm_in_
     }
     load_rows_at<T, RB, true>(xf, (const T*)p.x, off, (const T*)p.gamma, (const T*)p.beta, p.eps,
                               lane);
+  } else if constexpr (MODE == kTriMulOut) {
+    RowFrags<T, RB> zraw;
+    load_rows<T, RB, false>(zraw, (const T*)p.x, p.xmap, row0, p.n_rows, nullptr, nullptr, 0.0f,
+                            lane);
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) {
+#pragma unroll
+      for (int kk = 0; kk < kKSteps; ++kk)
+        store8<T>(&lds_res[wave][rb * 32 + n][16 * kk + 8 * g], zraw.f[rb][kk]);
+      normalize_raw<T>(zraw.f[rb], (const T*)p.gamma, (const T*)p.beta, p.eps, g, xf.f[rb]);
+    }
   } else {
     load_rows<T, RB, true>(xf, (const T*)p.x, p.xmap, row0, p.n_rows, (const T*)p.gamma,
                            (const T*)p.beta, p.eps, lane);
@@ -265,22 +280,17 @@ __global__ __launch_bounds__(256, (MODE == kTriAttnIn ? 1 : 2)) void rowgemm_in_
   for (int ch = 0; ch < nch; ++ch) {
     const int buf = C::NBUF == 2 ? (ch & 1) : 0;
     fetch(min(ch + 1, nch - 1));   // unconditional: keeps the outstanding-load count static
-    // kTriMulOut: the residual vectors of this chunk's columns, requested before the MFMAs
-    // (next to their stores they would cost a serialised memory round trip per chunk, since
-    // out may alias z and no load can move above the previous store)
+    // kTriMulOut: the residual vectors of this chunk's columns, from the wave's LDS copy of z
     VE_t resv[RB][C::NPASS];
     if constexpr (MODE == kTriMulOut) {
-      if (p.add_residual) {
 #pragma unroll
-        for (int rb = 0; rb < RB; ++rb)
+      for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
-          for (int ps = 0; ps < C::NPASS; ++ps) {
-            int mj, m0;
-            stage_coord<T>(ps, lane, mj, m0);
-            const int64_t pr = rrow[rb][ps] >= 0 ? rrow[rb][ps] : 0;
-            resv[rb][ps] = *reinterpret_cast<const VE_t*>((const T*)p.x + pr * kC + ch * 32 + m0);
-          }
-      }
+        for (int ps = 0; ps < C::NPASS; ++ps) {
+          int mj, m0;
+          stage_coord<T>(ps, lane, mj, m0);
+          resv[rb][ps] = *reinterpret_cast<const VE_t*>(&lds_res[wave][rb * 32 + mj][ch * 32 + m0]);
+        }
     }
     // Orientation: channel-major outputs want lane <-> channel (x as A operand).
     bool chan_on_lanes;
