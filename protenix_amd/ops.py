@@ -66,6 +66,24 @@ def _same(t: Optional[torch.Tensor], like: torch.Tensor, name: str) -> Optional[
     return t.contiguous()
 
 
+def autocast_compute_dtype(x: torch.Tensor) -> Optional[torch.dtype]:
+    """The dtype torch.autocast would run this fp32 CUDA tensor's matmuls in, else None.
+    Production inference keeps fp32 parameters and an fp32 pair tensor under
+    torch.autocast("cuda", bfloat16) (inference.py:220-224 of the reference)."""
+    if not (x.is_cuda and x.dtype == torch.float32):
+        return None
+    try:
+        enabled = torch.is_autocast_enabled("cuda")
+    except TypeError:   # older signature
+        enabled = torch.is_autocast_enabled()
+    if not enabled:
+        return None
+    try:
+        return torch.get_autocast_dtype("cuda")
+    except AttributeError:
+        return torch.get_autocast_gpu_dtype()
+
+
 def key_pitch(n: int) -> int:
     return _lib.load().ptx_key_pitch(n)
 

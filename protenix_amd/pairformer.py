@@ -15,6 +15,7 @@ from typing import Optional, Tuple
 import torch
 import torch.nn as nn
 
+from . import ops
 from .primitives import Transition
 from .transformer import AttentionPairBias
 from .triangular import (TriangleAttention, TriangleMultiplicationIncoming,
@@ -61,6 +62,9 @@ class PairformerBlock(nn.Module):
         assert triangle_attention in ("torch", "deepspeed", "triattention", "cuequivariance")
         if not inplace_safe or not z.is_contiguous():
             z = z.clone(memory_format=torch.contiguous_format)
+        ac = ops.autocast_compute_dtype(z)
+        if ac is not None:
+            return self._forward_autocast(s, z, pair_mask, ac)
         self._pair_track(z, pair_mask)
         if self.c_s > 0:
             s = self._single_track(s, self.attention_pair_bias.pair_bias(z))
@@ -75,6 +79,25 @@ class PairformerBlock(nn.Module):
         # mask^T, expressed through transposed addressing of z and mask
         self.tri_att_end._run(z, pair_mask, transposed=True, residual_inplace=True)
         self.pair_transition(z, _residual_out=z)
+
+    def _forward_autocast(self, s: Optional[torch.Tensor], z: torch.Tensor,
+                          pair_mask: Optional[torch.Tensor], ac: torch.dtype
+                          ) -> Tuple[Optional[torch.Tensor], torch.Tensor]:
+        """fp32 residual stream under torch.autocast, as the reference runs in production:
+        every update is computed by the kernels in the autocast dtype from a rounded copy of
+        z and added to the fp32 z (in place; z is private here).  Costs a cast and an add
+        pass per update on top of the fused bf16 path."""
+        m = None if pair_mask is None else pair_mask.to(ac)
+        z.add_(self.tri_mul_out(z.to(ac), mask=m))
+        z.add_(self.tri_mul_in(z.to(ac), mask=m))
+        z.add_(self.tri_att_start._run(z.to(ac), m, transposed=False, residual_inplace=False))
+        z.add_(self.tri_att_end._run(z.to(ac), m, transposed=True, residual_inplace=False))
+        z.add_(self.pair_transition(z.to(ac)))
+        if self.c_s > 0:
+            bias = self.attention_pair_bias.pair_bias(z.to(ac))
+            s = s + self.attention_pair_bias.forward_with_bias(s.to(ac), bias).to(s.dtype)
+            s = s + self.single_transition(s.to(ac)).to(s.dtype)
+        return s, z
 
     def _single_track(self, s: torch.Tensor, bias: torch.Tensor) -> torch.Tensor:
         """s += attention(s; bias from z); s += transition(s).  Needs nothing of z but
@@ -116,7 +139,8 @@ class PairformerStack(nn.Module):
                 "triangle_multiplicative must be 'cuequivariance' or 'torch', but got "
                 f"{triangle_multiplicative}")
         assert triangle_attention in ("torch", "deepspeed", "triattention", "cuequivariance")
-        if not z.is_cuda or s is None or any(b.c_s == 0 for b in self.blocks):
+        if (not z.is_cuda or s is None or any(b.c_s == 0 for b in self.blocks)
+                or ops.autocast_compute_dtype(z) is not None):
             for blk in self.blocks:
                 s, z = blk(s, z, pair_mask, inplace_safe=True)
             return s, z

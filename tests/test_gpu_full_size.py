@@ -160,3 +160,24 @@ def test_config5_n2048_pad64_two_blocks():
     assert torch.isfinite(z_full.float()).all()
     assert rel_err(z_full, z_crop) <= TOL_BF16
     assert torch.isfinite(s_full.float()).all() and torch.isfinite(s_crop.float()).all()
+
+
+def test_block_under_autocast_keeps_fp32_residual_stream():
+    """Production mode of the reference (inference.py:220-224): fp32 parameters and fp32 s, z
+    under torch.autocast(bf16).  The kernels run in bf16, the residual stream stays fp32;
+    the result must be within the bf16 tolerance of the fp32 oracle and the inputs untouched."""
+    n = 96
+    ref = O.seed_parameters_(O.PairformerBlock()).eval()
+    blk = P.PairformerBlock()
+    blk.load_state_dict(ref.state_dict())
+    blk = blk.to("cuda").eval()                      # fp32 parameters
+    s, z, pm = O.make_inputs(n, n_pad=8)
+    with torch.no_grad():
+        want_s, want_z = ref(s, z, pm)
+        zc, sc = z.cuda(), s.cuda()
+        with torch.autocast("cuda", dtype=BF16):
+            got_s, got_z = blk(sc, zc, pm.cuda())
+    assert got_z.dtype == torch.float32 and got_s.dtype == torch.float32
+    assert torch.equal(zc.cpu(), z) and torch.equal(sc.cpu(), s)
+    assert rel_err(got_z, want_z) <= TOL_BF16
+    assert rel_err(got_s, want_s) <= TOL_BF16
