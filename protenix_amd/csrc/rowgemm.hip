@@ -53,6 +53,11 @@ struct RowGemmInParams {
 
 enum RowGemmInMode { kTriMulIn = 0, kTriAttnIn = 1, kPairBias = 3, kTriMulOut = 4 };
 
+// Where the 16-byte stores of lanes without a valid destination row go (lane l writes bytes
+// 16*l .. +15).  Keeping every store unconditional makes the number of stores a wave issues
+// per chunk a constant, which the weight ring below counts on.
+static __device__ __attribute__((aligned(16))) uint32_t g_store_sink[kWave * 4];
+
 template <int MODE>
 __device__ __forceinline__ int n_chunks(const RowGemmInParams& p) {
   if (MODE == kTriMulIn) return 8;                 // {a,b} x 4 channel blocks
@@ -86,7 +91,7 @@ __device__ __forceinline__ void chunk_tile(const RowGemmInParams& p, int ch, int
 }
 
 template <typename T, int RB, int MODE>
-__global__ __launch_bounds__(256, (MODE == kTriAttnIn ? 1 : 2)) void rowgemm_in_kernel(RowGemmInParams p) {
+__global__ __launch_bounds__(256, 2) void rowgemm_in_kernel(RowGemmInParams p) {
   typedef typename Vec8<T>::type V8;
   typedef typename VecE<T>::type VE_t;
   typedef Cfg<T> C;
@@ -257,9 +262,34 @@ __global__ __launch_bounds__(256, (MODE == kTriAttnIn ? 1 : 2)) void rowgemm_in_
 #pragma unroll
     for (int j = 0; j < 4; ++j) lds_w[buf][wave * 4 + j][lane] = pre[j];
   };
-  fetch(0);
-  stash(0);
-  __syncthreads();
+  // bf16: the weight fragments go from global memory straight into their LDS slots.  The
+  // loads are invisible to the compiler's wait-count bookkeeping and are waited for by hand
+  // (end of the chunk loop), counting the stores issued after them: the compiler's own
+  // wait for a register-staged prefetch cannot count those stores across the loop edge and
+  // drains them all, which stalls every wave once per chunk until its previous chunk's stores
+  // have reached the L2.
+  constexpr bool kDma = sizeof(T) == 2;
+  auto dma = [&](int ch, int buf) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int fid = wave * 4 + j;
+      const T* w;
+      int n_out, col0;
+      chunk_tile<T, MODE>(p, ch, fid >> 3, w, n_out, col0);
+      const int col = min(col0 + (lane & 31), n_out - 1);   // as load_wfrag
+      load_to_lds16(w + (int64_t)col * kC + (fid & 7) * 16 + 8 * (lane >> 5),
+                    lds_address(&lds_w[buf][fid][0]));
+    }
+  };
+  T* const sink = reinterpret_cast<T*>(g_store_sink) + lane * C::VE;
+  if constexpr (kDma) {
+    dma(0, 0);
+    ring_barrier<0>();
+  } else {
+    fetch(0);
+    stash(0);
+    __syncthreads();
+  }
 
   // Row-major store of the staged tile (major = row, minor = 32 output columns at col0).
   auto store_row_major = [&](const T* stg, T* outp, int64_t ld, int col0, int rb, const VE_t* resv) {
@@ -267,19 +297,22 @@ __global__ __launch_bounds__(256, (MODE == kTriAttnIn ? 1 : 2)) void rowgemm_in_
     for (int ps = 0; ps < C::NPASS; ++ps) {
       int mj, m0;
       stage_coord<T>(ps, lane, mj, m0);
-      if (rrow[rb][ps] >= 0) {
-        const int64_t off = rrow[rb][ps] * ld + col0 + m0;
-        VE_t v = stage_get_vec<T>(stg, mj, m0);
-        if (resv) v = add_vec<T>(v, resv[ps]);
-        *reinterpret_cast<VE_t*>(outp + off) = v;
-      }
+      const int64_t off = rrow[rb][ps] * ld + col0 + m0;
+      VE_t v = stage_get_vec<T>(stg, mj, m0);
+      if (resv) v = add_vec<T>(v, resv[ps]);
+      *reinterpret_cast<VE_t*>(rrow[rb][ps] >= 0 ? outp + off : sink) = v;
     }
   };
   // (not unrolled: unrolled, the compiler hoists every chunk's loads to the top and spills them)
 #pragma clang loop unroll(disable)
   for (int ch = 0; ch < nch; ++ch) {
     const int buf = C::NBUF == 2 ? (ch & 1) : 0;
-    fetch(min(ch + 1, nch - 1));   // unconditional: keeps the outstanding-load count static
+    if constexpr (kDma) {
+      // the other buffer was last read in the previous chunk, which every wave has left
+      if (ch + 1 < nch) dma(ch + 1, buf ^ 1);
+    } else {
+      fetch(min(ch + 1, nch - 1));   // unconditional: keeps the outstanding-load count static
+    }
     // kTriMulOut: the residual vectors of this chunk's columns, from the wave's LDS copy of z
     VE_t resv[RB][C::NPASS];
     if constexpr (MODE == kTriMulOut) {
@@ -338,7 +371,7 @@ __global__ __launch_bounds__(256, (MODE == kTriAttnIn ? 1 : 2)) void rowgemm_in_
     // The next chunk's weights go to the other LDS buffer now, before this chunk's stores
     // are issued: waiting for those loads later would also wait for every store issued in
     // between (memory operations retire in order).
-    if (C::NBUF == 2) stash(buf ^ 1);
+    if (!kDma && C::NBUF == 2) stash(buf ^ 1);
 
     // ------------------------------ epilogues ------------------------------
     if constexpr (MODE == kTriMulIn) {
@@ -427,10 +460,10 @@ __global__ __launch_bounds__(256, (MODE == kTriAttnIn ? 1 : 2)) void rowgemm_in_
             for (int ps = 0; ps < C::NPASS; ++ps) {
               int mj, m0;
               stage_coord<T>(ps, lane, mj, m0);
-              if (rrow[rb][ps] >= 0)
-                *reinterpret_cast<VE_t*>(
-                    outp + attn_k_offset(h, rm_i[rb][ps], rm_j[rb][ps], m0, p.n, key_tiles)) =
-                    stage_get_vec<T>(stile(rb * 2 + t), mj, m0);
+              *reinterpret_cast<VE_t*>(
+                  rrow[rb][ps] >= 0
+                      ? outp + attn_k_offset(h, rm_i[rb][ps], rm_j[rb][ps], m0, p.n, key_tiles)
+                      : sink) = stage_get_vec<T>(stile(rb * 2 + t), mj, m0);
             }
           }
       } else {
@@ -452,17 +485,20 @@ __global__ __launch_bounds__(256, (MODE == kTriAttnIn ? 1 : 2)) void rowgemm_in_
               const VE_t v = stage_get_vec<T>(stile(rb * 2 + t), chn, r0);
               T* outp = (T*)p.out[which];
               if (vec_ok) {
-                if (cm_ok[rb]) {
-                  const int64_t off =
-                      which == 3 ? attn_v_offset(h, cm_i[rb], cm_j[rb], chn, p.n, key_tiles)
-                                 : attn_b_offset(chn, cm_i[rb], cm_j[rb], q_blocks, key_tiles);
-                  *reinterpret_cast<VE_t*>(outp + off) = v;
-                }
+                const int64_t off =
+                    which == 3 ? attn_v_offset(h, cm_i[rb], cm_j[rb], chn, p.n, key_tiles)
+                               : attn_b_offset(chn, cm_i[rb], cm_j[rb], q_blocks, key_tiles);
+                *reinterpret_cast<VE_t*>(cm_ok[rb] ? outp + off : sink) = v;
               } else {
+                // (the row is made opaque here: the divisions below do not depend on the
+                // chunk, so they would otherwise be hoisted out of the chunk loop for every
+                // element and occupy some 240 registers in launches that never take this path)
+                int64_t pr_here = pr;
+                asm volatile("" : "+v"(pr_here));
 #pragma unroll
                 for (int e = 0; e < C::VE; ++e) {
-                  if (pr + e < p.n_rows) {
-                    const uint32_t pe = (uint32_t)(pr + e);
+                  if (pr_here + e < p.n_rows) {
+                    const uint32_t pe = (uint32_t)(pr_here + e);
                     const uint32_t i = pe / (uint32_t)p.n, j = pe - i * (uint32_t)p.n;
                     const int64_t off = which == 3 ? attn_v_offset(h, i, j, chn, p.n, key_tiles)
                                                    : attn_b_offset(chn, i, j, q_blocks, key_tiles);
@@ -522,11 +558,23 @@ __global__ __launch_bounds__(256, (MODE == kTriAttnIn ? 1 : 2)) void rowgemm_in_
       }
     }
 
-    if (C::NBUF == 1) {
-      __syncthreads();      // everyone is done reading the single buffer
-      stash(0);
+    if constexpr (kDma) {
+      // The next chunk's weights must have landed: all but the stores this wave issued
+      // after requesting them (a lower bound on that count is what is safe; the triangle
+      // bias, whose store count varies, is the last chunk and has no successor).
+      constexpr int kStores = MODE == kTriMulIn    ? RB * C::NPASS
+                              : MODE == kTriAttnIn ? RB * 2 * C::NPASS
+                              : MODE == kTriMulOut ? RB * C::NPASS
+                                                   : 0;
+      if (MODE != kTriAttnIn || vec_ok) ring_barrier<kStores>();
+      else ring_barrier<0>();   // element-wise V^T stores: no fixed count
+    } else {
+      if (C::NBUF == 1) {
+        __syncthreads();      // everyone is done reading the single buffer
+        stash(0);
+      }
+      __syncthreads();
     }
-    __syncthreads();
   }
 }
 
