@@ -22,6 +22,7 @@
 #include "common.h"
 #include "kernels.h"
 #include "rowtile.h"
+#include <algorithm>
 #include <type_traits>
 
 namespace ptx {
@@ -90,39 +91,121 @@ __device__ __forceinline__ void chunk_tile(const RowGemmInParams& p, int ch, int
   }
 }
 
+// Geometry of one instantiation.  bf16 (all but the single-chunk pair bias) runs "resident":
+// one workgroup of 8 waves per CU loads ALL weight fragments of the launch into LDS once, and
+// its waves then walk over row tiles on their own, with no workgroup barrier and no weight
+// traffic in the loop.  (With the weights re-read per workgroup, a 256-row workgroup pulls as
+// many bytes of weights through the L2 as it moves pair-tensor data, and every wave's wait
+// for its share of them also waits for the stores it issued before.)  fp32 weights are twice
+// the size and do not fit: that path stages one chunk at a time through registers.
+template <typename T, int MODE> struct InCfg {
+  static constexpr bool RES = sizeof(T) == 2 && MODE != kPairBias;
+  static constexpr int NW = RES ? 8 : 4;   // waves per workgroup
+  static constexpr int NCH =
+      MODE == kTriMulIn ? 8 : MODE == kTriAttnIn ? 9 : MODE == kPairBias ? 1 : 4;
+  // weight fragments held in LDS (16 per chunk; the resident triangle bias is one tile of 8)
+  static constexpr int NFRAG =
+      RES ? (MODE == kTriAttnIn ? 8 * 16 + 8 : NCH * 16) : Cfg<T>::NBUF * 16;
+};
+
 template <typename T, int RB, int MODE>
-__global__ __launch_bounds__(256, 2) void rowgemm_in_kernel(RowGemmInParams p) {
+__global__ __launch_bounds__((InCfg<T, MODE>::NW * 64), (InCfg<T, MODE>::RES ? 1 : 2)) void
+rowgemm_in_kernel(RowGemmInParams p) {
   typedef typename Vec8<T>::type V8;
   typedef typename VecE<T>::type VE_t;
   typedef Cfg<T> C;
-  __shared__ V8 lds_w[C::NBUF][2 * kKSteps][kWave];
-  // One staging tile per 32 x 32 result tile of a chunk: all tiles of a chunk are written,
-  // then all are read back and stored, so that a chunk pays one LDS round trip, not one per tile.
-  constexpr int NST = MODE == kTriMulOut ? 1 : 2 * RB;
+  typedef InCfg<T, MODE> IC;
+  constexpr bool RES = IC::RES;
+  constexpr int NW = IC::NW;
+  __shared__ V8 lds_w[IC::NFRAG][kWave];
+  // Staging tiles per wave.  Resident: one (LDS is full of weights).  Otherwise one per
+  // 32 x 32 result tile of a chunk: all tiles of a chunk are written, then all are read back
+  // and stored, so that a chunk pays one LDS round trip, not one per tile.
+  constexpr int NST = (RES || MODE == kTriMulOut) ? 1 : 2 * RB;
   // kTriMulOut: the raw z rows of this wave, kept for the residual add (re-reading them from
   // HBM at the end costs a full extra pass: by then they have left the L2)
   constexpr int kResPitch = kC + 16 / (int)sizeof(T);
-  __shared__ __attribute__((aligned(16))) T lds_res[MODE == kTriMulOut ? 4 : 1][MODE == kTriMulOut ? RB * 32 : 1][kResPitch];
-  __shared__ __attribute__((aligned(16))) T lds_stage[4][NST][32 * C::PITCH];
-  __shared__ __attribute__((aligned(16))) float lds_mask[4][RB * 32];
+  __shared__ __attribute__((aligned(16))) T lds_res[MODE == kTriMulOut ? NW : 1][MODE == kTriMulOut ? RB * 32 : 1][kResPitch];
+  __shared__ __attribute__((aligned(16))) T lds_stage[NW][NST][32 * C::PITCH];
+  __shared__ __attribute__((aligned(16))) float lds_mask[MODE == kTriMulIn ? NW : 1][RB * 32];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int n = lane & 31, g = lane >> 5;
-  const int64_t row0 = ((int64_t)blockIdx.x * 4 + wave) * (RB * 32);
   T* st = lds_stage[wave][0];
   auto stile = [&](int k) { return lds_stage[wave][k]; };
   const bool vec_ok = (p.n % C::VE) == 0;   // channel-major vectors stay inside one plane row
+  T* const sink = reinterpret_cast<T*>(g_store_sink) + lane * C::VE;
+  const int nch = n_chunks<MODE>(p);
 
-  // kTriMulIn works on 2-D patches of the pair tensor instead of runs of logical rows: a
-  // workgroup covers 16*RB outer indices x 8 inner indices, a row block 4 x 8 (MFMA row r <->
-  // outer pi0 + 4*rb + r/8, inner pk0 + r%8), which makes a row block's 32 values of one
-  // channel 64 contiguous bytes of the contraction's fragment-ordered operands.
-  int pi0 = 0, pk0 = 0;
-  if constexpr (MODE == kTriMulIn) {
-    const uint32_t n_kb = (uint32_t)p.pitch >> 3;   // the K padding is written too (as zeros)
-    const uint32_t ip = blockIdx.x / n_kb;
-    pk0 = (int)(blockIdx.x - ip * n_kb) * 8;
-    pi0 = (int)ip * (16 * RB) + wave * (4 * RB);
+  // Work units ("wave tiles").  kTriMulIn works on 2-D patches of the pair tensor instead of
+  // runs of logical rows: four waves cover 16*RB outer indices x 8 inner indices, a row block
+  // 4 x 8 (MFMA row r <-> outer pi0 + 4*rb + r/8, inner pk0 + r%8), which makes a row block's
+  // 32 values of one channel 64 contiguous bytes of the contraction's fragment-ordered
+  // operands.  The other modes take RB*32 consecutive logical rows.
+  const uint32_t n_kb = (uint32_t)p.pitch >> 3;   // kTriMulIn: the K padding is written too (as zeros)
+  int64_t n_tiles;
+  if (MODE == kTriMulIn) n_tiles = (int64_t)((p.n + 16 * RB - 1) / (16 * RB)) * n_kb * 4;
+  else n_tiles = (p.n_rows + RB * 32 - 1) / (RB * 32);
+  // Resident: waves 0-3 of all workgroups come first in the walk, then waves 4-7, so that a
+  // last round that covers half the machine's waves still gives every CU (and SIMD) its share.
+  int64_t tile = RES ? (int64_t)(wave >> 2) * (gridDim.x * 4) + blockIdx.x * 4 + (wave & 3)
+                     : (int64_t)blockIdx.x * 4 + wave;
+  const int64_t tile_step = (int64_t)gridDim.x * NW;
+
+  // Weight fragment f = 16 * chunk + 8 * tile + K step, from global memory straight into its
+  // LDS slot (bf16).  These loads are invisible to the compiler's wait-count bookkeeping and
+  // are waited for by hand.
+  auto dma_frag = [&](int f_src, int f_dst) {
+    const T* w;
+    int n_out, col0;
+    chunk_tile<T, MODE>(p, f_src >> 4, (f_src >> 3) & 1, w, n_out, col0);
+    const int col = min(col0 + (lane & 31), n_out - 1);   // as load_wfrag
+    load_to_lds16(w + (int64_t)col * kC + (f_src & 7) * 16 + 8 * (lane >> 5),
+                  lds_address(&lds_w[f_dst][0]));
+  };
+  constexpr bool kDma = sizeof(T) == 2 && !RES;   // bf16 pair bias: its single chunk
+  if constexpr (RES) {
+    for (int f = wave; f < IC::NFRAG; f += NW) dma_frag(f, f);
+    ring_barrier<0>();
+  } else if constexpr (kDma) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) dma_frag(wave * 4 + j, wave * 4 + j);
+    ring_barrier<0>();
   }
+
+  // fp32: the next chunk's fragments are prefetched into registers and stored to LDS
+  V8 pre[4];
+  auto fetch = [&](int ch) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int fid = wave * 4 + j;   // 16 fragments per chunk: tile = fid/8, kk = fid%8
+      const T* w;
+      int n_out, col0;
+      chunk_tile<T, MODE>(p, ch, fid >> 3, w, n_out, col0);
+      pre[j] = load_wfrag<T>(w, kC, n_out, col0, (fid & 7) * 16, lane);
+    }
+  };
+  auto stash = [&](int buf) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) lds_w[buf * 16 + wave * 4 + j][lane] = pre[j];
+  };
+
+  while (true) {
+    if (RES && tile >= n_tiles) break;
+    const int64_t row0 = tile * (RB * 32);
+    int pi0 = 0, pk0 = 0;
+    if constexpr (MODE == kTriMulIn) {
+      const uint32_t vb = (uint32_t)(tile >> 2);
+      const uint32_t ip = vb / n_kb;
+      pk0 = (int)(vb - ip * n_kb) * 8;
+      pi0 = (int)ip * (16 * RB) + (int)(tile & 3) * (4 * RB);
+    }
+    // (resident: made opaque per tile, or the affine parameters' loads and conversions are
+    // hoisted out of the tile loop and held in registers)
+    const T* gamma = (const T*)p.gamma;
+    const T* beta = (const T*)p.beta;
+    const T* gamma2 = (const T*)p.gamma2;
+    const T* beta2 = (const T*)p.beta2;
+    if constexpr (RES) asm volatile("" : "+s"(gamma), "+s"(beta), "+s"(gamma2), "+s"(beta2));
 
   RowFrags<T, RB> xf;
   if constexpr (MODE == kTriMulIn) {
@@ -132,22 +215,21 @@ __global__ __launch_bounds__(256, 2) void rowgemm_in_kernel(RowGemmInParams p) {
       const int i = min(pi0 + 4 * rb + (n >> 3), p.n - 1), k = min(pk0 + (n & 7), p.n - 1);
       off[rb] = (int64_t)i * p.xmap.stride_outer + (int64_t)k * p.xmap.stride_inner;
     }
-    load_rows_at<T, RB, true>(xf, (const T*)p.x, off, (const T*)p.gamma, (const T*)p.beta, p.eps,
-                              lane);
+    load_rows_at<T, RB, true>(xf, (const T*)p.x, off, gamma, beta, p.eps, lane);
   } else if constexpr (MODE == kTriMulOut) {
     RowFrags<T, RB> zraw;
     load_rows<T, RB, false>(zraw, (const T*)p.x, p.xmap, row0, p.n_rows, nullptr, nullptr, 0.0f,
                             lane);
+    wave_lds_sync();   // the previous tile's residual reads are done
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb) {
 #pragma unroll
       for (int kk = 0; kk < kKSteps; ++kk)
         store8<T>(&lds_res[wave][rb * 32 + n][16 * kk + 8 * g], zraw.f[rb][kk]);
-      normalize_raw<T>(zraw.f[rb], (const T*)p.gamma, (const T*)p.beta, p.eps, g, xf.f[rb]);
+      normalize_raw<T>(zraw.f[rb], gamma, beta, p.eps, g, xf.f[rb]);
     }
   } else {
-    load_rows<T, RB, true>(xf, (const T*)p.x, p.xmap, row0, p.n_rows, (const T*)p.gamma,
-                           (const T*)p.beta, p.eps, lane);
+    load_rows<T, RB, true>(xf, (const T*)p.x, p.xmap, row0, p.n_rows, gamma, beta, p.eps, lane);
   }
 
   // kTriMulOut: second fragment set = LayerNorm_out of the channel-major triangle product,
@@ -196,13 +278,14 @@ __global__ __launch_bounds__(256, 2) void rowgemm_in_kernel(RowGemmInParams p) {
           for (int t = 0; t < 8; ++t)
             v[2 * cg + k2][t] = to_f32(st[(16 * k2 + 8 * g + t) * C::PITCH + n]);
       }
-      normalize_row<T>(v, (const T*)p.gamma2, (const T*)p.beta2, p.eps, g, xf2.f[rb]);
+      normalize_row<T>(v, gamma2, beta2, p.eps, g, xf2.f[rb]);
     }
   }
 
   // TriMulIn: the 32 mask values of each row block, shared through LDS
   // (inner indices between n and the pitch get factor 0: the contraction relies on zeros there)
   if constexpr (MODE == kTriMulIn) {
+    wave_lds_sync();   // the previous tile's mask reads are done
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb) {
       const int i = min(pi0 + 4 * rb + (n >> 3), p.n - 1), k = min(pk0 + (n & 7), p.n - 1);
@@ -216,8 +299,8 @@ __global__ __launch_bounds__(256, 2) void rowgemm_in_kernel(RowGemmInParams p) {
     wave_lds_sync();
   }
 
-  // Row-major destinations (kTriAttnIn q/k/g, kTransitionIn hidden, kTriMulOut out): the
-  // logical row this lane stores in each read-back pass, or -1.
+  // Row-major destinations (kTriAttnIn q/k/g, kTriMulOut out): the logical row this lane
+  // stores in each read-back pass, or -1.
   int64_t rrow[RB][C::NPASS];
   int rm_i[RB][C::NPASS], rm_j[RB][C::NPASS];   // the same rows as (outer, inner) of the pair tensor
 #pragma unroll
@@ -246,52 +329,14 @@ __global__ __launch_bounds__(256, 2) void rowgemm_in_kernel(RowGemmInParams p) {
     cm_j[rb] = pc - cm_i[rb] * (uint32_t)p.n;
   }
 
-  const int nch = n_chunks<MODE>(p);
-  V8 pre[4];
-  auto fetch = [&](int ch) {
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int fid = wave * 4 + j;   // 16 fragments per chunk: tile = fid/8, kk = fid%8
-      const T* w;
-      int n_out, col0;
-      chunk_tile<T, MODE>(p, ch, fid >> 3, w, n_out, col0);
-      pre[j] = load_wfrag<T>(w, kC, n_out, col0, (fid & 7) * 16, lane);
-    }
-  };
-  auto stash = [&](int buf) {
-#pragma unroll
-    for (int j = 0; j < 4; ++j) lds_w[buf][wave * 4 + j][lane] = pre[j];
-  };
-  // bf16: the weight fragments go from global memory straight into their LDS slots.  The
-  // loads are invisible to the compiler's wait-count bookkeeping and are waited for by hand
-  // (end of the chunk loop), counting the stores issued after them: the compiler's own
-  // wait for a register-staged prefetch cannot count those stores across the loop edge and
-  // drains them all, which stalls every wave once per chunk until its previous chunk's stores
-  // have reached the L2.
-  constexpr bool kDma = sizeof(T) == 2;
-  auto dma = [&](int ch, int buf) {
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int fid = wave * 4 + j;
-      const T* w;
-      int n_out, col0;
-      chunk_tile<T, MODE>(p, ch, fid >> 3, w, n_out, col0);
-      const int col = min(col0 + (lane & 31), n_out - 1);   // as load_wfrag
-      load_to_lds16(w + (int64_t)col * kC + (fid & 7) * 16 + 8 * (lane >> 5),
-                    lds_address(&lds_w[buf][fid][0]));
-    }
-  };
-  T* const sink = reinterpret_cast<T*>(g_store_sink) + lane * C::VE;
-  if constexpr (kDma) {
-    dma(0, 0);
-    ring_barrier<0>();
-  } else {
+  if constexpr (!RES && !kDma) {
     fetch(0);
     stash(0);
     __syncthreads();
   }
 
   // Row-major store of the staged tile (major = row, minor = 32 output columns at col0).
+  // Lanes without a valid row store to the sink: the store count stays fixed.
   auto store_row_major = [&](const T* stg, T* outp, int64_t ld, int col0, int rb, const VE_t* resv) {
 #pragma unroll
     for (int ps = 0; ps < C::NPASS; ++ps) {
@@ -306,13 +351,11 @@ __global__ __launch_bounds__(256, 2) void rowgemm_in_kernel(RowGemmInParams p) {
   // (not unrolled: unrolled, the compiler hoists every chunk's loads to the top and spills them)
 #pragma clang loop unroll(disable)
   for (int ch = 0; ch < nch; ++ch) {
-    const int buf = C::NBUF == 2 ? (ch & 1) : 0;
-    if constexpr (kDma) {
-      // the other buffer was last read in the previous chunk, which every wave has left
-      if (ch + 1 < nch) dma(ch + 1, buf ^ 1);
-    } else {
-      fetch(min(ch + 1, nch - 1));   // unconditional: keeps the outstanding-load count static
-    }
+    const int buf = (!RES && C::NBUF == 2) ? (ch & 1) : 0;
+    if constexpr (!RES && !kDma) fetch(min(ch + 1, nch - 1));   // unconditional: static load count
+    // first fragment of this chunk's two weight tiles (the resident triangle bias is one tile)
+    const int wf0 = RES ? ch * 16 : buf * 16;
+    const int wf1 = wf0 + ((RES && MODE == kTriAttnIn && ch == 8) ? 0 : kKSteps);
     // kTriMulOut: the residual vectors of this chunk's columns, from the wave's LDS copy of z
     VE_t resv[RB][C::NPASS];
     if constexpr (MODE == kTriMulOut) {
@@ -342,8 +385,8 @@ __global__ __launch_bounds__(256, 2) void rowgemm_in_kernel(RowGemmInParams p) {
     if (chan_on_lanes) {
 #pragma unroll
       for (int kk = 0; kk < kKSteps; ++kk) {
-        const V8 w0 = lds_w[buf][kk][lane];
-        const V8 w1 = lds_w[buf][kKSteps + kk][lane];
+        const V8 w0 = lds_w[wf0 + kk][lane];
+        const V8 w1 = lds_w[wf1 + kk][lane];
 #pragma unroll
         for (int rb = 0; rb < RB; ++rb) {
           mma32(acc[rb][0], xf.f[rb][kk], w0);
@@ -353,8 +396,8 @@ __global__ __launch_bounds__(256, 2) void rowgemm_in_kernel(RowGemmInParams p) {
     } else {
 #pragma unroll
       for (int kk = 0; kk < kKSteps; ++kk) {
-        const V8 w0 = lds_w[buf][kk][lane];
-        const V8 w1 = lds_w[buf][kKSteps + kk][lane];
+        const V8 w0 = lds_w[wf0 + kk][lane];
+        const V8 w1 = lds_w[wf1 + kk][lane];
 #pragma unroll
         for (int rb = 0; rb < RB; ++rb) {
           if constexpr (MODE == kTriMulOut) {
@@ -368,59 +411,69 @@ __global__ __launch_bounds__(256, 2) void rowgemm_in_kernel(RowGemmInParams p) {
       }
     }
 
-    // The next chunk's weights go to the other LDS buffer now, before this chunk's stores
-    // are issued: waiting for those loads later would also wait for every store issued in
-    // between (memory operations retire in order).
-    if (!kDma && C::NBUF == 2) stash(buf ^ 1);
+    // fp32: the next chunk's weights go to LDS now, before this chunk's stores are issued:
+    // waiting for those loads later would also wait for every store issued in between
+    // (memory operations retire in order).
+    if (!RES && !kDma && C::NBUF == 2) stash(buf ^ 1);
 
     // ------------------------------ epilogues ------------------------------
     if constexpr (MODE == kTriMulIn) {
       // a/b[c][i][k] = mask * sigmoid(gate) * proj ; lane <-> channel, register <-> row
       T* outp = (T*)p.out[ch >> 2];
       const int c0 = (ch & 3) * 32;
-      wave_lds_sync();
+      const int n_rb = (p.n + 31) >> 5, n_ks = p.pitch >> 4;
+      constexpr int GT = NST < RB ? NST : RB;   // result tiles per LDS round trip
 #pragma unroll
-      for (int rb = 0; rb < RB; ++rb) {
-        float vals[16];
+      for (int rb0 = 0; rb0 < RB; rb0 += GT) {
+        wave_lds_sync();
 #pragma unroll
-        for (int qd = 0; qd < 4; ++qd) {
-          const f32x4 m4 = *reinterpret_cast<const f32x4*>(&lds_mask[wave][rb * 32 + 8 * qd + 4 * g]);
+        for (int q = 0; q < GT; ++q) {
+          const int rb = rb0 + q;
+          float vals[16];
 #pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            const int r = 4 * qd + e;
-            vals[r] = m4[e] * sigmoidf_fast(acc[rb][1][r]) * acc[rb][0][r];
+          for (int qd = 0; qd < 4; ++qd) {
+            const f32x4 m4 = *reinterpret_cast<const f32x4*>(&lds_mask[wave][rb * 32 + 8 * qd + 4 * g]);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const int r = 4 * qd + e;
+              vals[r] = m4[e] * sigmoidf_fast(acc[rb][1][r]) * acc[rb][0][r];
+            }
+          }
+          stage_put<T>(stile(q), vals, lane);
+        }
+        wave_lds_sync();
+        // fragment-ordered store: 8 consecutive inner indices of one outer index = the 16
+        // bytes of one operand lane (half-wave (pk0/8)%2, row outer%32)
+#pragma unroll
+        for (int q = 0; q < GT; ++q) {
+          const int rb = rb0 + q;
+#pragma unroll
+          for (int ps = 0; ps < C::NPASS; ++ps) {
+            int chn, r0;
+            stage_coord<T>(ps, lane, chn, r0);
+            const int i = pi0 + 4 * rb + (r0 >> 3);
+            const int64_t off = trimul_frag_offset(c0 + chn, i >> 5, pk0 >> 4, n_rb, n_ks) +
+                                ((pk0 >> 3) & 1) * 256 + (i & 31) * 8 + (r0 & 7);
+            *reinterpret_cast<VE_t*>(outp + off) = stage_get_vec<T>(stile(q), chn, r0);
           }
         }
-        stage_put<T>(stile(rb), vals, lane);
       }
-      wave_lds_sync();
-      // fragment-ordered store: 8 consecutive inner indices of one outer index = the 16
-      // bytes of one operand lane (half-wave (pk0/8)%2, row outer%32)
-      const int n_rb = (p.n + 31) >> 5, n_ks = p.pitch >> 4;
-#pragma unroll
-      for (int rb = 0; rb < RB; ++rb)
-#pragma unroll
-        for (int ps = 0; ps < C::NPASS; ++ps) {
-          int chn, r0;
-          stage_coord<T>(ps, lane, chn, r0);
-          const int i = pi0 + 4 * rb + (r0 >> 3);
-          const int64_t off = trimul_frag_offset(c0 + chn, i >> 5, pk0 >> 4, n_rb, n_ks) +
-                              ((pk0 >> 3) & 1) * 256 + (i & 31) * 8 + (r0 & 7);
-          *reinterpret_cast<VE_t*>(outp + off) = stage_get_vec<T>(stile(rb), chn, r0);
-        }
     } else if constexpr (MODE == kTriAttnIn) {
       // Outputs in the attention core's layouts (common.h): q and the gate head-major
       // [h][p][32], K / V^T / bias in fragment-ordered key tiles.
       const int which = ch >> 1;
       const int key_tiles = p.pitch >> 6;
-      // all result tiles of the chunk go to their staging tiles first ...
-      wave_lds_sync();
-      auto put_all = [&](auto kind) {   // kind: 0 = q (rounded, then scaled), 2 = gate, 1 = as is
-        constexpr int KIND = decltype(kind)::value;
+      const int q_blocks = (p.n + 31) >> 5;
+      constexpr int GT = NST < 2 * RB ? NST : 2 * RB;   // result tiles per LDS round trip
 #pragma unroll
-        for (int rb = 0; rb < RB; ++rb)
+      for (int k0 = 0; k0 < 2 * RB; k0 += GT) {
+        // the group's result tiles go to the staging tiles first ...
+        wave_lds_sync();
+        auto put_group = [&](auto kind) {   // kind: 0 = q (rounded, then scaled), 2 = gate, 1 = as is
+          constexpr int KIND = decltype(kind)::value;
 #pragma unroll
-          for (int t = 0; t < 2; ++t) {
+          for (int q = 0; q < GT; ++q) {
+            const int rb = (k0 + q) >> 1, t = (k0 + q) & 1;
             float vals[16];
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
@@ -429,33 +482,26 @@ __global__ __launch_bounds__(256, 2) void rowgemm_in_kernel(RowGemmInParams p) {
               if (KIND == 2) v = sigmoidf_fast(v);
               vals[r] = v;
             }
-            stage_put<T>(stile(rb * 2 + t), vals, lane);
+            stage_put<T>(stile(q), vals, lane);
           }
-      };
-      if (which == 0) put_all(std::integral_constant<int, 0>{});
-      else if (which == 2) put_all(std::integral_constant<int, 2>{});
-      else put_all(std::integral_constant<int, 1>{});
-      wave_lds_sync();
-      // ... and are then read back as 16-byte vectors and stored
-      if (which == 0 || which == 2) {
-        // q and sigmoid(g): one 32 x 32 tile = one head, head-major rows
+        };
+        if (which == 0) put_group(std::integral_constant<int, 0>{});
+        else if (which == 2) put_group(std::integral_constant<int, 2>{});
+        else put_group(std::integral_constant<int, 1>{});
+        wave_lds_sync();
+        // ... and are then read back as 16-byte vectors and stored
 #pragma unroll
-        for (int rb = 0; rb < RB; ++rb)
-#pragma unroll
-          for (int t = 0; t < 2; ++t) {
-            const int h = (ch & 1) * 2 + t;
-            store_row_major(stile(rb * 2 + t), (T*)p.out[which] + (int64_t)h * p.n_rows * 32, 32, 0,
-                            rb, nullptr);
-          }
-      } else if (which == 1) {
-        // K: staged row-major (major = key row, minor = d); each 16-byte d-chunk goes to
-        // its fragment slot
-        T* outp = (T*)p.out[1];
-#pragma unroll
-        for (int rb = 0; rb < RB; ++rb)
-#pragma unroll
-          for (int t = 0; t < 2; ++t) {
-            const int h = (ch & 1) * 2 + t;
+        for (int q = 0; q < GT; ++q) {
+          const int rb = (k0 + q) >> 1, t = (k0 + q) & 1;
+          const int h = (ch & 1) * 2 + t;
+          const T* stg = stile(q);
+          if (which == 0 || which == 2) {
+            // q and sigmoid(g): one 32 x 32 tile = one head, head-major rows
+            store_row_major(stg, (T*)p.out[which] + (int64_t)h * p.n_rows * 32, 32, 0, rb, nullptr);
+          } else if (which == 1) {
+            // K: staged row-major (major = key row, minor = d); each 16-byte d-chunk goes to
+            // its fragment slot
+            T* outp = (T*)p.out[1];
 #pragma unroll
             for (int ps = 0; ps < C::NPASS; ++ps) {
               int mj, m0;
@@ -463,26 +509,19 @@ __global__ __launch_bounds__(256, 2) void rowgemm_in_kernel(RowGemmInParams p) {
               *reinterpret_cast<VE_t*>(
                   rrow[rb][ps] >= 0
                       ? outp + attn_k_offset(h, rm_i[rb][ps], rm_j[rb][ps], m0, p.n, key_tiles)
-                      : sink) = stage_get_vec<T>(stile(rb * 2 + t), mj, m0);
+                      : sink) = stage_get_vec<T>(stg, mj, m0);
             }
-          }
-      } else {
-        // V^T (which == 3, major = channel d of head h) and the triangle bias (which == 4,
-        // major = head, logical row = (query i, key j)): vectors of VE consecutive keys
-        const int q_blocks = (p.n + 31) >> 5;
-#pragma unroll
-        for (int rb = 0; rb < RB; ++rb)
-#pragma unroll
-          for (int t = 0; t < 2; ++t) {
+          } else {
+            // V^T (which == 3, major = channel d of head h) and the triangle bias (which == 4,
+            // major = head, logical row = (query i, key j)): vectors of VE consecutive keys
             if (which == 4 && t == 1) continue;
-            const int h = (ch & 1) * 2 + t;
 #pragma unroll
             for (int ps = 0; ps < C::NPASS; ++ps) {
               int chn, r0;
               stage_coord<T>(ps, lane, chn, r0);
               const int64_t pr = row0 + rb * 32 + r0;
               if (which == 4 && chn >= p.aux) continue;
-              const VE_t v = stage_get_vec<T>(stile(rb * 2 + t), chn, r0);
+              const VE_t v = stage_get_vec<T>(stg, chn, r0);
               T* outp = (T*)p.out[which];
               if (vec_ok) {
                 const int64_t off =
@@ -508,6 +547,7 @@ __global__ __launch_bounds__(256, 2) void rowgemm_in_kernel(RowGemmInParams p) {
               }
             }
           }
+        }
       }
     } else if constexpr (MODE == kPairBias) {
       // bias[h][p], dense planes of n*n elements, fp32 or T; lane <-> head, register <-> row
@@ -542,7 +582,7 @@ __global__ __launch_bounds__(256, 2) void rowgemm_in_kernel(RowGemmInParams p) {
       }
     } else {
       // kTriMulOut: out[p][col] = [z +] (W_z LN_out(x)) * sigmoid(W_g LN_in(z)), row-major.
-      // out may alias z: a lane reads the residual vector it is about to overwrite.
+      // out may alias z: the residual comes from the copy of z made before any store.
 #pragma unroll
       for (int rb = 0; rb < RB; ++rb) {
         float vals[16];
@@ -558,17 +598,7 @@ __global__ __launch_bounds__(256, 2) void rowgemm_in_kernel(RowGemmInParams p) {
       }
     }
 
-    if constexpr (kDma) {
-      // The next chunk's weights must have landed: all but the stores this wave issued
-      // after requesting them (a lower bound on that count is what is safe; the triangle
-      // bias, whose store count varies, is the last chunk and has no successor).
-      constexpr int kStores = MODE == kTriMulIn    ? RB * C::NPASS
-                              : MODE == kTriAttnIn ? RB * 2 * C::NPASS
-                              : MODE == kTriMulOut ? RB * C::NPASS
-                                                   : 0;
-      if (MODE != kTriAttnIn || vec_ok) ring_barrier<kStores>();
-      else ring_barrier<0>();   // element-wise V^T stores: no fixed count
-    } else {
+    if constexpr (!RES && !kDma) {
       if (C::NBUF == 1) {
         __syncthreads();      // everyone is done reading the single buffer
         stash(0);
@@ -576,17 +606,35 @@ __global__ __launch_bounds__(256, 2) void rowgemm_in_kernel(RowGemmInParams p) {
       __syncthreads();
     }
   }
+    if (!RES) break;
+    tile += tile_step;
+  }
+}
+
+// Compute units of the current device (the resident kernels launch one workgroup per CU).
+static int device_cu_count() {
+  static int cache[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (cache[dev] == 0) {
+    int v = 0;
+    if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0)
+      v = 256;
+    cache[dev] = v;
+  }
+  return cache[dev];
 }
 
 template <typename T, int MODE>
 int launch_rowgemm_in(const RowGemmInParams& p, hipStream_t stream) {
+  typedef InCfg<T, MODE> IC;
   constexpr int RB = (sizeof(T) == 2 && MODE != kTriMulOut) ? 2 : 1;
-  const int64_t rows_per_block = 4 * RB * 32;
-  int64_t blocks = (p.n_rows + rows_per_block - 1) / rows_per_block;
-  if (MODE == kTriMulIn)   // 2-D patches: 16*RB outer x 8 inner indices per workgroup
-    blocks = (int64_t)((p.n + 16 * RB - 1) / (16 * RB)) * (p.pitch / 8);
-  if (blocks == 0) return 0;
-  rowgemm_in_kernel<T, RB, MODE><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(p);
+  int64_t tiles = (p.n_rows + RB * 32 - 1) / (RB * 32);   // wave tiles, as in the kernel
+  if (MODE == kTriMulIn) tiles = (int64_t)((p.n + 16 * RB - 1) / (16 * RB)) * (p.pitch / 8) * 4;
+  if (tiles == 0) return 0;
+  int64_t blocks = (tiles + 3) / 4;
+  if (IC::RES) blocks = std::min<int64_t>((tiles + IC::NW - 1) / IC::NW, device_cu_count());
+  rowgemm_in_kernel<T, RB, MODE><<<dim3((unsigned)blocks), dim3(IC::NW * 64), 0, stream>>>(p);
   return 0;
 }
 
