@@ -90,8 +90,9 @@ PTX_API int ptx_trimul_project(const void* z, const void* mask, const void* ln_w
                        float eps, int dtype, void* stream) {
   PTX_REQUIRE(dtype_ok(dtype), PTX_ERR_BAD_ARG, "trimul_project: unknown dtype %d", dtype);
   PTX_REQUIRE(n >= 0, PTX_ERR_BAD_ARG, "trimul_project: n=%d", n);
-  PTX_REQUIRE(c_z == 128 && c_hidden == 128, PTX_ERR_UNSUPPORTED,
-              "trimul_project: only c_z = c_hidden = 128 is built (got %d, %d)", c_z, c_hidden);
+  PTX_REQUIRE((c_z == 128 || c_z == 64) && c_hidden == 128, PTX_ERR_UNSUPPORTED,
+              "trimul_project: only c_z = 64 or 128 with c_hidden = 128 is built (got %d, %d)", c_z,
+              c_hidden);
   PTX_REQUIRE(k_pitch == ptx_key_pitch(n), PTX_ERR_BAD_ARG,
               "trimul_project: k_pitch=%d, expected ptx_key_pitch(%d)=%d", k_pitch, n,
               ptx_key_pitch(n));
@@ -104,7 +105,7 @@ PTX_API int ptx_trimul_project(const void* z, const void* mask, const void* ln_w
                   (!ln_b || aligned16(ln_b)),
               PTX_ERR_BAD_ARG, "trimul_project: pointers must be 16-byte aligned");
   PTX_DISPATCH(dtype, ptx::trimul_project<T>(z, mask, ln_w, ln_b, w_ap, w_ag, w_bp, w_bg, a, b, n,
-                                             k_pitch, incoming, eps, (hipStream_t)stream));
+                                             c_z, k_pitch, incoming, eps, (hipStream_t)stream));
   return after_launch("trimul_project");
 }
 
@@ -130,8 +131,9 @@ PTX_API int ptx_trimul_output(const void* x, const void* z, const void* ln_in_w,
                       float eps, int dtype, void* stream) {
   PTX_REQUIRE(dtype_ok(dtype), PTX_ERR_BAD_ARG, "trimul_output: unknown dtype %d", dtype);
   PTX_REQUIRE(n >= 0, PTX_ERR_BAD_ARG, "trimul_output: n=%d", n);
-  PTX_REQUIRE(c_z == 128 && c_hidden == 128, PTX_ERR_UNSUPPORTED,
-              "trimul_output: only c_z = c_hidden = 128 is built (got %d, %d)", c_z, c_hidden);
+  PTX_REQUIRE((c_z == 128 || c_z == 64) && c_hidden == 128, PTX_ERR_UNSUPPORTED,
+              "trimul_output: only c_z = 64 or 128 with c_hidden = 128 is built (got %d, %d)", c_z,
+              c_hidden);
   PTX_REQUIRE(n < 32768, PTX_ERR_UNSUPPORTED, "trimul_output: n=%d too large", n);
   if (n == 0) return PTX_OK;
   PTX_REQUIRE(x && z && ln_out_w && ln_out_b && w_z && w_g && out, PTX_ERR_BAD_ARG,
@@ -142,7 +144,7 @@ PTX_API int ptx_trimul_output(const void* x, const void* z, const void* ln_in_w,
                   (!ln_in_b || aligned16(ln_in_b)),
               PTX_ERR_BAD_ARG, "trimul_output: pointers must be 16-byte aligned");
   PTX_DISPATCH(dtype, ptx::trimul_output<T>(x, z, ln_in_w, ln_in_b, ln_out_w, ln_out_b, w_z, w_g,
-                                            out, n, add_residual, eps, (hipStream_t)stream));
+                                            out, n, c_z, add_residual, eps, (hipStream_t)stream));
   return after_launch("trimul_output");
 }
 
@@ -153,8 +155,9 @@ PTX_API int ptx_triattn_project(const void* z, const void* ln_w, const void* ln_
                         void* stream) {
   PTX_REQUIRE(dtype_ok(dtype), PTX_ERR_BAD_ARG, "triattn_project: unknown dtype %d", dtype);
   PTX_REQUIRE(n >= 0, PTX_ERR_BAD_ARG, "triattn_project: n=%d", n);
-  PTX_REQUIRE(c_in == 128 && d == 32 && heads == 4, PTX_ERR_UNSUPPORTED,
-              "triattn_project: only c_in=128, 4 heads x 32 is built (got c_in=%d heads=%d d=%d)",
+  PTX_REQUIRE((c_in == 128 || c_in == 64) && d == 32 && heads == 4, PTX_ERR_UNSUPPORTED,
+              "triattn_project: only c_in = 64 or 128, 4 heads x 32 is built (got c_in=%d heads=%d "
+              "d=%d)",
               c_in, heads, d);
   PTX_REQUIRE(key_pitch == ptx_key_pitch(n), PTX_ERR_BAD_ARG,
               "triattn_project: key_pitch=%d, expected %d", key_pitch, ptx_key_pitch(n));
@@ -169,7 +172,7 @@ PTX_API int ptx_triattn_project(const void* z, const void* ln_w, const void* ln_
                   (!ln_b || aligned16(ln_b)),
               PTX_ERR_BAD_ARG, "triattn_project: pointers must be 16-byte aligned");
   PTX_DISPATCH(dtype, ptx::triattn_project<T>(z, ln_w, ln_b, w_q, w_k, w_v, w_g, w_b, q, k, vt, g,
-                                              tri_bias, n, heads, d, key_pitch, transposed, eps,
+                                              tri_bias, n, c_in, heads, d, key_pitch, transposed, eps,
                                               (hipStream_t)stream));
   return after_launch("triattn_project");
 }
@@ -198,8 +201,8 @@ PTX_API int ptx_triattn_output(const void* o, const void* w_o, const void* z, vo
                        int transposed, int add_residual, int dtype, void* stream) {
   PTX_REQUIRE(dtype_ok(dtype), PTX_ERR_BAD_ARG, "triattn_output: unknown dtype %d", dtype);
   PTX_REQUIRE(n >= 0, PTX_ERR_BAD_ARG, "triattn_output: n=%d", n);
-  PTX_REQUIRE(c_in == 128, PTX_ERR_UNSUPPORTED, "triattn_output: only c_in=128 is built (got %d)",
-              c_in);
+  PTX_REQUIRE(c_in == 128 || c_in == 64, PTX_ERR_UNSUPPORTED,
+              "triattn_output: only c_in = 64 or 128 is built (got %d)", c_in);
   PTX_REQUIRE(n < 32768, PTX_ERR_UNSUPPORTED, "triattn_output: n=%d too large", n);
   if (n == 0) return PTX_OK;
   PTX_REQUIRE(o && w_o && out && (!add_residual || z), PTX_ERR_BAD_ARG,
@@ -207,7 +210,7 @@ PTX_API int ptx_triattn_output(const void* o, const void* w_o, const void* z, vo
   PTX_REQUIRE(aligned16(o) && aligned16(w_o) && aligned16(out) && (!z || aligned16(z)),
               PTX_ERR_BAD_ARG,
               "triattn_output: pointers must be 16-byte aligned");
-  PTX_DISPATCH(dtype, ptx::triattn_output<T>(o, w_o, z, out, n, transposed, add_residual,
+  PTX_DISPATCH(dtype, ptx::triattn_output<T>(o, w_o, z, out, n, c_in, transposed, add_residual,
                                              (hipStream_t)stream));
   return after_launch("triattn_output");
 }
@@ -221,12 +224,16 @@ PTX_API int ptx_transition_pack(const void* w_a, const void* w_b, const void* w_
                         int n_factor, int dtype, void* stream) {
   PTX_REQUIRE(dtype_ok(dtype), PTX_ERR_BAD_ARG, "transition_pack: unknown dtype %d", dtype);
   PTX_REQUIRE(n_factor > 0, PTX_ERR_BAD_ARG, "transition_pack: n_factor=%d", n_factor);
-  PTX_REQUIRE(c == 128, PTX_ERR_UNSUPPORTED, "transition_pack: only c=128 is built (got %d)", c);
+  PTX_REQUIRE(c == 128 || c == 64, PTX_ERR_UNSUPPORTED,
+              "transition_pack: only c = 64 or 128 is built (got %d)", c);
+  PTX_REQUIRE((n_factor * c) % 64 == 0, PTX_ERR_UNSUPPORTED,
+              "transition_pack: the hidden width %d is not a multiple of 64", n_factor * c);
   PTX_REQUIRE(n_factor <= 64, PTX_ERR_UNSUPPORTED, "transition_pack: n_factor=%d too large",
               n_factor);
   PTX_REQUIRE(w_a && w_b && w_o && packed, PTX_ERR_BAD_ARG, "transition_pack: null pointer");
   PTX_REQUIRE(aligned16(packed), PTX_ERR_BAD_ARG, "transition_pack: packed must be 16-byte aligned");
-  PTX_DISPATCH(dtype, ptx::transition_pack<T>(w_a, w_b, w_o, packed, n_factor, (hipStream_t)stream));
+  PTX_DISPATCH(dtype, ptx::transition_pack<T>(w_a, w_b, w_o, packed, c, n_factor,
+                                              (hipStream_t)stream));
   return after_launch("transition_pack");
 }
 
@@ -236,7 +243,10 @@ PTX_API int ptx_transition_fwd(const void* x, const void* ln_w, const void* ln_b
   PTX_REQUIRE(dtype_ok(dtype), PTX_ERR_BAD_ARG, "transition: unknown dtype %d", dtype);
   PTX_REQUIRE(rows >= 0 && n_factor > 0, PTX_ERR_BAD_ARG, "transition: rows=%lld n_factor=%d",
               (long long)rows, n_factor);
-  PTX_REQUIRE(c == 128, PTX_ERR_UNSUPPORTED, "transition: only c=128 is built (got %d)", c);
+  PTX_REQUIRE(c == 128 || c == 64, PTX_ERR_UNSUPPORTED,
+              "transition: only c = 64 or 128 is built (got %d)", c);
+  PTX_REQUIRE((n_factor * c) % 64 == 0, PTX_ERR_UNSUPPORTED,
+              "transition: the hidden width %d is not a multiple of 64", n_factor * c);
   PTX_REQUIRE(n_factor <= 64, PTX_ERR_UNSUPPORTED, "transition: n_factor=%d too large", n_factor);
   PTX_REQUIRE(rows < ((int64_t)1 << 30), PTX_ERR_UNSUPPORTED, "transition: rows=%lld too large",
               (long long)rows);
@@ -245,7 +255,7 @@ PTX_API int ptx_transition_fwd(const void* x, const void* ln_w, const void* ln_b
   PTX_REQUIRE(aligned16(x) && aligned16(packed) && aligned16(out) && (!ln_w || aligned16(ln_w)) &&
                   (!ln_b || aligned16(ln_b)),
               PTX_ERR_BAD_ARG, "transition: pointers must be 16-byte aligned");
-  PTX_DISPATCH(dtype, ptx::transition_fwd<T>(x, ln_w, ln_b, packed, out, rows, n_factor,
+  PTX_DISPATCH(dtype, ptx::transition_fwd<T>(x, ln_w, ln_b, packed, out, rows, c, n_factor,
                                              add_residual, eps, (hipStream_t)stream));
   return after_launch("transition");
 }

@@ -1,5 +1,6 @@
 // Host-callable launchers, one per kernel family; api.hip validates arguments
-// and dispatches on dtype.  All return 0 after enqueueing on `stream`.
+// and dispatches on dtype.  c_z / c: channels of a pair-tensor row, 64 or 128 (the hidden
+// widths - c_hidden_mul, heads * d - are 128).  All return 0 after enqueueing on `stream`.
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -13,26 +14,27 @@ int layernorm_fwd(const T* x, const T* gamma, const T* beta, T* y, float* mean, 
 template <typename T>
 int trimul_project(const void* z, const void* mask, const void* ln_w, const void* ln_b,
                    const void* w_ap, const void* w_ag, const void* w_bp, const void* w_bg, void* a,
-                   void* b, int n, int k_pitch, int incoming, float eps, hipStream_t stream);
+                   void* b, int n, int c_z, int k_pitch, int incoming, float eps,
+                   hipStream_t stream);
 template <typename T>
 int trimul_output(const void* x, const void* z, const void* ln_in_w, const void* ln_in_b,
                   const void* ln_out_w, const void* ln_out_b, const void* w_z, const void* w_g,
-                  void* out, int n, int add_residual, float eps, hipStream_t stream);
+                  void* out, int n, int c_z, int add_residual, float eps, hipStream_t stream);
 template <typename T>
 int triattn_project(const void* z, const void* ln_w, const void* ln_b, const void* w_q,
                     const void* w_k, const void* w_v, const void* w_g, const void* w_b, void* q,
-                    void* k, void* vt, void* g, void* tri_bias, int n, int heads, int d,
+                    void* k, void* vt, void* g, void* tri_bias, int n, int c_z, int heads, int d,
                     int key_pitch, int transposed, float eps, hipStream_t stream);
 template <typename T>
-int triattn_output(const void* o, const void* w_o, const void* z, void* out, int n, int transposed,
-                   int add_residual, hipStream_t stream);
-// transition weights -> fragment-ordered chunks of 32 hidden (3 * n_factor*128 * 128 elements)
+int triattn_output(const void* o, const void* w_o, const void* z, void* out, int n, int c_z,
+                   int transposed, int add_residual, hipStream_t stream);
+// transition weights -> fragment-ordered chunks of 32 hidden (3 * n_factor*c * c elements)
 template <typename T>
-int transition_pack(const void* w_a, const void* w_b, const void* w_o, void* packed, int n_factor,
-                    hipStream_t stream);
+int transition_pack(const void* w_a, const void* w_b, const void* w_o, void* packed, int c,
+                    int n_factor, hipStream_t stream);
 template <typename T>
 int transition_fwd(const void* x, const void* ln_w, const void* ln_b, const void* packed,
-                   void* out, int64_t rows, int n_factor, int add_residual, float eps,
+                   void* out, int64_t rows, int c, int n_factor, int add_residual, float eps,
                    hipStream_t stream);
 template <typename T>
 int pair_bias_fwd(const void* z, const void* ln_w, const void* ln_b, const void* w, void* bias,

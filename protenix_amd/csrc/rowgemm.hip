@@ -59,18 +59,13 @@ enum RowGemmInMode { kTriMulIn = 0, kTriAttnIn = 1, kPairBias = 3, kTriMulOut = 
 // per chunk a constant, which the weight ring below counts on.
 static __device__ __attribute__((aligned(16))) uint32_t g_store_sink[kWave * 4];
 
-template <int MODE>
-__device__ __forceinline__ int n_chunks(const RowGemmInParams& p) {
-  if (MODE == kTriMulIn) return 8;                 // {a,b} x 4 channel blocks
-  if (MODE == kTriAttnIn) return 9;                // q,k,g,v: 2 chunks each; bias: 1
-  if (MODE == kPairBias) return 1;
-  return 4;                                        // kTriMulOut: 4 column blocks
-}
-
-// Weight matrix, its row count and first row for tile `t` (0/1) of chunk `ch`.
-template <typename T, int MODE>
+// Weight matrix, its row count, first row, row length and K steps for tile `t` (0/1) of
+// chunk `ch`.  KS = K steps of a pair-tensor row (c_z / 16); the hidden widths are 128.
+template <typename T, int MODE, int KS>
 __device__ __forceinline__ void chunk_tile(const RowGemmInParams& p, int ch, int t, const T*& w,
-                                           int& n_out, int& col0) {
+                                           int& n_out, int& col0, int& ldw, int& ksteps) {
+  ldw = 16 * KS;
+  ksteps = KS;
   if (MODE == kTriMulIn) {            // w: ap, ag, bp, bg ; tile0 = projection, tile1 = gate
     w = (const T*)p.w[(ch >> 2) * 2 + t];
     n_out = kC;
@@ -84,10 +79,14 @@ __device__ __forceinline__ void chunk_tile(const RowGemmInParams& p, int ch, int
     w = (const T*)p.w[0];
     n_out = p.aux & 0xff;
     col0 = 0;
-  } else {                            // kTriMulOut: w: z, g
+  } else {                            // kTriMulOut: w: z [c_z][128], g [c_z][c_z]
     w = (const T*)p.w[t];
-    n_out = kC;
+    n_out = 16 * KS;
     col0 = ch * 32;
+    if (t == 0) {
+      ldw = kC;
+      ksteps = kKSteps;
+    }
   }
 }
 
@@ -98,23 +97,25 @@ __device__ __forceinline__ void chunk_tile(const RowGemmInParams& p, int ch, int
 // many bytes of weights through the L2 as it moves pair-tensor data, and every wave's wait
 // for its share of them also waits for the stores it issued before.)  fp32 weights are twice
 // the size and do not fit: that path stages one chunk at a time through registers.
-template <typename T, int MODE> struct InCfg {
+template <typename T, int MODE, int KS> struct InCfg {
   static constexpr bool RES = sizeof(T) == 2 && MODE != kPairBias;
   static constexpr int NW = RES ? 8 : 4;   // waves per workgroup
+  // chunks of two 32-column weight tiles: {a,b} x 4 channel blocks | q,k,g,v: 2 each, bias: 1 |
+  // the pair bias | c_z / 32 output column blocks
   static constexpr int NCH =
-      MODE == kTriMulIn ? 8 : MODE == kTriAttnIn ? 9 : MODE == kPairBias ? 1 : 4;
+      MODE == kTriMulIn ? 8 : MODE == kTriAttnIn ? 9 : MODE == kPairBias ? 1 : KS / 2;
   // weight fragments held in LDS (16 per chunk; the resident triangle bias is one tile of 8)
   static constexpr int NFRAG =
       RES ? (MODE == kTriAttnIn ? 8 * 16 + 8 : NCH * 16) : Cfg<T>::NBUF * 16;
 };
 
-template <typename T, int RB, int MODE>
-__global__ __launch_bounds__((InCfg<T, MODE>::NW * 64), (InCfg<T, MODE>::RES ? 1 : 2)) void
+template <typename T, int RB, int MODE, int KS>
+__global__ __launch_bounds__((InCfg<T, MODE, KS>::NW * 64), (InCfg<T, MODE, KS>::RES ? 1 : 2)) void
 rowgemm_in_kernel(RowGemmInParams p) {
   typedef typename Vec8<T>::type V8;
   typedef typename VecE<T>::type VE_t;
   typedef Cfg<T> C;
-  typedef InCfg<T, MODE> IC;
+  typedef InCfg<T, MODE, KS> IC;
   constexpr bool RES = IC::RES;
   constexpr int NW = IC::NW;
   __shared__ V8 lds_w[IC::NFRAG][kWave];
@@ -124,7 +125,8 @@ rowgemm_in_kernel(RowGemmInParams p) {
   constexpr int NST = (RES || MODE == kTriMulOut) ? 1 : 2 * RB;
   // kTriMulOut: the raw z rows of this wave, kept for the residual add (re-reading them from
   // HBM at the end costs a full extra pass: by then they have left the L2)
-  constexpr int kResPitch = kC + 16 / (int)sizeof(T);
+  constexpr int kCz = 16 * KS;   // channels of a pair-tensor row
+  constexpr int kResPitch = kCz + 16 / (int)sizeof(T);
   __shared__ __attribute__((aligned(16))) T lds_res[MODE == kTriMulOut ? NW : 1][MODE == kTriMulOut ? RB * 32 : 1][kResPitch];
   __shared__ __attribute__((aligned(16))) T lds_stage[NW][NST][32 * C::PITCH];
   __shared__ __attribute__((aligned(16))) float lds_mask[MODE == kTriMulIn ? NW : 1][RB * 32];
@@ -134,7 +136,7 @@ rowgemm_in_kernel(RowGemmInParams p) {
   auto stile = [&](int k) { return lds_stage[wave][k]; };
   const bool vec_ok = (p.n % C::VE) == 0;   // channel-major vectors stay inside one plane row
   T* const sink = reinterpret_cast<T*>(g_store_sink) + lane * C::VE;
-  const int nch = n_chunks<MODE>(p);
+  constexpr int nch = IC::NCH;
 
   // Work units ("wave tiles").  kTriMulIn works on 2-D patches of the pair tensor instead of
   // runs of logical rows: four waves cover 16*RB outer indices x 8 inner indices, a row block
@@ -156,10 +158,11 @@ rowgemm_in_kernel(RowGemmInParams p) {
   // are waited for by hand.
   auto dma_frag = [&](int f_src, int f_dst) {
     const T* w;
-    int n_out, col0;
-    chunk_tile<T, MODE>(p, f_src >> 4, (f_src >> 3) & 1, w, n_out, col0);
+    int n_out, col0, ldw, ksteps;
+    chunk_tile<T, MODE, KS>(p, f_src >> 4, (f_src >> 3) & 1, w, n_out, col0, ldw, ksteps);
+    if ((f_src & 7) >= ksteps) return;   // narrow rows: the slot stays unused
     const int col = min(col0 + (lane & 31), n_out - 1);   // as load_wfrag
-    load_to_lds16(w + (int64_t)col * kC + (f_src & 7) * 16 + 8 * (lane >> 5),
+    load_to_lds16(w + (int64_t)col * ldw + (f_src & 7) * 16 + 8 * (lane >> 5),
                   lds_address(&lds_w[f_dst][0]));
   };
   constexpr bool kDma = sizeof(T) == 2 && !RES;   // bf16 pair bias: its single chunk
@@ -179,9 +182,10 @@ rowgemm_in_kernel(RowGemmInParams p) {
     for (int j = 0; j < 4; ++j) {
       const int fid = wave * 4 + j;   // 16 fragments per chunk: tile = fid/8, kk = fid%8
       const T* w;
-      int n_out, col0;
-      chunk_tile<T, MODE>(p, ch, fid >> 3, w, n_out, col0);
-      pre[j] = load_wfrag<T>(w, kC, n_out, col0, (fid & 7) * 16, lane);
+      int n_out, col0, ldw, ksteps;
+      chunk_tile<T, MODE, KS>(p, ch, fid >> 3, w, n_out, col0, ldw, ksteps);
+      // (K steps beyond a narrow row re-read the last one: their slots are never used)
+      pre[j] = load_wfrag<T>(w, ldw, n_out, col0, min(fid & 7, ksteps - 1) * 16, lane);
     }
   };
   auto stash = [&](int buf) {
@@ -207,7 +211,7 @@ rowgemm_in_kernel(RowGemmInParams p) {
     const T* beta2 = (const T*)p.beta2;
     if constexpr (RES) asm volatile("" : "+s"(gamma), "+s"(beta), "+s"(gamma2), "+s"(beta2));
 
-  RowFrags<T, RB> xf;
+  RowFrags<T, RB, KS> xf;
   if constexpr (MODE == kTriMulIn) {
     int64_t off[RB];
 #pragma unroll
@@ -217,14 +221,14 @@ rowgemm_in_kernel(RowGemmInParams p) {
     }
     load_rows_at<T, RB, true>(xf, (const T*)p.x, off, gamma, beta, p.eps, lane);
   } else if constexpr (MODE == kTriMulOut) {
-    RowFrags<T, RB> zraw;
+    RowFrags<T, RB, KS> zraw;
     load_rows<T, RB, false>(zraw, (const T*)p.x, p.xmap, row0, p.n_rows, nullptr, nullptr, 0.0f,
                             lane);
     wave_lds_sync();   // the previous tile's residual reads are done
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb) {
 #pragma unroll
-      for (int kk = 0; kk < kKSteps; ++kk)
+      for (int kk = 0; kk < KS; ++kk)
         store8<T>(&lds_res[wave][rb * 32 + n][16 * kk + 8 * g], zraw.f[rb][kk]);
       normalize_raw<T>(zraw.f[rb], gamma, beta, p.eps, g, xf.f[rb]);
     }
@@ -384,7 +388,7 @@ rowgemm_in_kernel(RowGemmInParams p) {
 
     if (chan_on_lanes) {
 #pragma unroll
-      for (int kk = 0; kk < kKSteps; ++kk) {
+      for (int kk = 0; kk < KS; ++kk) {
         const V8 w0 = lds_w[wf0 + kk][lane];
         const V8 w1 = lds_w[wf1 + kk][lane];
 #pragma unroll
@@ -393,20 +397,27 @@ rowgemm_in_kernel(RowGemmInParams p) {
           mma32(acc[rb][1], xf.f[rb][kk], w1);
         }
       }
-    } else {
+    } else if constexpr (MODE == kTriMulOut) {
 #pragma unroll
       for (int kk = 0; kk < kKSteps; ++kk) {
+        const V8 w0 = lds_w[wf0 + kk][lane];
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) mma32(acc[rb][0], w0, xf2.f[rb][kk]);   // W_z LN_out(x)
+        if (kk < KS) {
+          const V8 w1 = lds_w[wf1 + kk][lane];
+#pragma unroll
+          for (int rb = 0; rb < RB; ++rb) mma32(acc[rb][1], w1, xf.f[rb][kk]);  // W_g LN_in(z)
+        }
+      }
+    } else {
+#pragma unroll
+      for (int kk = 0; kk < KS; ++kk) {
         const V8 w0 = lds_w[wf0 + kk][lane];
         const V8 w1 = lds_w[wf1 + kk][lane];
 #pragma unroll
         for (int rb = 0; rb < RB; ++rb) {
-          if constexpr (MODE == kTriMulOut) {
-            mma32(acc[rb][0], w0, xf2.f[rb][kk]);   // W_z LN_out(x)
-            mma32(acc[rb][1], w1, xf.f[rb][kk]);    // W_g LN_in(z)
-          } else {
-            mma32(acc[rb][0], w0, xf.f[rb][kk]);
-            mma32(acc[rb][1], w1, xf.f[rb][kk]);
-          }
+          mma32(acc[rb][0], w0, xf.f[rb][kk]);
+          mma32(acc[rb][1], w1, xf.f[rb][kk]);
         }
       }
     }
@@ -594,7 +605,7 @@ rowgemm_in_kernel(RowGemmInParams p) {
         wave_lds_sync();
         stage_put<T>(st, vals, lane);
         wave_lds_sync();
-        store_row_major(st, (T*)p.out[0], kC, ch * 32, rb, p.add_residual ? resv[rb] : nullptr);
+        store_row_major(st, (T*)p.out[0], kCz, ch * 32, rb, p.add_residual ? resv[rb] : nullptr);
       }
     }
 
@@ -625,16 +636,16 @@ static int device_cu_count() {
   return cache[dev];
 }
 
-template <typename T, int MODE>
+template <typename T, int MODE, int KS>
 int launch_rowgemm_in(const RowGemmInParams& p, hipStream_t stream) {
-  typedef InCfg<T, MODE> IC;
+  typedef InCfg<T, MODE, KS> IC;
   constexpr int RB = (sizeof(T) == 2 && MODE != kTriMulOut) ? 2 : 1;
   int64_t tiles = (p.n_rows + RB * 32 - 1) / (RB * 32);   // wave tiles, as in the kernel
   if (MODE == kTriMulIn) tiles = (int64_t)((p.n + 16 * RB - 1) / (16 * RB)) * (p.pitch / 8) * 4;
   if (tiles == 0) return 0;
   int64_t blocks = (tiles + 3) / 4;
   if (IC::RES) blocks = std::min<int64_t>((tiles + IC::NW - 1) / IC::NW, device_cu_count());
-  rowgemm_in_kernel<T, RB, MODE><<<dim3((unsigned)blocks), dim3(IC::NW * 64), 0, stream>>>(p);
+  rowgemm_in_kernel<T, RB, MODE, KS><<<dim3((unsigned)blocks), dim3(IC::NW * 64), 0, stream>>>(p);
   return 0;
 }
 
@@ -654,7 +665,8 @@ struct RowGemmOutParams {
   int64_t n_rows;
 };
 
-template <typename T, int RB>
+// NOB = output column blocks of 32 (c_z / 32).
+template <typename T, int RB, int NOB>
 __global__ __launch_bounds__(256, 2) void rowgemm_out_kernel(RowGemmOutParams p) {
   typedef typename Vec8<T>::type V8;
   typedef typename VecE<T>::type VE_t;
@@ -667,22 +679,24 @@ __global__ __launch_bounds__(256, 2) void rowgemm_out_kernel(RowGemmOutParams p)
   const T* w = (const T*)p.w;
   T* st = lds_stage[wave];
 
-  f32x16 acc[RB][4];
+  f32x16 acc[RB][NOB];
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
-    for (int t = 0; t < 4; ++t)
+    for (int t = 0; t < NOB; ++t)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[rb][t][r] = 0.0f;
 
-  // chunk c -> (slab = c/2, column pair = c%2); one slab (two chunks) per outer iteration
+  // chunk c -> (slab = c / NH, column pair = c % NH), NH = NOB/2 chunks per slab; one slab
+  // per outer iteration
+  constexpr int NH = NOB / 2;
   V8 pre[4];
   auto fetch = [&](int ch) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int fid = wave * 4 + j;
-      const int col0 = ((ch & 1) * 2 + (fid >> 3)) * 32;
-      pre[j] = load_wfrag<T>(w, K, kC, col0, (ch >> 1) * kC + (fid & 7) * 16, lane);
+      const int col0 = ((ch % NH) * 2 + (fid >> 3)) * 32;
+      pre[j] = load_wfrag<T>(w, K, 32 * NOB, col0, (ch / NH) * kC + (fid & 7) * 16, lane);
     }
   };
   auto stash = [&](int buf) {
@@ -694,7 +708,7 @@ __global__ __launch_bounds__(256, 2) void rowgemm_out_kernel(RowGemmOutParams p)
   __syncthreads();
 
   const RowMap amap{(int64_t)K, 0, 1};   // row p -> p*K (n_inner = 1, so outer = p)
-  const int nch = 2 * p.n_slab;
+  const int nch = NH * p.n_slab;
   for (int slab = 0; slab < p.n_slab; ++slab) {
     RowFrags<T, RB> af;
     if (p.a_head_major) {
@@ -714,9 +728,9 @@ __global__ __launch_bounds__(256, 2) void rowgemm_out_kernel(RowGemmOutParams p)
                               nullptr, 0.0f, lane);
     }
 #pragma unroll
-    for (int half = 0; half < 2; ++half) {
-      const int ch = 2 * slab + half;
-      const int buf = C::NBUF == 2 ? half : 0;
+    for (int half = 0; half < NH; ++half) {
+      const int ch = NH * slab + half;
+      const int buf = C::NBUF == 2 ? (ch & 1) : 0;
       fetch(min(ch + 1, nch - 1));
 #pragma unroll
       for (int kk = 0; kk < kKSteps; ++kk) {
@@ -741,7 +755,7 @@ __global__ __launch_bounds__(256, 2) void rowgemm_out_kernel(RowGemmOutParams p)
   T* outp = (T*)p.out;
   const T* resp = (const T*)p.res;
   int64_t obase[RB][C::NPASS];
-  VE_t resv[RB][4][C::NPASS];
+  VE_t resv[RB][NOB][C::NPASS];
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
@@ -755,7 +769,7 @@ __global__ __launch_bounds__(256, 2) void rowgemm_out_kernel(RowGemmOutParams p)
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
-      for (int t = 0; t < 4; ++t)
+      for (int t = 0; t < NOB; ++t)
 #pragma unroll
         for (int ps = 0; ps < C::NPASS; ++ps)
           if (obase[rb][ps] >= 0)
@@ -764,7 +778,7 @@ __global__ __launch_bounds__(256, 2) void rowgemm_out_kernel(RowGemmOutParams p)
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
 #pragma unroll
-    for (int t = 0; t < 4; ++t) {
+    for (int t = 0; t < NOB; ++t) {
       float vals[16];
 #pragma unroll
       for (int r = 0; r < 16; ++r) vals[r] = acc[rb][t][r];
@@ -785,13 +799,13 @@ __global__ __launch_bounds__(256, 2) void rowgemm_out_kernel(RowGemmOutParams p)
   }
 }
 
-template <typename T>
+template <typename T, int NOB>
 int launch_rowgemm_out(const RowGemmOutParams& p, hipStream_t stream) {
   constexpr int RB = sizeof(T) == 2 ? 2 : 1;
   const int64_t rows_per_block = 4 * RB * 32;
   const int64_t blocks = (p.n_rows + rows_per_block - 1) / rows_per_block;
   if (blocks == 0) return 0;
-  rowgemm_out_kernel<T, RB><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(p);
+  rowgemm_out_kernel<T, RB, NOB><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(p);
   return 0;
 }
 
@@ -809,10 +823,11 @@ static RowMap pair_map(int n, int c, bool transposed) {
 template <typename T>
 int trimul_project(const void* z, const void* mask, const void* ln_w, const void* ln_b,
                    const void* w_ap, const void* w_ag, const void* w_bp, const void* w_bg, void* a,
-                   void* b, int n, int k_pitch, int incoming, float eps, hipStream_t stream) {
+                   void* b, int n, int c_z, int k_pitch, int incoming, float eps,
+                   hipStream_t stream) {
   RowGemmInParams p = {};
   p.x = z;
-  p.xmap = pair_map(n, kC, incoming != 0);
+  p.xmap = pair_map(n, c_z, incoming != 0);
   p.n_rows = (int64_t)n * n;
   p.gamma = ln_w;
   p.beta = ln_b;
@@ -823,16 +838,17 @@ int trimul_project(const void* z, const void* mask, const void* ln_w, const void
   p.mmap = pair_map(n, 1, incoming != 0);
   p.n = n;
   p.pitch = k_pitch;
-  return launch_rowgemm_in<T, kTriMulIn>(p, stream);
+  return c_z == 64 ? launch_rowgemm_in<T, kTriMulIn, 4>(p, stream)
+                   : launch_rowgemm_in<T, kTriMulIn, 8>(p, stream);
 }
 
 template <typename T>
 int trimul_output(const void* x, const void* z, const void* ln_in_w, const void* ln_in_b,
                   const void* ln_out_w, const void* ln_out_b, const void* w_z, const void* w_g,
-                  void* out, int n, int add_residual, float eps, hipStream_t stream) {
+                  void* out, int n, int c_z, int add_residual, float eps, hipStream_t stream) {
   RowGemmInParams p = {};
   p.x = z;
-  p.xmap = pair_map(n, kC, false);
+  p.xmap = pair_map(n, c_z, false);
   p.n_rows = (int64_t)n * n;
   p.gamma = ln_in_w;
   p.beta = ln_in_b;
@@ -844,17 +860,18 @@ int trimul_output(const void* x, const void* z, const void* ln_in_w, const void*
   p.gamma2 = ln_out_w;
   p.beta2 = ln_out_b;
   p.add_residual = add_residual;
-  return launch_rowgemm_in<T, kTriMulOut>(p, stream);
+  return c_z == 64 ? launch_rowgemm_in<T, kTriMulOut, 4>(p, stream)
+                   : launch_rowgemm_in<T, kTriMulOut, 8>(p, stream);
 }
 
 template <typename T>
 int triattn_project(const void* z, const void* ln_w, const void* ln_b, const void* w_q,
                     const void* w_k, const void* w_v, const void* w_g, const void* w_b, void* q,
-                    void* k, void* vt, void* g, void* tri_bias, int n, int heads, int d,
+                    void* k, void* vt, void* g, void* tri_bias, int n, int c_z, int heads, int d,
                     int key_pitch, int transposed, float eps, hipStream_t stream) {
   RowGemmInParams p = {};
   p.x = z;
-  p.xmap = pair_map(n, kC, transposed != 0);
+  p.xmap = pair_map(n, c_z, transposed != 0);
   p.n_rows = (int64_t)n * n;
   p.gamma = ln_w;
   p.beta = ln_b;
@@ -865,12 +882,13 @@ int triattn_project(const void* z, const void* ln_w, const void* ln_b, const voi
   p.aux = heads;
   p.pitch = key_pitch;
   p.q_scale = 1.0f / sqrtf((float)d);
-  return launch_rowgemm_in<T, kTriAttnIn>(p, stream);
+  return c_z == 64 ? launch_rowgemm_in<T, kTriAttnIn, 4>(p, stream)
+                   : launch_rowgemm_in<T, kTriAttnIn, 8>(p, stream);
 }
 
 template <typename T>
-int triattn_output(const void* o, const void* w_o, const void* z, void* out, int n, int transposed,
-                   int add_residual, hipStream_t stream) {
+int triattn_output(const void* o, const void* w_o, const void* z, void* out, int n, int c_z,
+                   int transposed, int add_residual, hipStream_t stream) {
   RowGemmOutParams p = {};
   p.a = o;
   p.a_head_major = 1;
@@ -878,9 +896,9 @@ int triattn_output(const void* o, const void* w_o, const void* z, void* out, int
   p.w = w_o;
   p.res = add_residual ? z : nullptr;
   p.out = out;
-  p.omap = pair_map(n, kC, transposed != 0);
+  p.omap = pair_map(n, c_z, transposed != 0);
   p.n_rows = (int64_t)n * n;
-  return launch_rowgemm_out<T>(p, stream);
+  return c_z == 64 ? launch_rowgemm_out<T, 2>(p, stream) : launch_rowgemm_out<T, 4>(p, stream);
 }
 
 template <typename T>
@@ -897,20 +915,21 @@ int pair_bias_fwd(const void* z, const void* ln_w, const void* ln_b, const void*
   p.out[0] = bias;
   p.n = n;
   p.aux = heads | (out_f32 ? 0x100 : 0);
-  return launch_rowgemm_in<T, kPairBias>(p, stream);
+  return launch_rowgemm_in<T, kPairBias, 8>(p, stream);
 }
 
 #define PTX_INSTANTIATE(T)                                                                          \
   template int trimul_project<T>(const void*, const void*, const void*, const void*, const void*,  \
                                  const void*, const void*, const void*, void*, void*, int, int,    \
-                                 int, float, hipStream_t);                                         \
+                                 int, int, float, hipStream_t);                                    \
   template int trimul_output<T>(const void*, const void*, const void*, const void*, const void*,   \
-                                const void*, const void*, const void*, void*, int, int, float,     \
-                                hipStream_t);                                                      \
+                                const void*, const void*, const void*, void*, int, int, int,       \
+                                float, hipStream_t);                                               \
   template int triattn_project<T>(const void*, const void*, const void*, const void*, const void*, \
                                   const void*, const void*, const void*, void*, void*, void*,      \
-                                  void*, void*, int, int, int, int, int, float, hipStream_t);      \
-  template int triattn_output<T>(const void*, const void*, const void*, void*, int, int, int,      \
+                                  void*, void*, int, int, int, int, int, int, float,               \
+                                  hipStream_t);                                                    \
+  template int triattn_output<T>(const void*, const void*, const void*, void*, int, int, int, int, \
                                  hipStream_t);                                                     \
   template int pair_bias_fwd<T>(const void*, const void*, const void*, const void*, void*, int,    \
                                 int, int, float, hipStream_t);

@@ -7,8 +7,10 @@
 
 namespace ptx {
 
-constexpr int kC = 128;       // channels per pair-tensor row == K of every product here
+constexpr int kC = 128;       // hidden channels (c_hidden_mul, heads * d) and the default row width
 constexpr int kKSteps = 8;    // kC / 16
+// Rows of the pair tensor itself may be narrower: KS = c_z / 16 K steps (template
+// parameter of the helpers below, 8 by default; 4 serves c_z = 64).
 
 template <typename T> struct Cfg {
   static constexpr int VE = 16 / (int)sizeof(T);     // elements per 16-byte vector
@@ -22,9 +24,9 @@ template <typename T> struct Cfg {
   static constexpr int NBUF = sizeof(T) == 2 ? 2 : 1;    // weight buffers in LDS
 };
 
-template <typename T, int RB>
+template <typename T, int RB, int KS = kKSteps>
 struct RowFrags {
-  typename Vec8<T>::type f[RB][kKSteps];
+  typename Vec8<T>::type f[RB][KS];
 };
 
 // gamma = 1 / beta = 0 stand-ins for a LayerNorm without weight / bias: the affine loads
@@ -49,34 +51,34 @@ template <typename T> __device__ __forceinline__ const T* default_beta() {
   return reinterpret_cast<const T*>(kZerosAny);
 }
 
-// Mean / rstd of a 128-channel row spread over the two half-wave lanes that hold it,
+// Mean / rstd of a row of 16*KS channels spread over the two half-wave lanes that hold it,
 // then gamma/beta (either may be null); result rounded to T like the reference's
 // LayerNorm output.
-template <typename T>
-__device__ __forceinline__ void normalize_row(f32x8 (&v)[kKSteps], const T* __restrict__ gamma,
+template <typename T, int KS>
+__device__ __forceinline__ void normalize_row(f32x8 (&v)[KS], const T* __restrict__ gamma,
                                               const T* __restrict__ beta, float eps, int g,
-                                              typename Vec8<T>::type (&out)[kKSteps]) {
+                                              typename Vec8<T>::type (&out)[KS]) {
   const T* gp = (gamma ? gamma : default_gamma<T>()) + 8 * g;
   const T* bp = (beta ? beta : default_beta<T>()) + 8 * g;
   float s = 0.0f;
 #pragma unroll
-  for (int kk = 0; kk < kKSteps; ++kk)
+  for (int kk = 0; kk < KS; ++kk)
 #pragma unroll
     for (int t = 0; t < 8; ++t) s += v[kk][t];
   s += swap32(s);
-  const float mean = s * (1.0f / kC);
+  const float mean = s * (1.0f / (16 * KS));
   float q = 0.0f;
 #pragma unroll
-  for (int kk = 0; kk < kKSteps; ++kk)
+  for (int kk = 0; kk < KS; ++kk)
 #pragma unroll
     for (int t = 0; t < 8; ++t) {
       const float d = v[kk][t] - mean;
       q += d * d;
     }
   q += swap32(q);
-  const float rstd = rsqrtf(q * (1.0f / kC) + eps);
+  const float rstd = rsqrtf(q * (1.0f / (16 * KS)) + eps);
 #pragma unroll
-  for (int kk = 0; kk < kKSteps; ++kk) {
+  for (int kk = 0; kk < KS; ++kk) {
     // (no branch around these loads, so the compiler may issue them as early as registers allow)
     const f32x8 gmf = to_f32(load8<T>(gp + 16 * kk)), btf = to_f32(load8<T>(bp + 16 * kk));
     f32x8 o;
@@ -88,25 +90,25 @@ __device__ __forceinline__ void normalize_row(f32x8 (&v)[kKSteps], const T* __re
 
 // The same LayerNorm straight from the stored fragments, converting on the fly in each of
 // its three passes: no fp32 copy of the row is kept, for callers short of registers.
-template <typename T>
-__device__ __forceinline__ void normalize_raw(const typename Vec8<T>::type (&raw)[kKSteps],
+template <typename T, int KS>
+__device__ __forceinline__ void normalize_raw(const typename Vec8<T>::type (&raw)[KS],
                                               const T* __restrict__ gamma,
                                               const T* __restrict__ beta, float eps, int g,
-                                              typename Vec8<T>::type (&out)[kKSteps]) {
+                                              typename Vec8<T>::type (&out)[KS]) {
   const T* gp = (gamma ? gamma : default_gamma<T>()) + 8 * g;
   const T* bp = (beta ? beta : default_beta<T>()) + 8 * g;
   float s = 0.0f;
 #pragma unroll
-  for (int kk = 0; kk < kKSteps; ++kk) {
+  for (int kk = 0; kk < KS; ++kk) {
     const f32x8 v = to_f32(raw[kk]);
 #pragma unroll
     for (int t = 0; t < 8; ++t) s += v[t];
   }
   s += swap32(s);
-  const float mean = s * (1.0f / kC);
+  const float mean = s * (1.0f / (16 * KS));
   float q = 0.0f;
 #pragma unroll
-  for (int kk = 0; kk < kKSteps; ++kk) {
+  for (int kk = 0; kk < KS; ++kk) {
     const f32x8 v = to_f32(raw[kk]);
 #pragma unroll
     for (int t = 0; t < 8; ++t) {
@@ -115,9 +117,9 @@ __device__ __forceinline__ void normalize_raw(const typename Vec8<T>::type (&raw
     }
   }
   q += swap32(q);
-  const float rstd = rsqrtf(q * (1.0f / kC) + eps);
+  const float rstd = rsqrtf(q * (1.0f / (16 * KS)) + eps);
 #pragma unroll
-  for (int kk = 0; kk < kKSteps; ++kk) {
+  for (int kk = 0; kk < KS; ++kk) {
     const f32x8 v = to_f32(raw[kk]);
     const f32x8 gmf = to_f32(load8<T>(gp + 16 * kk)), btf = to_f32(load8<T>(bp + 16 * kk));
     f32x8 o;
@@ -129,8 +131,8 @@ __device__ __forceinline__ void normalize_raw(const typename Vec8<T>::type (&raw
 
 // Load RB row blocks whose lane rows start at element offsets off[rb] (+ 8*g added here)
 // and, if LN, normalise them.
-template <typename T, int RB, bool LN>
-__device__ __forceinline__ void load_rows_at(RowFrags<T, RB>& out, const T* __restrict__ x,
+template <typename T, int RB, bool LN, int KS>
+__device__ __forceinline__ void load_rows_at(RowFrags<T, RB, KS>& out, const T* __restrict__ x,
                                              const int64_t (&off)[RB], const T* __restrict__ gamma,
                                              const T* __restrict__ beta, float eps, int lane) {
   const int g = lane >> 5;
@@ -139,11 +141,11 @@ __device__ __forceinline__ void load_rows_at(RowFrags<T, RB>& out, const T* __re
     const T* rp = x + off[rb] + 8 * g;
     if (!LN) {
 #pragma unroll
-      for (int kk = 0; kk < kKSteps; ++kk) out.f[rb][kk] = load8<T>(rp + 16 * kk);
+      for (int kk = 0; kk < KS; ++kk) out.f[rb][kk] = load8<T>(rp + 16 * kk);
     } else {
-      f32x8 v[kKSteps];
+      f32x8 v[KS];
 #pragma unroll
-      for (int kk = 0; kk < kKSteps; ++kk) v[kk] = to_f32(load8<T>(rp + 16 * kk));
+      for (int kk = 0; kk < KS; ++kk) v[kk] = to_f32(load8<T>(rp + 16 * kk));
       normalize_row<T>(v, gamma, beta, eps, g, out.f[rb]);
     }
   }
@@ -151,8 +153,8 @@ __device__ __forceinline__ void load_rows_at(RowFrags<T, RB>& out, const T* __re
 
 // Load RB*32 consecutive logical rows starting at row0 (rows >= n_rows re-read the last
 // valid row; their results are never stored).
-template <typename T, int RB, bool LN>
-__device__ __forceinline__ void load_rows(RowFrags<T, RB>& out, const T* __restrict__ x,
+template <typename T, int RB, bool LN, int KS>
+__device__ __forceinline__ void load_rows(RowFrags<T, RB, KS>& out, const T* __restrict__ x,
                                           const RowMap& map, int64_t row0, int64_t n_rows,
                                           const T* __restrict__ gamma, const T* __restrict__ beta,
                                           float eps, int lane) {
@@ -163,7 +165,7 @@ __device__ __forceinline__ void load_rows(RowFrags<T, RB>& out, const T* __restr
     p = p < n_rows ? p : n_rows - 1;
     off[rb] = map(p);
   }
-  load_rows_at<T, RB, LN>(out, x, off, gamma, beta, eps, lane);
+  load_rows_at<T, RB, LN, KS>(out, x, off, gamma, beta, eps, lane);
 }
 
 // One weight fragment: 32 output columns x 16 K values, lane -> (column l%32,

@@ -1,6 +1,7 @@
-// Transition (SwiGLU feed-forward) on rows of 128 channels, one kernel:
-//   out = [x +] W_o ( silu(W_a LN(x)) * (W_b LN(x)) ),   W_a, W_b [128*n_factor][128]
-// The hidden activations (n_factor * 128 per row) never leave the chip: a wave
+// Transition (SwiGLU feed-forward) on rows of c = 128 (or 64) channels, one kernel:
+//   out = [x +] W_o ( silu(W_a LN(x)) * (W_b LN(x)) ),   W_a, W_b [c*n_factor][c]
+// (the comments below give the sizes for c = 128).
+// The hidden activations (n_factor * c per row) never leave the chip: a wave
 // keeps its rows as MFMA operand fragments, walks the hidden dimension in chunks
 // of 32 and accumulates the output projection as it goes.
 //
@@ -26,40 +27,43 @@
 
 namespace ptx {
 
-constexpr int kTrFrags = 24;   // fragments per chunk of 32 hidden: W_a 8 K steps, W_b 8, W_o 4 x 2
-
-template <typename T> struct TrCfg {
+// KS = K steps of a row (c / 16: 8 for c = 128, 4 for c = 64); NOB = c / 32 output blocks.
+template <typename T, int KS> struct TrCfg {
   static constexpr int RB = sizeof(T) == 2 ? 2 : 1;     // row blocks of 32 per wave
   static constexpr int NBUF = sizeof(T) == 2 ? 4 : 3;   // chunk buffers in LDS
   static constexpr int D = NBUF - 2;                    // chunks the loads run ahead (two are in use)
   static constexpr int PIECES = (int)sizeof(T) / 2;     // 16-byte pieces per lane and fragment
-  static constexpr int FPW = kTrFrags / 4;              // fragments each wave moves per chunk
+  static constexpr int NOB = KS / 2;
+  // fragments per chunk of 32 hidden: W_a KS K steps, W_b KS, W_o NOB x 2
+  static constexpr int FRAGS = 3 * KS;
+  static constexpr int FPW = FRAGS / 4;                 // fragments each wave moves per chunk
   static constexpr int DMA_PER_CHUNK = FPW * PIECES;
 };
 
 // packed[chunk j][fragment f][lane][8]:
-//   f <  8: W_a, K step f:      lane (m, g) = W_a[32j + m][16f + 8g .. +7]
-//   f < 16: W_b, K step f - 8
-//   else:   W_o, output block ob = (f-16)/2, K step u = (f-16)%2:
+//   f <  KS:  W_a, K step f:      lane (m, g) = W_a[32j + m][16f + 8g .. +7]
+//   f < 2KS:  W_b, K step f - KS
+//   else:     W_o, output block ob = (f-2KS)/2, K step u = (f-2KS)%2:
 //           lane (m, g), slot t = W_o[32 ob + m][32j + 8(2u + t/4) + 4g + t%4]
 //           (slot t of K step u <-> accumulator register 8u + t of GEMM1)
-template <typename T>
+template <typename T, int KS>
 __global__ void transition_pack_kernel(const T* __restrict__ w_a, const T* __restrict__ w_b,
                                        const T* __restrict__ w_o, T* __restrict__ packed,
                                        int n_hidden) {
+  constexpr int kFrags = 3 * KS;
   const int idx = blockIdx.x * blockDim.x + threadIdx.x;
   const int n_chunks = n_hidden / 32;
-  if (idx >= n_chunks * kTrFrags * kWave) return;
-  const int lane = idx & 63, f = (idx >> 6) % kTrFrags, j = idx / (kWave * kTrFrags);
+  if (idx >= n_chunks * kFrags * kWave) return;
+  const int lane = idx & 63, f = (idx >> 6) % kFrags, j = idx / (kWave * kFrags);
   const int m = lane & 31, g = lane >> 5;
   typename Vec8<T>::type v;
-  if (f < 16) {
-    const T* w = f < 8 ? w_a : w_b;
-    const int kk = f & 7;
+  if (f < 2 * KS) {
+    const T* w = f < KS ? w_a : w_b;
+    const int kk = f % KS;
 #pragma unroll
-    for (int t = 0; t < 8; ++t) v[t] = w[(int64_t)(32 * j + m) * kC + 16 * kk + 8 * g + t];
+    for (int t = 0; t < 8; ++t) v[t] = w[(int64_t)(32 * j + m) * (16 * KS) + 16 * kk + 8 * g + t];
   } else {
-    const int ob = (f - 16) >> 1, u = (f - 16) & 1;
+    const int ob = (f - 2 * KS) >> 1, u = (f - 2 * KS) & 1;
 #pragma unroll
     for (int t = 0; t < 8; ++t) {
       const int hidden = 32 * j + 8 * (2 * u + (t >> 2)) + 4 * g + (t & 3);
@@ -69,16 +73,17 @@ __global__ void transition_pack_kernel(const T* __restrict__ w_a, const T* __res
   store8<T>(packed + (int64_t)idx * 8, v);
 }
 
-template <typename T>
+template <typename T, int KS>
 __global__ __launch_bounds__(256) void transition_fused_kernel(
     const T* x, const T* __restrict__ gamma, const T* __restrict__ beta,
     const T* __restrict__ packed, T* out, int64_t n_rows, int n_chunks, int add_residual,
     float eps) {
   typedef typename Vec8<T>::type V8;
   typedef typename VecE<T>::type VE_t;
-  typedef TrCfg<T> G;
+  typedef TrCfg<T, KS> G;
   typedef Cfg<T> C;
   constexpr int RB = G::RB, NBUF = G::NBUF, D = G::D, PIECES = G::PIECES, FPW = G::FPW;
+  constexpr int NOB = G::NOB, kTrFrags = G::FRAGS, kCx = 16 * KS;
   __shared__ u32x4_t lds_w[NBUF][kTrFrags][PIECES][kWave];
   static_assert(sizeof(T) * 4 * 32 * C::PITCH <= sizeof(u32x4_t) * kTrFrags * PIECES * kWave,
                 "the staging tiles reuse chunk buffer 0");
@@ -110,27 +115,27 @@ __global__ __launch_bounds__(256) void transition_fused_kernel(
   // start the weight ring, then fetch and normalise this wave's rows
 #pragma unroll
   for (int j = 0; j < D; ++j) dma_chunk(j);
-  RowFrags<T, RB> xf;
-  load_rows<T, RB, true>(xf, x, RowMap{kC, 0, 1}, row0, n_rows, gamma, beta, eps, lane);
+  RowFrags<T, RB, KS> xf;
+  load_rows<T, RB, true>(xf, x, RowMap{kCx, 0, 1}, row0, n_rows, gamma, beta, eps, lane);
 
-  f32x16 acc_o[RB][4];   // [row block][output column block]: lane <-> row, register <-> column
+  f32x16 acc_o[RB][NOB];   // [row block][output column block]: lane <-> row, register <-> column
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
-    for (int ob = 0; ob < 4; ++ob)
+    for (int ob = 0; ob < NOB; ++ob)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc_o[rb][ob][r] = 0.0f;
   f32x16 ab0[RB][2], ab1[RB][2];   // GEMM1 accumulators (a, b) of even / odd chunks
   V8 hf[RB][2];                    // activated hidden values as GEMM2 operand fragments
 
-  // One eighth of a chunk's activation: accumulator registers 2*part, 2*part + 1.
+  // One KS-th of a chunk's activation: accumulator registers (16/KS)*part .. +16/KS-1.
   // a and b stay in fp32 through the activation; the product is rounded to T once.
   auto act_part = [&](int part, f32x16 (&ab)[RB][2]) {
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
-      for (int e = 0; e < 2; ++e) {
-        const int r = 2 * part + e;
+      for (int e = 0; e < 16 / KS; ++e) {
+        const int r = (16 / KS) * part + e;
         const float a = ab[rb][0][r], b = ab[rb][1][r];
         hf[rb][r >> 3][r & 7] = from_f32<T>(a * b * sigmoidf_fast(a));
       }
@@ -142,15 +147,15 @@ __global__ __launch_bounds__(256) void transition_fused_kernel(
   auto gemm1 = [&](auto act_tag, int buf, f32x16 (&cur)[RB][2], f32x16 (&prev)[RB][2],
                    int tail_buf) {
     constexpr bool ACT = decltype(act_tag)::value;
-    V8 wa = read_frag(buf, 0), wb = read_frag(buf, 8);
+    V8 wa = read_frag(buf, 0), wb = read_frag(buf, KS);
 #pragma unroll
-    for (int kk = 0; kk < kKSteps; ++kk) {
+    for (int kk = 0; kk < KS; ++kk) {
       V8 na, nb = wb;
-      if (kk + 1 < kKSteps) {
+      if (kk + 1 < KS) {
         na = read_frag(buf, kk + 1);
-        nb = read_frag(buf, 8 + kk + 1);
+        nb = read_frag(buf, KS + kk + 1);
       } else {
-        na = read_frag(tail_buf, 16);
+        na = read_frag(tail_buf, 2 * KS);
       }
 #pragma unroll
       for (int rb = 0; rb < RB; ++rb) {
@@ -171,10 +176,10 @@ __global__ __launch_bounds__(256) void transition_fused_kernel(
   // GEMM2 of the chunk whose W_o fragments sit in buffer `buf`; `wo` is its first fragment.
   auto gemm2 = [&](int buf, V8 wo) {
 #pragma unroll
-    for (int s2 = 0; s2 < 8; ++s2) {
-      const int u = s2 >> 2, ob = s2 & 3;
+    for (int s2 = 0; s2 < 2 * NOB; ++s2) {
+      const int u = s2 / NOB, ob = s2 % NOB;
       V8 nw = wo;
-      if (s2 + 1 < 8) nw = read_frag(buf, 16 + ((s2 + 1) & 3) * 2 + ((s2 + 1) >> 2));
+      if (s2 + 1 < 2 * NOB) nw = read_frag(buf, 2 * KS + ((s2 + 1) % NOB) * 2 + ((s2 + 1) / NOB));
 #pragma unroll
       for (int rb = 0; rb < RB; ++rb) mma32(acc_o[rb][ob], wo, hf[rb][u]);
       wo = nw;
@@ -208,7 +213,7 @@ __global__ __launch_bounds__(256) void transition_fused_kernel(
   // full memory round trip per tile: out may alias x, so no load could move above the
   // previous store).  Each lane reads exactly the vectors it later overwrites.
   int64_t obase[RB][C::NPASS];
-  VE_t resv[RB][4][C::NPASS];
+  VE_t resv[RB][NOB][C::NPASS];
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
@@ -216,13 +221,13 @@ __global__ __launch_bounds__(256) void transition_fused_kernel(
       int mj, m0;
       stage_coord<T>(ps, lane, mj, m0);
       const int64_t pr = row0 + rb * 32 + mj;
-      obase[rb][ps] = pr < n_rows ? pr * kC + m0 : -1;
+      obase[rb][ps] = pr < n_rows ? pr * kCx + m0 : -1;
     }
   if (add_residual) {
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
-      for (int ob = 0; ob < 4; ++ob)
+      for (int ob = 0; ob < NOB; ++ob)
 #pragma unroll
         for (int ps = 0; ps < C::NPASS; ++ps)
           if (obase[rb][ps] >= 0)
@@ -230,8 +235,8 @@ __global__ __launch_bounds__(256) void transition_fused_kernel(
   }
   // drain: activation and GEMM2 of the last chunk
 #pragma unroll
-  for (int kk = 0; kk < kKSteps; ++kk) act_part(kk, ab1);
-  gemm2((n_chunks - 1) % NBUF, read_frag((n_chunks - 1) % NBUF, 16));
+  for (int kk = 0; kk < KS; ++kk) act_part(kk, ab1);
+  gemm2((n_chunks - 1) % NBUF, read_frag((n_chunks - 1) % NBUF, 2 * KS));
 
   // ---- epilogue: out rows through the per-wave staging tile (reuses chunk buffer 0 once
   // every wave is past its last fragment read and all loads have landed) ----
@@ -240,7 +245,7 @@ __global__ __launch_bounds__(256) void transition_fused_kernel(
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
 #pragma unroll
-    for (int ob = 0; ob < 4; ++ob) {
+    for (int ob = 0; ob < NOB; ++ob) {
       float vals[16];
 #pragma unroll
       for (int r = 0; r < 16; ++r) vals[r] = acc_o[rb][ob][r];
@@ -261,36 +266,54 @@ __global__ __launch_bounds__(256) void transition_fused_kernel(
   }
 }
 
-template <typename T>
-int transition_pack(const void* w_a, const void* w_b, const void* w_o, void* packed, int n_factor,
-                    hipStream_t stream) {
-  const int n_hidden = kC * n_factor;
-  const int total = (n_hidden / 32) * kTrFrags * kWave;
+template <typename T, int KS>
+static int transition_pack_ks(const void* w_a, const void* w_b, const void* w_o, void* packed,
+                              int n_factor, hipStream_t stream) {
+  const int n_hidden = 16 * KS * n_factor;
+  const int total = (n_hidden / 32) * TrCfg<T, KS>::FRAGS * kWave;
   if (total == 0) return 0;
-  transition_pack_kernel<T><<<dim3((total + 255) / 256), dim3(256), 0, stream>>>(
+  transition_pack_kernel<T, KS><<<dim3((total + 255) / 256), dim3(256), 0, stream>>>(
       (const T*)w_a, (const T*)w_b, (const T*)w_o, (T*)packed, n_hidden);
   return 0;
 }
 
 template <typename T>
-int transition_fwd(const void* x, const void* ln_w, const void* ln_b, const void* packed,
-                   void* out, int64_t rows, int n_factor, int add_residual, float eps,
-                   hipStream_t stream) {
-  if (rows == 0) return 0;
-  const int64_t rows_per_block = 4 * TrCfg<T>::RB * 32;
+int transition_pack(const void* w_a, const void* w_b, const void* w_o, void* packed, int c,
+                    int n_factor, hipStream_t stream) {
+  return c == 64 ? transition_pack_ks<T, 4>(w_a, w_b, w_o, packed, n_factor, stream)
+                 : transition_pack_ks<T, 8>(w_a, w_b, w_o, packed, n_factor, stream);
+}
+
+template <typename T, int KS>
+static int transition_fwd_ks(const void* x, const void* ln_w, const void* ln_b, const void* packed,
+                             void* out, int64_t rows, int n_factor, int add_residual, float eps,
+                             hipStream_t stream) {
+  const int64_t rows_per_block = 4 * TrCfg<T, KS>::RB * 32;
   const int64_t blocks = (rows + rows_per_block - 1) / rows_per_block;
-  transition_fused_kernel<T><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(
-      (const T*)x, (const T*)ln_w, (const T*)ln_b, (const T*)packed, (T*)out, rows, 4 * n_factor,
-      add_residual, eps);
+  transition_fused_kernel<T, KS><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(
+      (const T*)x, (const T*)ln_w, (const T*)ln_b, (const T*)packed, (T*)out, rows,
+      16 * KS * n_factor / 32, add_residual, eps);
   return 0;
 }
 
-template int transition_pack<float>(const void*, const void*, const void*, void*, int, hipStream_t);
-template int transition_pack<bf16_t>(const void*, const void*, const void*, void*, int,
+template <typename T>
+int transition_fwd(const void* x, const void* ln_w, const void* ln_b, const void* packed,
+                   void* out, int64_t rows, int c, int n_factor, int add_residual, float eps,
+                   hipStream_t stream) {
+  if (rows == 0) return 0;
+  return c == 64 ? transition_fwd_ks<T, 4>(x, ln_w, ln_b, packed, out, rows, n_factor,
+                                           add_residual, eps, stream)
+                 : transition_fwd_ks<T, 8>(x, ln_w, ln_b, packed, out, rows, n_factor,
+                                           add_residual, eps, stream);
+}
+
+template int transition_pack<float>(const void*, const void*, const void*, void*, int, int,
+                                    hipStream_t);
+template int transition_pack<bf16_t>(const void*, const void*, const void*, void*, int, int,
                                      hipStream_t);
 template int transition_fwd<float>(const void*, const void*, const void*, const void*, void*,
-                                   int64_t, int, int, float, hipStream_t);
+                                   int64_t, int, int, int, float, hipStream_t);
 template int transition_fwd<bf16_t>(const void*, const void*, const void*, const void*, void*,
-                                    int64_t, int, int, float, hipStream_t);
+                                    int64_t, int, int, int, float, hipStream_t);
 
 }  // namespace ptx

@@ -185,7 +185,7 @@ def triangle_attention(z: torch.Tensor, mask: Optional[torch.Tensor], w: dict, h
 
 
 def transition_pack(w_a: torch.Tensor, w_b: torch.Tensor, w_o: torch.Tensor) -> torch.Tensor:
-    """Packs the three Transition weights (c = 128) into the fused kernel's streaming order."""
+    """Packs the three Transition weights (c = 64 or 128) into the fused kernel's streaming order."""
     _dev(w_a, "w_a")
     lib = _lib.load()
     c = w_a.shape[1]
@@ -201,7 +201,7 @@ def transition_pack(w_a: torch.Tensor, w_b: torch.Tensor, w_o: torch.Tensor) -> 
 
 def transition(x: torch.Tensor, w: dict, n_factor: int, add_residual: bool,
                out: Optional[torch.Tensor] = None, eps: float = 1e-5) -> torch.Tensor:
-    """x [..., 128] -> [x +] W_o(silu(W_a LN x) * W_b LN x); `w["packed"]` comes from
+    """x [..., c] -> [x +] W_o(silu(W_a LN x) * W_b LN x), c = 64 or 128; `w["packed"]` comes from
     transition_pack."""
     _dev(x, "x")
     lib = _lib.load()

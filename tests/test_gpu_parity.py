@@ -195,3 +195,62 @@ def test_stack_4_blocks(dtype):
         s_ref, z_ref = ref(s.float(), z.float(), pm.float())
         s_got, z_got = prod(s.cuda(), z.cuda(), pm.cuda())
     assert rel_err(z_got, z_ref) <= tol(dtype) and rel_err(s_got, s_ref) <= tol(dtype)
+
+
+# ------------------------------------------------------------------ c_z = 64 (the template embedder's pair stack)
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("cls", ["TriangleMultiplicationOutgoing", "TriangleMultiplicationIncoming"])
+@pytest.mark.parametrize("n,n_pad", [(64, 0), (100, 7), (37, 0)])
+def test_trimul_cz64(dtype, cls, n, n_pad):
+    """c_z = 64 with the default c_hidden_mul = 128 (pairformer.py:969-977 of the reference)."""
+    ref, prod = oracle_and_product(getattr(O, cls), getattr(P, cls), 64, 128, dtype=dtype)
+    z = _z(n, dtype, c=64)
+    mask = pad_mask(n, n_pad, dtype) if n_pad else None
+    with torch.no_grad():
+        want = ref(z.float(), None if mask is None else mask.float())
+        got = prod(z.cuda(), None if mask is None else mask.cuda())
+        assert got.shape == want.shape and rel_err(got, want) <= tol(dtype)
+        zc = z.cuda().clone()
+        got2 = prod(zc, None if mask is None else mask.cuda(), inplace_safe=True, _add_with_inplace=True)
+        assert got2.data_ptr() == zc.data_ptr()
+        assert rel_err(got2, z.float() + want) <= tol(dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("starting", [True, False])
+@pytest.mark.parametrize("n,n_pad", [(64, 0), (100, 7), (37, 5)])
+def test_triattn_cz64(dtype, starting, n, n_pad):
+    ref, prod = oracle_and_product(O.TriangleAttention, P.TriangleAttention, 64, 32, 4,
+                                   starting=starting, dtype=dtype)
+    z = _z(n, dtype, c=64)
+    mask = pad_mask(n, n_pad, dtype) if n_pad else None
+    with torch.no_grad():
+        want = ref(z.float(), None if mask is None else mask.float(), chunk_size=64)
+        got = prod(z.cuda(), None if mask is None else mask.cuda())
+    assert got.shape == want.shape and rel_err(got, want) <= tol(dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shape,factor", [((1, 50, 50, 64), 2), ((3001, 64), 4), ((77, 64), 1)])
+def test_transition_cz64(dtype, shape, factor):
+    ref, prod = oracle_and_product(O.Transition, P.Transition, 64, factor, dtype=dtype)
+    x = torch.randn(*shape, generator=torch.Generator().manual_seed(11)).to(dtype)
+    with torch.no_grad():
+        assert rel_err(prod(x.cuda()), ref(x.float())) <= tol(dtype)
+        xc = x.cuda().clone()
+        got = prod(xc, _residual_out=xc)
+        assert got.data_ptr() == xc.data_ptr()
+        assert rel_err(got, x.float() + ref(x.float())) <= tol(dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_template_pair_stack_cz64(dtype):
+    """The stack as the template embedder builds it: c_z = 64, no single track, two blocks,
+    transition factor 2 (pairformer.py:969-977 of the reference)."""
+    kw = dict(n_blocks=2, c_z=64, c_s=0, num_intermediate_factor=2)
+    ref, prod = oracle_and_product(O.PairformerStack, P.PairformerStack, dtype=dtype, **kw)
+    _, z, pm = O.make_inputs(90, c_z=64, n_pad=6, dtype=dtype)
+    with torch.no_grad():
+        _, z_ref = ref(None, z.float(), pm.float())
+        s_got, z_got = prod(None, z.cuda(), pm.cuda())
+    assert s_got is None and rel_err(z_got, z_ref) <= tol(dtype)
