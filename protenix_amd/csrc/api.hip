@@ -84,15 +84,23 @@ PTX_API int ptx_layernorm_fwd(const void* x, const void* gamma, const void* beta
   return after_launch("layernorm");
 }
 
+// Pair-row widths the kernels are built for: c_z = 64 or 128 with hidden widths (c_hidden,
+// heads * 32) of 128, or c_z = 256 in bf16 with hidden widths of 256.
+static bool pair_width_ok(int c_z, int hidden, int dtype) {
+  if (c_z == 64 || c_z == 128) return hidden == 128;
+  return c_z == 256 && hidden == 256 && dtype == PTX_BF16;
+}
+static const char* const kWidthMsg =
+    "only c_z = 64 / 128 with hidden width 128, or c_z = 256 with hidden width 256 in bf16, is built";
+
 PTX_API int ptx_trimul_project(const void* z, const void* mask, const void* ln_w, const void* ln_b,
                        const void* w_ap, const void* w_ag, const void* w_bp, const void* w_bg,
                        void* a, void* b, int n, int c_z, int c_hidden, int k_pitch, int incoming,
                        float eps, int dtype, void* stream) {
   PTX_REQUIRE(dtype_ok(dtype), PTX_ERR_BAD_ARG, "trimul_project: unknown dtype %d", dtype);
   PTX_REQUIRE(n >= 0, PTX_ERR_BAD_ARG, "trimul_project: n=%d", n);
-  PTX_REQUIRE((c_z == 128 || c_z == 64) && c_hidden == 128, PTX_ERR_UNSUPPORTED,
-              "trimul_project: only c_z = 64 or 128 with c_hidden = 128 is built (got %d, %d)", c_z,
-              c_hidden);
+  PTX_REQUIRE(pair_width_ok(c_z, c_hidden, dtype), PTX_ERR_UNSUPPORTED,
+              "trimul_project: %s (got c_z=%d c_hidden=%d)", kWidthMsg, c_z, c_hidden);
   PTX_REQUIRE(k_pitch == ptx_key_pitch(n), PTX_ERR_BAD_ARG,
               "trimul_project: k_pitch=%d, expected ptx_key_pitch(%d)=%d", k_pitch, n,
               ptx_key_pitch(n));
@@ -131,9 +139,8 @@ PTX_API int ptx_trimul_output(const void* x, const void* z, const void* ln_in_w,
                       float eps, int dtype, void* stream) {
   PTX_REQUIRE(dtype_ok(dtype), PTX_ERR_BAD_ARG, "trimul_output: unknown dtype %d", dtype);
   PTX_REQUIRE(n >= 0, PTX_ERR_BAD_ARG, "trimul_output: n=%d", n);
-  PTX_REQUIRE((c_z == 128 || c_z == 64) && c_hidden == 128, PTX_ERR_UNSUPPORTED,
-              "trimul_output: only c_z = 64 or 128 with c_hidden = 128 is built (got %d, %d)", c_z,
-              c_hidden);
+  PTX_REQUIRE(pair_width_ok(c_z, c_hidden, dtype), PTX_ERR_UNSUPPORTED,
+              "trimul_output: %s (got c_z=%d c_hidden=%d)", kWidthMsg, c_z, c_hidden);
   PTX_REQUIRE(n < 32768, PTX_ERR_UNSUPPORTED, "trimul_output: n=%d too large", n);
   if (n == 0) return PTX_OK;
   PTX_REQUIRE(x && z && ln_out_w && ln_out_b && w_z && w_g && out, PTX_ERR_BAD_ARG,
@@ -155,10 +162,9 @@ PTX_API int ptx_triattn_project(const void* z, const void* ln_w, const void* ln_
                         void* stream) {
   PTX_REQUIRE(dtype_ok(dtype), PTX_ERR_BAD_ARG, "triattn_project: unknown dtype %d", dtype);
   PTX_REQUIRE(n >= 0, PTX_ERR_BAD_ARG, "triattn_project: n=%d", n);
-  PTX_REQUIRE((c_in == 128 || c_in == 64) && d == 32 && heads == 4, PTX_ERR_UNSUPPORTED,
-              "triattn_project: only c_in = 64 or 128, 4 heads x 32 is built (got c_in=%d heads=%d "
-              "d=%d)",
-              c_in, heads, d);
+  PTX_REQUIRE(d == 32 && heads > 0 && heads <= 8 && pair_width_ok(c_in, heads * 32, dtype),
+              PTX_ERR_UNSUPPORTED, "triattn_project: %s, head dim 32 (got c_in=%d heads=%d d=%d)",
+              kWidthMsg, c_in, heads, d);
   PTX_REQUIRE(key_pitch == ptx_key_pitch(n), PTX_ERR_BAD_ARG,
               "triattn_project: key_pitch=%d, expected %d", key_pitch, ptx_key_pitch(n));
   PTX_REQUIRE(n < 32768, PTX_ERR_UNSUPPORTED, "triattn_project: n=%d too large", n);
@@ -201,8 +207,8 @@ PTX_API int ptx_triattn_output(const void* o, const void* w_o, const void* z, vo
                        int transposed, int add_residual, int dtype, void* stream) {
   PTX_REQUIRE(dtype_ok(dtype), PTX_ERR_BAD_ARG, "triattn_output: unknown dtype %d", dtype);
   PTX_REQUIRE(n >= 0, PTX_ERR_BAD_ARG, "triattn_output: n=%d", n);
-  PTX_REQUIRE(c_in == 128 || c_in == 64, PTX_ERR_UNSUPPORTED,
-              "triattn_output: only c_in = 64 or 128 is built (got %d)", c_in);
+  PTX_REQUIRE(pair_width_ok(c_in, c_in == 256 ? 256 : 128, dtype), PTX_ERR_UNSUPPORTED,
+              "triattn_output: %s (got c_in=%d)", kWidthMsg, c_in);
   PTX_REQUIRE(n < 32768, PTX_ERR_UNSUPPORTED, "triattn_output: n=%d too large", n);
   if (n == 0) return PTX_OK;
   PTX_REQUIRE(o && w_o && out && (!add_residual || z), PTX_ERR_BAD_ARG,
@@ -224,8 +230,8 @@ PTX_API int ptx_transition_pack(const void* w_a, const void* w_b, const void* w_
                         int n_factor, int dtype, void* stream) {
   PTX_REQUIRE(dtype_ok(dtype), PTX_ERR_BAD_ARG, "transition_pack: unknown dtype %d", dtype);
   PTX_REQUIRE(n_factor > 0, PTX_ERR_BAD_ARG, "transition_pack: n_factor=%d", n_factor);
-  PTX_REQUIRE(c == 128 || c == 64, PTX_ERR_UNSUPPORTED,
-              "transition_pack: only c = 64 or 128 is built (got %d)", c);
+  PTX_REQUIRE(c == 128 || c == 64 || (c == 256 && dtype == PTX_BF16), PTX_ERR_UNSUPPORTED,
+              "transition_pack: only c = 64, 128, or 256 in bf16, is built (got %d)", c);
   PTX_REQUIRE((n_factor * c) % 64 == 0, PTX_ERR_UNSUPPORTED,
               "transition_pack: the hidden width %d is not a multiple of 64", n_factor * c);
   PTX_REQUIRE(n_factor <= 64, PTX_ERR_UNSUPPORTED, "transition_pack: n_factor=%d too large",
@@ -243,8 +249,8 @@ PTX_API int ptx_transition_fwd(const void* x, const void* ln_w, const void* ln_b
   PTX_REQUIRE(dtype_ok(dtype), PTX_ERR_BAD_ARG, "transition: unknown dtype %d", dtype);
   PTX_REQUIRE(rows >= 0 && n_factor > 0, PTX_ERR_BAD_ARG, "transition: rows=%lld n_factor=%d",
               (long long)rows, n_factor);
-  PTX_REQUIRE(c == 128 || c == 64, PTX_ERR_UNSUPPORTED,
-              "transition: only c = 64 or 128 is built (got %d)", c);
+  PTX_REQUIRE(c == 128 || c == 64 || (c == 256 && dtype == PTX_BF16), PTX_ERR_UNSUPPORTED,
+              "transition: only c = 64, 128, or 256 in bf16, is built (got %d)", c);
   PTX_REQUIRE((n_factor * c) % 64 == 0, PTX_ERR_UNSUPPORTED,
               "transition: the hidden width %d is not a multiple of 64", n_factor * c);
   PTX_REQUIRE(n_factor <= 64, PTX_ERR_UNSUPPORTED, "transition: n_factor=%d too large", n_factor);
@@ -265,7 +271,8 @@ PTX_API int ptx_pair_bias_fwd(const void* z, const void* ln_w, const void* ln_b,
                       void* stream) {
   PTX_REQUIRE(dtype_ok(dtype), PTX_ERR_BAD_ARG, "pair_bias: unknown dtype %d", dtype);
   PTX_REQUIRE(n >= 0, PTX_ERR_BAD_ARG, "pair_bias: n=%d", n);
-  PTX_REQUIRE(c_z == 128, PTX_ERR_UNSUPPORTED, "pair_bias: only c_z=128 is built (got %d)", c_z);
+  PTX_REQUIRE(c_z == 128 || (c_z == 256 && dtype == PTX_BF16), PTX_ERR_UNSUPPORTED,
+              "pair_bias: only c_z = 128, or 256 in bf16, is built (got %d)", c_z);
   PTX_REQUIRE(heads >= 1 && heads <= 32, PTX_ERR_UNSUPPORTED,
               "pair_bias: heads=%d outside 1..32", heads);
   PTX_REQUIRE(n < 32768, PTX_ERR_UNSUPPORTED, "pair_bias: n=%d too large", n);
@@ -274,7 +281,7 @@ PTX_API int ptx_pair_bias_fwd(const void* z, const void* ln_w, const void* ln_b,
   PTX_REQUIRE(aligned16(z) && aligned16(w) && aligned16(bias) && (!ln_w || aligned16(ln_w)) &&
                   (!ln_b || aligned16(ln_b)),
               PTX_ERR_BAD_ARG, "pair_bias: pointers must be 16-byte aligned");
-  PTX_DISPATCH(dtype, ptx::pair_bias_fwd<T>(z, ln_w, ln_b, w, bias, n, heads, out_f32, eps,
+  PTX_DISPATCH(dtype, ptx::pair_bias_fwd<T>(z, ln_w, ln_b, w, bias, n, c_z, heads, out_f32, eps,
                                             (hipStream_t)stream));
   return after_launch("pair_bias");
 }

@@ -1,6 +1,6 @@
 // Host-callable launchers, one per kernel family; api.hip validates arguments
-// and dispatches on dtype.  c_z / c: channels of a pair-tensor row, 64 or 128 (the hidden
-// widths - c_hidden_mul, heads * d - are 128).  All return 0 after enqueueing on `stream`.
+// and dispatches on dtype.  c_z / c: channels of a pair-tensor row: 64 or 128 (hidden
+// widths - c_hidden_mul, heads * d - of 128), or 256 in bf16 (hidden widths of 256).  All return 0 after enqueueing on `stream`.
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -38,7 +38,7 @@ int transition_fwd(const void* x, const void* ln_w, const void* ln_b, const void
                    hipStream_t stream);
 template <typename T>
 int pair_bias_fwd(const void* z, const void* ln_w, const void* ln_b, const void* w, void* bias,
-                  int n, int heads, int out_f32, float eps, hipStream_t stream);
+                  int n, int c_z, int heads, int out_f32, float eps, hipStream_t stream);
 
 // x[c][i][j] = sum_k a[c][i][k] * b[c][j][k] for `batch` independent products;
 // a, b rows have pitch k_pitch (a multiple of 64, >= n), x is dense [batch][n][n].

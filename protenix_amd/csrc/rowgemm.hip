@@ -59,33 +59,46 @@ enum RowGemmInMode { kTriMulIn = 0, kTriAttnIn = 1, kPairBias = 3, kTriMulOut = 
 // per chunk a constant, which the weight ring below counts on.
 static __device__ __attribute__((aligned(16))) uint32_t g_store_sink[kWave * 4];
 
+// Widths.  KS = K steps of a pair-tensor row (c_z / 16: 4, 8 or 16).  The hidden widths
+// (c_hidden_mul, heads * 32) are 128 for c_z <= 128 and c_z beyond ("hidden_scale_up" of the
+// reference, pairformer.py:76-78): SL = hidden / 16 K steps, which is also the number of
+// fragment slots a weight tile takes in LDS.
+template <int KS> struct Widths {
+  static constexpr int SL = KS > 8 ? KS : 8;
+  static constexpr int HIDDEN = 16 * SL;
+  static constexpr int HEADS = HIDDEN / 32;
+};
+
 // Weight matrix, its row count, first row, row length and K steps for tile `t` (0/1) of
-// chunk `ch`.  KS = K steps of a pair-tensor row (c_z / 16); the hidden widths are 128.
+// chunk `ch`.
 template <typename T, int MODE, int KS>
 __device__ __forceinline__ void chunk_tile(const RowGemmInParams& p, int ch, int t, const T*& w,
                                            int& n_out, int& col0, int& ldw, int& ksteps) {
+  typedef Widths<KS> W;
   ldw = 16 * KS;
   ksteps = KS;
   if (MODE == kTriMulIn) {            // w: ap, ag, bp, bg ; tile0 = projection, tile1 = gate
-    w = (const T*)p.w[(ch >> 2) * 2 + t];
-    n_out = kC;
-    col0 = (ch & 3) * 32;
+    constexpr int CPM = W::HIDDEN / 32;   // chunks per operand
+    w = (const T*)p.w[(ch / CPM) * 2 + t];
+    n_out = W::HIDDEN;
+    col0 = (ch % CPM) * 32;
   } else if (MODE == kTriAttnIn) {    // w: q, k, g, v, bias
-    const int which = ch >> 1;
+    constexpr int CPM = W::HIDDEN / 64;   // chunks (of two heads) per matrix
+    const int which = ch / CPM;
     w = (const T*)p.w[which];
-    n_out = which == 4 ? p.aux : kC;
-    col0 = which == 4 ? 0 : ((ch & 1) * 2 + t) * 32;
+    n_out = which == 4 ? p.aux : W::HIDDEN;
+    col0 = which == 4 ? 0 : ((ch % CPM) * 2 + t) * 32;
   } else if (MODE == kPairBias) {
     w = (const T*)p.w[0];
     n_out = p.aux & 0xff;
     col0 = 0;
-  } else {                            // kTriMulOut: w: z [c_z][128], g [c_z][c_z]
+  } else {                            // kTriMulOut: w: z [c_z][hidden], g [c_z][c_z]
     w = (const T*)p.w[t];
     n_out = 16 * KS;
     col0 = ch * 32;
     if (t == 0) {
-      ldw = kC;
-      ksteps = kKSteps;
+      ldw = W::HIDDEN;
+      ksteps = W::SL;
     }
   }
 }
@@ -98,26 +111,32 @@ __device__ __forceinline__ void chunk_tile(const RowGemmInParams& p, int ch, int
 // for its share of them also waits for the stores it issued before.)  fp32 weights are twice
 // the size and do not fit: that path stages one chunk at a time through registers.
 template <typename T, int MODE, int KS> struct InCfg {
-  static constexpr bool RES = sizeof(T) == 2 && MODE != kPairBias;
+  static constexpr int SL = Widths<KS>::SL;
+  // (256-channel rows: the weights do not fit either; bf16 then takes the staged path too)
+  static constexpr bool RES = sizeof(T) == 2 && MODE != kPairBias && KS <= 8;
   static constexpr int NW = RES ? 8 : 4;   // waves per workgroup
-  // chunks of two 32-column weight tiles: {a,b} x 4 channel blocks | q,k,g,v: 2 each, bias: 1 |
-  // the pair bias | c_z / 32 output column blocks
-  static constexpr int NCH =
-      MODE == kTriMulIn ? 8 : MODE == kTriAttnIn ? 9 : MODE == kPairBias ? 1 : KS / 2;
-  // weight fragments held in LDS (16 per chunk; the resident triangle bias is one tile of 8)
-  static constexpr int NFRAG =
-      RES ? (MODE == kTriAttnIn ? 8 * 16 + 8 : NCH * 16) : Cfg<T>::NBUF * 16;
+  // chunks of two 32-column weight tiles: {a,b} x hidden/32 channel blocks | q,k,g,v: one per
+  // two heads, bias: 1 | the pair bias | c_z / 32 output column blocks
+  static constexpr int NCH = MODE == kTriMulIn    ? 2 * (SL / 2)
+                             : MODE == kTriAttnIn ? 4 * (SL / 4) + 1
+                             : MODE == kPairBias  ? 1
+                                                  : KS / 2;
+  // weight fragments held in LDS (2*SL per chunk; the resident triangle bias is one tile)
+  static constexpr int NFRAG = RES ? (MODE == kTriAttnIn ? (NCH - 1) * 2 * SL + SL : NCH * 2 * SL)
+                                   : Cfg<T>::NBUF * 2 * SL;
+  static constexpr int FPW = 2 * SL / 4;   // staged path: fragments per wave and chunk
+  static constexpr int MIN_WG = (RES || KS > 8) ? 1 : 2;
 };
 
 template <typename T, int RB, int MODE, int KS>
-__global__ __launch_bounds__((InCfg<T, MODE, KS>::NW * 64), (InCfg<T, MODE, KS>::RES ? 1 : 2)) void
+__global__ __launch_bounds__((InCfg<T, MODE, KS>::NW * 64), (InCfg<T, MODE, KS>::MIN_WG)) void
 rowgemm_in_kernel(RowGemmInParams p) {
   typedef typename Vec8<T>::type V8;
   typedef typename VecE<T>::type VE_t;
   typedef Cfg<T> C;
   typedef InCfg<T, MODE, KS> IC;
   constexpr bool RES = IC::RES;
-  constexpr int NW = IC::NW;
+  constexpr int NW = IC::NW, SL = IC::SL, FPW = IC::FPW;
   __shared__ V8 lds_w[IC::NFRAG][kWave];
   // Staging tiles per wave.  Resident: one (LDS is full of weights).  Otherwise one per
   // 32 x 32 result tile of a chunk: all tiles of a chunk are written, then all are read back
@@ -153,44 +172,46 @@ rowgemm_in_kernel(RowGemmInParams p) {
                      : (int64_t)blockIdx.x * 4 + wave;
   const int64_t tile_step = (int64_t)gridDim.x * NW;
 
-  // Weight fragment f = 16 * chunk + 8 * tile + K step, from global memory straight into its
+  // Weight fragment f = 2*SL * chunk + SL * tile + K step, from global memory straight into its
   // LDS slot (bf16).  These loads are invisible to the compiler's wait-count bookkeeping and
   // are waited for by hand.
   auto dma_frag = [&](int f_src, int f_dst) {
     const T* w;
     int n_out, col0, ldw, ksteps;
-    chunk_tile<T, MODE, KS>(p, f_src >> 4, (f_src >> 3) & 1, w, n_out, col0, ldw, ksteps);
-    if ((f_src & 7) >= ksteps) return;   // narrow rows: the slot stays unused
+    const int kk = f_src % SL;
+    chunk_tile<T, MODE, KS>(p, f_src / (2 * SL), (f_src / SL) & 1, w, n_out, col0, ldw, ksteps);
+    if (kk >= ksteps) return;   // narrow rows: the slot stays unused
     const int col = min(col0 + (lane & 31), n_out - 1);   // as load_wfrag
-    load_to_lds16(w + (int64_t)col * ldw + (f_src & 7) * 16 + 8 * (lane >> 5),
+    load_to_lds16(w + (int64_t)col * ldw + kk * 16 + 8 * (lane >> 5),
                   lds_address(&lds_w[f_dst][0]));
   };
-  constexpr bool kDma = sizeof(T) == 2 && !RES;   // bf16 pair bias: its single chunk
+  constexpr bool kDma = sizeof(T) == 2 && MODE == kPairBias;   // bf16 pair bias: its single chunk
   if constexpr (RES) {
     for (int f = wave; f < IC::NFRAG; f += NW) dma_frag(f, f);
     ring_barrier<0>();
   } else if constexpr (kDma) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) dma_frag(wave * 4 + j, wave * 4 + j);
+    for (int j = 0; j < FPW; ++j) dma_frag(wave * FPW + j, wave * FPW + j);
     ring_barrier<0>();
   }
 
-  // fp32: the next chunk's fragments are prefetched into registers and stored to LDS
-  V8 pre[4];
+  // Staged path (fp32; bf16 rows of 256 channels): the next chunk's fragments are prefetched
+  // into registers and stored to LDS
+  V8 pre[FPW];
   auto fetch = [&](int ch) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int fid = wave * 4 + j;   // 16 fragments per chunk: tile = fid/8, kk = fid%8
+    for (int j = 0; j < FPW; ++j) {
+      const int fid = wave * FPW + j;   // 2*SL fragments per chunk: tile = fid/SL, kk = fid%SL
       const T* w;
       int n_out, col0, ldw, ksteps;
-      chunk_tile<T, MODE, KS>(p, ch, fid >> 3, w, n_out, col0, ldw, ksteps);
+      chunk_tile<T, MODE, KS>(p, ch, fid / SL, w, n_out, col0, ldw, ksteps);
       // (K steps beyond a narrow row re-read the last one: their slots are never used)
-      pre[j] = load_wfrag<T>(w, ldw, n_out, col0, min(fid & 7, ksteps - 1) * 16, lane);
+      pre[j] = load_wfrag<T>(w, ldw, n_out, col0, min(fid % SL, ksteps - 1) * 16, lane);
     }
   };
   auto stash = [&](int buf) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) lds_w[buf * 16 + wave * 4 + j][lane] = pre[j];
+    for (int j = 0; j < FPW; ++j) lds_w[buf * 2 * SL + wave * FPW + j][lane] = pre[j];
   };
 
   while (true) {
@@ -238,16 +259,16 @@ rowgemm_in_kernel(RowGemmInParams p) {
 
   // kTriMulOut: second fragment set = LayerNorm_out of the channel-major triangle product,
   // transposed through the staging tile 32 channels at a time.
-  RowFrags<T, RB> xf2;   // dead (and removed by the compiler) in the other modes
+  RowFrags<T, RB, SL> xf2;   // dead (and removed by the compiler) in the other modes
   if constexpr (MODE == kTriMulOut) {
     const T* x2 = (const T*)p.x2;
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb) {
-      f32x8 v[kKSteps];
-      // all four channel groups are requested at once: one memory round trip, not four
-      VE_t vec[4][C::NPASS];
+      f32x8 v[SL];
+      // all channel groups (of 32) are requested at once: one memory round trip
+      VE_t vec[SL / 2][C::NPASS];
 #pragma unroll
-      for (int cg = 0; cg < 4; ++cg)
+      for (int cg = 0; cg < SL / 2; ++cg)
 #pragma unroll
         for (int ps = 0; ps < C::NPASS; ++ps) {
           int chn, r0;
@@ -266,7 +287,7 @@ rowgemm_in_kernel(RowGemmInParams p) {
           }
         }
 #pragma unroll
-      for (int cg = 0; cg < 4; ++cg) {           // channels 32*cg .. +31
+      for (int cg = 0; cg < SL / 2; ++cg) {      // channels 32*cg .. +31
         wave_lds_sync();
 #pragma unroll
         for (int ps = 0; ps < C::NPASS; ++ps) {
@@ -358,8 +379,8 @@ rowgemm_in_kernel(RowGemmInParams p) {
     const int buf = (!RES && C::NBUF == 2) ? (ch & 1) : 0;
     if constexpr (!RES && !kDma) fetch(min(ch + 1, nch - 1));   // unconditional: static load count
     // first fragment of this chunk's two weight tiles (the resident triangle bias is one tile)
-    const int wf0 = RES ? ch * 16 : buf * 16;
-    const int wf1 = wf0 + ((RES && MODE == kTriAttnIn && ch == 8) ? 0 : kKSteps);
+    const int wf0 = RES ? ch * 2 * SL : buf * 2 * SL;
+    const int wf1 = wf0 + ((RES && MODE == kTriAttnIn && ch == nch - 1) ? 0 : SL);
     // kTriMulOut: the residual vectors of this chunk's columns, from the wave's LDS copy of z
     VE_t resv[RB][C::NPASS];
     if constexpr (MODE == kTriMulOut) {
@@ -375,7 +396,7 @@ rowgemm_in_kernel(RowGemmInParams p) {
     // Orientation: channel-major outputs want lane <-> channel (x as A operand).
     bool chan_on_lanes;
     if (MODE == kTriMulIn || MODE == kPairBias) chan_on_lanes = true;
-    else if (MODE == kTriAttnIn) chan_on_lanes = (ch >= 6);   // v^T and the triangle bias
+    else if (MODE == kTriAttnIn) chan_on_lanes = (ch >= 3 * (SL / 4));   // v^T and the triangle bias
     else chan_on_lanes = false;
 
     f32x16 acc[RB][2];
@@ -399,7 +420,7 @@ rowgemm_in_kernel(RowGemmInParams p) {
       }
     } else if constexpr (MODE == kTriMulOut) {
 #pragma unroll
-      for (int kk = 0; kk < kKSteps; ++kk) {
+      for (int kk = 0; kk < SL; ++kk) {
         const V8 w0 = lds_w[wf0 + kk][lane];
 #pragma unroll
         for (int rb = 0; rb < RB; ++rb) mma32(acc[rb][0], w0, xf2.f[rb][kk]);   // W_z LN_out(x)
@@ -430,8 +451,8 @@ rowgemm_in_kernel(RowGemmInParams p) {
     // ------------------------------ epilogues ------------------------------
     if constexpr (MODE == kTriMulIn) {
       // a/b[c][i][k] = mask * sigmoid(gate) * proj ; lane <-> channel, register <-> row
-      T* outp = (T*)p.out[ch >> 2];
-      const int c0 = (ch & 3) * 32;
+      T* outp = (T*)p.out[ch / (SL / 2)];
+      const int c0 = (ch % (SL / 2)) * 32;
       const int n_rb = (p.n + 31) >> 5, n_ks = p.pitch >> 4;
       constexpr int GT = NST < RB ? NST : RB;   // result tiles per LDS round trip
 #pragma unroll
@@ -472,7 +493,7 @@ rowgemm_in_kernel(RowGemmInParams p) {
     } else if constexpr (MODE == kTriAttnIn) {
       // Outputs in the attention core's layouts (common.h): q and the gate head-major
       // [h][p][32], K / V^T / bias in fragment-ordered key tiles.
-      const int which = ch >> 1;
+      const int which = ch / (SL / 4);
       const int key_tiles = p.pitch >> 6;
       const int q_blocks = (p.n + 31) >> 5;
       constexpr int GT = NST < 2 * RB ? NST : 2 * RB;   // result tiles per LDS round trip
@@ -504,7 +525,7 @@ rowgemm_in_kernel(RowGemmInParams p) {
 #pragma unroll
         for (int q = 0; q < GT; ++q) {
           const int rb = (k0 + q) >> 1, t = (k0 + q) & 1;
-          const int h = (ch & 1) * 2 + t;
+          const int h = (ch % (SL / 4)) * 2 + t;
           const T* stg = stile(q);
           if (which == 0 || which == 2) {
             // q and sigmoid(g): one 32 x 32 tile = one head, head-major rows
@@ -639,7 +660,7 @@ static int device_cu_count() {
 template <typename T, int MODE, int KS>
 int launch_rowgemm_in(const RowGemmInParams& p, hipStream_t stream) {
   typedef InCfg<T, MODE, KS> IC;
-  constexpr int RB = (sizeof(T) == 2 && MODE != kTriMulOut) ? 2 : 1;
+  constexpr int RB = (sizeof(T) == 2 && MODE != kTriMulOut && KS <= 8) ? 2 : 1;
   int64_t tiles = (p.n_rows + RB * 32 - 1) / (RB * 32);   // wave tiles, as in the kernel
   if (MODE == kTriMulIn) tiles = (int64_t)((p.n + 16 * RB - 1) / (16 * RB)) * (p.pitch / 8) * 4;
   if (tiles == 0) return 0;
@@ -712,7 +733,7 @@ __global__ __launch_bounds__(256, 2) void rowgemm_out_kernel(RowGemmOutParams p)
   for (int slab = 0; slab < p.n_slab; ++slab) {
     RowFrags<T, RB> af;
     if (p.a_head_major) {
-      // channel 16*kk + 8*g + t = head kk/2, d = 16*(kk%2) + 8*g + t
+      // channel 128*slab + 16*kk + 8*g + t = head 4*slab + kk/2, d = 16*(kk%2) + 8*g + t
       const int ln_ = lane & 31, g_ = lane >> 5;
 #pragma unroll
       for (int rb = 0; rb < RB; ++rb) {
@@ -720,7 +741,7 @@ __global__ __launch_bounds__(256, 2) void rowgemm_out_kernel(RowGemmOutParams p)
         pr = pr < p.n_rows ? pr : p.n_rows - 1;
 #pragma unroll
         for (int kk = 0; kk < kKSteps; ++kk)
-          af.f[rb][kk] = load8<T>((const T*)p.a + ((int64_t)(kk >> 1) * p.n_rows + pr) * 32 +
+          af.f[rb][kk] = load8<T>((const T*)p.a + ((int64_t)(slab * 4 + (kk >> 1)) * p.n_rows + pr) * 32 +
                                   16 * (kk & 1) + 8 * g_);
       }
     } else {
@@ -801,7 +822,7 @@ __global__ __launch_bounds__(256, 2) void rowgemm_out_kernel(RowGemmOutParams p)
 
 template <typename T, int NOB>
 int launch_rowgemm_out(const RowGemmOutParams& p, hipStream_t stream) {
-  constexpr int RB = sizeof(T) == 2 ? 2 : 1;
+  constexpr int RB = (sizeof(T) == 2 && NOB <= 4) ? 2 : 1;
   const int64_t rows_per_block = 4 * RB * 32;
   const int64_t blocks = (p.n_rows + rows_per_block - 1) / rows_per_block;
   if (blocks == 0) return 0;
@@ -838,8 +859,12 @@ int trimul_project(const void* z, const void* mask, const void* ln_w, const void
   p.mmap = pair_map(n, 1, incoming != 0);
   p.n = n;
   p.pitch = k_pitch;
-  return c_z == 64 ? launch_rowgemm_in<T, kTriMulIn, 4>(p, stream)
-                   : launch_rowgemm_in<T, kTriMulIn, 8>(p, stream);
+  if (c_z == 64) return launch_rowgemm_in<T, kTriMulIn, 4>(p, stream);
+  if (c_z == 256) {
+    if constexpr (sizeof(T) == 2) return launch_rowgemm_in<T, kTriMulIn, 16>(p, stream);
+    else return -1;   // 256-channel rows are built for bf16 only (refused by the caller)
+  }
+  return launch_rowgemm_in<T, kTriMulIn, 8>(p, stream);
 }
 
 template <typename T>
@@ -860,8 +885,12 @@ int trimul_output(const void* x, const void* z, const void* ln_in_w, const void*
   p.gamma2 = ln_out_w;
   p.beta2 = ln_out_b;
   p.add_residual = add_residual;
-  return c_z == 64 ? launch_rowgemm_in<T, kTriMulOut, 4>(p, stream)
-                   : launch_rowgemm_in<T, kTriMulOut, 8>(p, stream);
+  if (c_z == 64) return launch_rowgemm_in<T, kTriMulOut, 4>(p, stream);
+  if (c_z == 256) {
+    if constexpr (sizeof(T) == 2) return launch_rowgemm_in<T, kTriMulOut, 16>(p, stream);
+    else return -1;   // 256-channel rows are built for bf16 only (refused by the caller)
+  }
+  return launch_rowgemm_in<T, kTriMulOut, 8>(p, stream);
 }
 
 template <typename T>
@@ -882,8 +911,12 @@ int triattn_project(const void* z, const void* ln_w, const void* ln_b, const voi
   p.aux = heads;
   p.pitch = key_pitch;
   p.q_scale = 1.0f / sqrtf((float)d);
-  return c_z == 64 ? launch_rowgemm_in<T, kTriAttnIn, 4>(p, stream)
-                   : launch_rowgemm_in<T, kTriAttnIn, 8>(p, stream);
+  if (c_z == 64) return launch_rowgemm_in<T, kTriAttnIn, 4>(p, stream);
+  if (c_z == 256) {
+    if constexpr (sizeof(T) == 2) return launch_rowgemm_in<T, kTriAttnIn, 16>(p, stream);
+    else return -1;   // 256-channel rows are built for bf16 only (refused by the caller)
+  }
+  return launch_rowgemm_in<T, kTriAttnIn, 8>(p, stream);
 }
 
 template <typename T>
@@ -892,21 +925,26 @@ int triattn_output(const void* o, const void* w_o, const void* z, void* out, int
   RowGemmOutParams p = {};
   p.a = o;
   p.a_head_major = 1;
-  p.n_slab = 1;
+  p.n_slab = c_z == 256 ? 2 : 1;   // K = heads * 32 = 128, or 256 with the scaled-up hidden width
   p.w = w_o;
   p.res = add_residual ? z : nullptr;
   p.out = out;
   p.omap = pair_map(n, c_z, transposed != 0);
   p.n_rows = (int64_t)n * n;
-  return c_z == 64 ? launch_rowgemm_out<T, 2>(p, stream) : launch_rowgemm_out<T, 4>(p, stream);
+  if (c_z == 64) return launch_rowgemm_out<T, 2>(p, stream);
+  if (c_z == 256) {
+    if constexpr (sizeof(T) == 2) return launch_rowgemm_out<T, 8>(p, stream);
+    else return -1;
+  }
+  return launch_rowgemm_out<T, 4>(p, stream);
 }
 
 template <typename T>
 int pair_bias_fwd(const void* z, const void* ln_w, const void* ln_b, const void* w, void* bias,
-                  int n, int heads, int out_f32, float eps, hipStream_t stream) {
+                  int n, int c_z, int heads, int out_f32, float eps, hipStream_t stream) {
   RowGemmInParams p = {};
   p.x = z;
-  p.xmap = pair_map(n, kC, false);
+  p.xmap = pair_map(n, c_z, false);
   p.n_rows = (int64_t)n * n;
   p.gamma = ln_w;
   p.beta = ln_b;
@@ -915,6 +953,10 @@ int pair_bias_fwd(const void* z, const void* ln_w, const void* ln_b, const void*
   p.out[0] = bias;
   p.n = n;
   p.aux = heads | (out_f32 ? 0x100 : 0);
+  if (c_z == 256) {
+    if constexpr (sizeof(T) == 2) return launch_rowgemm_in<T, kPairBias, 16>(p, stream);
+    else return -1;
+  }
   return launch_rowgemm_in<T, kPairBias, 8>(p, stream);
 }
 
@@ -932,7 +974,7 @@ int pair_bias_fwd(const void* z, const void* ln_w, const void* ln_b, const void*
   template int triattn_output<T>(const void*, const void*, const void*, void*, int, int, int, int, \
                                  hipStream_t);                                                     \
   template int pair_bias_fwd<T>(const void*, const void*, const void*, const void*, void*, int,    \
-                                int, int, float, hipStream_t);
+                                int, int, int, float, hipStream_t);
 PTX_INSTANTIATE(float)
 PTX_INSTANTIATE(bf16_t)
 #undef PTX_INSTANTIATE

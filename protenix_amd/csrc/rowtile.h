@@ -37,9 +37,10 @@ struct RowFrags {
   PTX_REP8(x), PTX_REP8(x), PTX_REP8(x), PTX_REP8(x), PTX_REP8(x), PTX_REP8(x), PTX_REP8(x),   \
       PTX_REP8(x), PTX_REP8(x), PTX_REP8(x), PTX_REP8(x), PTX_REP8(x), PTX_REP8(x), PTX_REP8(x), \
       PTX_REP8(x), PTX_REP8(x)
-static __device__ const float kOnesF32[kC] = {PTX_REP128(1.0f)};
-static __device__ const uint16_t kOnesBf16[kC] = {PTX_REP128(0x3F80)};
-static __device__ const float kZerosAny[kC] = {PTX_REP128(0.0f)};
+// (256 entries: the widest row)
+static __device__ const float kOnesF32[2 * kC] = {PTX_REP128(1.0f), PTX_REP128(1.0f)};
+static __device__ const uint16_t kOnesBf16[2 * kC] = {PTX_REP128(0x3F80), PTX_REP128(0x3F80)};
+static __device__ const float kZerosAny[2 * kC] = {PTX_REP128(0.0f), PTX_REP128(0.0f)};
 #undef PTX_REP128
 #undef PTX_REP8
 template <typename T> __device__ __forceinline__ const T* default_gamma();

@@ -27,10 +27,12 @@
 
 namespace ptx {
 
-// KS = K steps of a row (c / 16: 8 for c = 128, 4 for c = 64); NOB = c / 32 output blocks.
+// KS = K steps of a row (c / 16: 8 for c = 128, 4 for c = 64, 16 for c = 256);
+// NOB = c / 32 output blocks.
 template <typename T, int KS> struct TrCfg {
-  static constexpr int RB = sizeof(T) == 2 ? 2 : 1;     // row blocks of 32 per wave
-  static constexpr int NBUF = sizeof(T) == 2 ? 4 : 3;   // chunk buffers in LDS
+  // (rows of 256 channels, bf16 only: one row block, and three 48 KB chunk buffers)
+  static constexpr int RB = (sizeof(T) == 2 && KS <= 8) ? 2 : 1;     // row blocks of 32 per wave
+  static constexpr int NBUF = (sizeof(T) == 2 && KS <= 8) ? 4 : 3;   // chunk buffers in LDS
   static constexpr int D = NBUF - 2;                    // chunks the loads run ahead (two are in use)
   static constexpr int PIECES = (int)sizeof(T) / 2;     // 16-byte pieces per lane and fragment
   static constexpr int NOB = KS / 2;
@@ -280,8 +282,9 @@ static int transition_pack_ks(const void* w_a, const void* w_b, const void* w_o,
 template <typename T>
 int transition_pack(const void* w_a, const void* w_b, const void* w_o, void* packed, int c,
                     int n_factor, hipStream_t stream) {
-  return c == 64 ? transition_pack_ks<T, 4>(w_a, w_b, w_o, packed, n_factor, stream)
-                 : transition_pack_ks<T, 8>(w_a, w_b, w_o, packed, n_factor, stream);
+  if (c == 64) return transition_pack_ks<T, 4>(w_a, w_b, w_o, packed, n_factor, stream);
+  if (c == 256) return transition_pack_ks<T, 16>(w_a, w_b, w_o, packed, n_factor, stream);
+  return transition_pack_ks<T, 8>(w_a, w_b, w_o, packed, n_factor, stream);
 }
 
 template <typename T, int KS>
@@ -301,10 +304,19 @@ int transition_fwd(const void* x, const void* ln_w, const void* ln_b, const void
                    void* out, int64_t rows, int c, int n_factor, int add_residual, float eps,
                    hipStream_t stream) {
   if (rows == 0) return 0;
-  return c == 64 ? transition_fwd_ks<T, 4>(x, ln_w, ln_b, packed, out, rows, n_factor,
-                                           add_residual, eps, stream)
-                 : transition_fwd_ks<T, 8>(x, ln_w, ln_b, packed, out, rows, n_factor,
-                                           add_residual, eps, stream);
+  if (c == 64)
+    return transition_fwd_ks<T, 4>(x, ln_w, ln_b, packed, out, rows, n_factor, add_residual, eps,
+                                   stream);
+  if (c == 256) {
+    // bf16 only: an fp32 chunk of weights (96 KB) leaves no room for a ring in LDS
+    if constexpr (sizeof(T) == 2)
+      return transition_fwd_ks<T, 16>(x, ln_w, ln_b, packed, out, rows, n_factor, add_residual,
+                                      eps, stream);
+    else
+      return -1;
+  }
+  return transition_fwd_ks<T, 8>(x, ln_w, ln_b, packed, out, rows, n_factor, add_residual, eps,
+                                 stream);
 }
 
 template int transition_pack<float>(const void*, const void*, const void*, void*, int, int,

@@ -2,7 +2,7 @@
 
 Mirrors protenix/model/modules/primitives.py:33-101 (Linear / LinearNoBias),
 :166-230 (Transition) and protenix/model/triangular/layers.py:104-197
-(OpenfoldLinear, by its initialiser names).  The pair Transition (c_in = 64 or 128)
+(OpenfoldLinear, by its initialiser names).  The pair Transition (c_in = 64, 128, or 256 in bf16)
 runs on the fused HIP kernels; other widths (the single track, c_in = 384) use
 the HIP LayerNorm and library GEMMs.
 """
@@ -111,7 +111,8 @@ class Transition(nn.Module):
         x + update there instead and returns it."""
         _forward_only(x, *self.parameters())
         add = _residual_out is not None
-        if self.c_in in (64, 128) and (self.n * self.c_in) % 64 == 0:
+        fused = self.c_in in (64, 128) or (self.c_in == 256 and x.dtype == torch.bfloat16)
+        if fused and (self.n * self.c_in) % 64 == 0:
             return ops.transition(x, self._weights(x.dtype, x.device), self.n, add_residual=add,
                                   out=_residual_out)
         # other widths: HIP LayerNorm + library GEMMs

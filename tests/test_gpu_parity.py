@@ -254,3 +254,65 @@ def test_template_pair_stack_cz64(dtype):
         _, z_ref = ref(None, z.float(), pm.float())
         s_got, z_got = prod(None, z.cuda(), pm.cuda())
     assert s_got is None and rel_err(z_got, z_ref) <= tol(dtype)
+
+
+# ------------------------------------------------------------------ c_z = 256 (scaled-up hidden widths, bf16)
+BF16 = torch.bfloat16
+
+
+@pytest.mark.parametrize("cls", ["TriangleMultiplicationOutgoing", "TriangleMultiplicationIncoming"])
+@pytest.mark.parametrize("n,n_pad", [(64, 0), (100, 7), (37, 0)])
+def test_trimul_cz256(cls, n, n_pad):
+    """c_z = c_hidden = 256, as `hidden_scale_up` gives (pairformer.py:76-78 of the reference)."""
+    ref, prod = oracle_and_product(getattr(O, cls), getattr(P, cls), 256, 256, dtype=BF16)
+    z = _z(n, BF16, c=256)
+    mask = pad_mask(n, n_pad, BF16) if n_pad else None
+    with torch.no_grad():
+        want = ref(z.float(), None if mask is None else mask.float())
+        got = prod(z.cuda(), None if mask is None else mask.cuda())
+        assert got.shape == want.shape and rel_err(got, want) <= tol(BF16)
+        zc = z.cuda().clone()
+        got2 = prod(zc, None if mask is None else mask.cuda(), inplace_safe=True, _add_with_inplace=True)
+        assert rel_err(got2, z.float() + want) <= tol(BF16)
+
+
+@pytest.mark.parametrize("starting", [True, False])
+@pytest.mark.parametrize("n,n_pad", [(64, 0), (100, 7), (37, 5)])
+def test_triattn_cz256(starting, n, n_pad):
+    ref, prod = oracle_and_product(O.TriangleAttention, P.TriangleAttention, 256, 32, 8,
+                                   starting=starting, dtype=BF16)
+    z = _z(n, BF16, c=256)
+    mask = pad_mask(n, n_pad, BF16) if n_pad else None
+    with torch.no_grad():
+        want = ref(z.float(), None if mask is None else mask.float(), chunk_size=64)
+        got = prod(z.cuda(), None if mask is None else mask.cuda())
+    assert got.shape == want.shape and rel_err(got, want) <= tol(BF16)
+
+
+@pytest.mark.parametrize("shape,factor", [((1, 50, 50, 256), 4), ((3001, 256), 2)])
+def test_transition_cz256(shape, factor):
+    ref, prod = oracle_and_product(O.Transition, P.Transition, 256, factor, dtype=BF16)
+    x = torch.randn(*shape, generator=torch.Generator().manual_seed(11)).to(BF16)
+    with torch.no_grad():
+        assert rel_err(prod(x.cuda()), ref(x.float())) <= tol(BF16)
+        xc = x.cuda().clone()
+        got = prod(xc, _residual_out=xc)
+        assert rel_err(got, x.float() + ref(x.float())) <= tol(BF16)
+
+
+def test_block_cz256_scaled_up():
+    """A block as the scaled-up model builds it: c_z = 256, hidden_scale_up (8 pair heads,
+    c_hidden_mul = 256), with the single track."""
+    kw = dict(c_z=256, hidden_scale_up=True)
+    ref, prod = oracle_and_product(O.PairformerBlock, P.PairformerBlock, dtype=BF16, **kw)
+    s, z, pm = O.make_inputs(72, c_z=256, n_pad=5, dtype=BF16)
+    with torch.no_grad():
+        s_ref, z_ref = ref(s.float(), z.float(), pm.float())
+        s_got, z_got = prod(s.cuda(), z.cuda(), pm.cuda())
+    assert rel_err(z_got, z_ref) <= tol(BF16) and rel_err(s_got, s_ref) <= tol(BF16)
+
+
+def test_cz256_fp32_is_refused():
+    blk = P.TriangleMultiplicationOutgoing(256, 256).cuda()
+    with torch.no_grad(), pytest.raises(RuntimeError, match="unsupported"):
+        blk(torch.randn(1, 8, 8, 256, device="cuda"))
