@@ -100,7 +100,8 @@ PTX_API int ptx_layernorm_fwd(const void* x, const void* gamma, const void* beta
  *   w_* [c_hidden][c_z]; a, b: workspaces of ptx_trimul_operand_elems(n, c_hidden)
  *   elements each, written in the contraction's operand order (K between n and
  *   k_pitch is written as zeros, rows beyond n stay unwritten);
- *   k_pitch = ptx_key_pitch(n).  c_z = 64 or 128, c_hidden = 128.
+ *   k_pitch = ptx_key_pitch(n).  Widths: c_z = 64 or 128 with c_hidden = 128, or
+ *   (bf16 only) c_z = c_hidden = 256.
  */
 PTX_API int ptx_trimul_project(const void* z, const void* mask, const void* ln_w, const void* ln_b,
                        const void* w_ap, const void* w_ag, const void* w_bp, const void* w_bg,
@@ -121,7 +122,7 @@ PTX_API int ptx_trimul_contract(const void* a, const void* b, void* x, int n, in
  * Triangle multiplication, stage 3 (triangular.py:560-565):
  *   out = [residual z +] W_z LN_out(x) * sigmoid(W_g LN_in(z))
  *   x [c_hidden][n][n] from stage 2, z [n][n][c_z], out [n][n][c_z] (may alias z);
- *   w_z [c_z][c_hidden], w_g [c_z][c_z].  c_z = 64 or 128, c_hidden = 128.
+ *   w_z [c_z][c_hidden], w_g [c_z][c_z].  Widths as for stage 1.
  * add_residual = 1 gives z + update (the reference's `_add_with_inplace`).
  */
 PTX_API int ptx_trimul_output(const void* x, const void* z, const void* ln_in_w, const void* ln_in_b,
@@ -136,8 +137,9 @@ PTX_API int ptx_trimul_output(const void* x, const void* z, const void* ln_in_w,
  * over logical rows p = i*n + j of x = z (transposed = 0) or z^T (transposed = 1).
  *   q, g [heads][n][n][d] (logical row p = i*n + j);  k, vt: workspaces of
  *   ptx_triattn_kv_elems(n, heads) elements;  tri_bias: ptx_triattn_bias_elems(n, heads)
- *   elements;  key_pitch = ptx_key_pitch(n).   c_in = 64 or 128, heads = 4, d = 32
- *   (w_q, w_k, w_v, w_g [heads*d][c_in], w_b [heads][c_in]).
+ *   elements;  key_pitch = ptx_key_pitch(n).   d = 32;  c_in = 64 or 128 with 4 heads,
+ *   or (bf16 only) c_in = 256 with 8 heads  (w_q, w_k, w_v, w_g [heads*d][c_in],
+ *   w_b [heads][c_in]).
  */
 PTX_API int ptx_triattn_project(const void* z, const void* ln_w, const void* ln_b, const void* w_q,
                         const void* w_k, const void* w_v, const void* w_g, const void* w_b,
@@ -165,7 +167,8 @@ PTX_API int ptx_triattn_fwd(const void* q, const void* k, const void* vt, const 
  * Triangle attention, stage 3 (layers.py:392-396 + the caller's residual add,
  * pairformer.py:189-213):  out(p) = [z(p) +] W_o o[p], where logical row p maps
  * to z[i][j] or, transposed = 1, z[j][i].  o [heads][n][n][d] as written by
- * stage 2; w_o [c_in][heads*d]; out may alias z.  c_in = 64 or 128, heads*d = 128.
+ * stage 2; w_o [c_in][heads*d]; out may alias z.  c_in = 64 or 128 (heads*d = 128), or
+ * (bf16 only) c_in = heads*d = 256.
  */
 PTX_API int ptx_triattn_output(const void* o, const void* w_o, const void* z, void* out, int n,
                        int c_in, int transposed, int add_residual, int dtype, void* stream);
@@ -180,8 +183,8 @@ PTX_API int ptx_triattn_output(const void* o, const void* w_o, const void* z, vo
  *     packed, ptx_transition_packed_elems(c, n_factor) = 3*n_factor*c*c elements.
  *   ptx_transition_fwd:   x, out [rows][c] (out may alias x), ln_w / ln_b may be NULL.
  * a and b stay in fp32 through the activation (the reference rounds them to the
- * storage dtype first); the product is rounded once.   c = 64 or 128, n_factor*c a
- * multiple of 64.
+ * storage dtype first); the product is rounded once.   c = 64, 128 or (bf16 only) 256;
+ * n_factor*c a multiple of 64.
  */
 PTX_API int64_t ptx_transition_packed_elems(int c, int n_factor);
 PTX_API int ptx_transition_pack(const void* w_a, const void* w_b, const void* w_o, void* packed, int c,
@@ -192,7 +195,8 @@ PTX_API int ptx_transition_fwd(const void* x, const void* ln_w, const void* ln_b
 
 /*
  * Pair bias of the single-representation attention (transformer.py:191-194):
- *   bias[h][i][j] = (W LN(z[i][j]))[h],  W [heads][c_z], heads <= 32, c_z = 128.
+ *   bias[h][i][j] = (W LN(z[i][j]))[h],  W [heads][c_z], heads <= 32, c_z = 128 or
+ * (bf16 only) 256.
  * ln_b may be NULL.  bias is fp32 when out_f32 = 1, else `dtype`.
  */
 PTX_API int ptx_pair_bias_fwd(const void* z, const void* ln_w, const void* ln_b, const void* w,

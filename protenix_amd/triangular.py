@@ -6,8 +6,9 @@ Update and its Outgoing/Incoming flavours) and :589-727 (TriangleAttention),
 with the attention sub-module of protenix/model/triangular/layers.py:299-473
 kept as the parameter container `mha`.  The kernel-selection strings of the
 reference are accepted and validated; every valid value runs the HIP kernels.
-Forward only, c_z = 64 or 128 with c_hidden = 128 and 4 heads x 32 (anything else is
-refused by the library with an "unsupported shape" error).
+Forward only; widths: c_z = 64 or 128 with c_hidden = 128 and 4 heads x 32, or (bf16, also
+fp32 tensors under bf16 autocast) c_z = c_hidden = 256 with 8 heads x 32.  Anything else is
+refused by the library with an "unsupported shape" error.
 """
 from __future__ import annotations
 
