@@ -134,6 +134,7 @@ PTX_API int ptx_trimul_output(const void* x, const void* z, const void* ln_in_w,
  * Triangle attention, stage 1 (triangular.py:683-692, layers.py:361-382, 386):
  *   xn = LN(x);  q = W_q xn / sqrt(d);  k = W_k xn;  v = W_v xn;
  *   g = sigmoid(W_g xn);  tri_bias = W_b xn
+ * (q and tri_bias are stored multiplied by log2(e): stage 2 exponentiates in base 2)
  * over logical rows p = i*n + j of x = z (transposed = 0) or z^T (transposed = 1).
  *   q, g [heads][n][n][d] (logical row p = i*n + j);  k, vt: workspaces of
  *   ptx_triattn_kv_elems(n, heads) elements;  tri_bias: ptx_triattn_bias_elems(n, heads)

@@ -44,7 +44,7 @@ struct RowGemmInParams {
   int n;                // tokens (n_rows = n*n for pair tensors)
   int pitch;            // row pitch of a, b (TRIMUL_IN) / v^T, triangle bias (TRIATTN_IN)
   int aux;              // TRIATTN_IN: heads; PAIRBIAS: heads | out_f32 << 8; TRANSITION_IN: n_factor
-  float q_scale;        // TRIATTN_IN: 1/sqrt(d)
+  float q_scale;        // TRIATTN_IN: log2(e)/sqrt(d)
   // TRIMUL_OUT only
   const void* x2;       // channel-major triangle product [128][n_rows]
   const void* gamma2;
@@ -501,7 +501,7 @@ rowgemm_in_kernel(RowGemmInParams p) {
       for (int k0 = 0; k0 < 2 * RB; k0 += GT) {
         // the group's result tiles go to the staging tiles first ...
         wave_lds_sync();
-        auto put_group = [&](auto kind) {   // kind: 0 = q (rounded, then scaled), 2 = gate, 1 = as is
+        auto put_group = [&](auto kind) {   // kind: 0 = q (rounded, then scaled), 2 = gate, 3 = bias, 1 = as is
           constexpr int KIND = decltype(kind)::value;
 #pragma unroll
           for (int q = 0; q < GT; ++q) {
@@ -512,6 +512,7 @@ rowgemm_in_kernel(RowGemmInParams p) {
               float v = acc[rb][t][r];
               if (KIND == 0) v = to_f32(from_f32<T>(v)) * p.q_scale;
               if (KIND == 2) v = sigmoidf_fast(v);
+              if (KIND == 3) v *= 1.4426950408889634f;   // log2(e): the attention core works in log2 units
               vals[r] = v;
             }
             stage_put<T>(stile(q), vals, lane);
@@ -519,6 +520,7 @@ rowgemm_in_kernel(RowGemmInParams p) {
         };
         if (which == 0) put_group(std::integral_constant<int, 0>{});
         else if (which == 2) put_group(std::integral_constant<int, 2>{});
+        else if (which == 4) put_group(std::integral_constant<int, 3>{});
         else put_group(std::integral_constant<int, 1>{});
         wave_lds_sync();
         // ... and are then read back as 16-byte vectors and stored
@@ -910,7 +912,7 @@ int triattn_project(const void* z, const void* ln_w, const void* ln_b, const voi
   p.n = n;
   p.aux = heads;
   p.pitch = key_pitch;
-  p.q_scale = 1.0f / sqrtf((float)d);
+  p.q_scale = 1.4426950408889634f / sqrtf((float)d);   // log2(e) / sqrt(d), see triattn.hip
   if (c_z == 64) return launch_rowgemm_in<T, kTriAttnIn, 4>(p, stream);
   if (c_z == 256) {
     if constexpr (sizeof(T) == 2) return launch_rowgemm_in<T, kTriAttnIn, 16>(p, stream);

@@ -13,8 +13,9 @@
 // keys -> 16-byte bias loads, and 8 consecutive keys per P.V operand slot group.
 // The triangle bias never touches the vector ALU: its raw bf16 registers are the
 // B operand of an MFMA whose A operand is the constant 0/1 matrix that undoes the
-// key permutation, accumulating straight into S^T.  Per logit the vector ALU
-// executes one fma, one exp2, half a max3 and half a packed bf16 convert.
+// key permutation, accumulating straight into S^T.  q and the bias are stored multiplied
+// by log2(e) (by the projection kernel), so on the common path the vector ALU executes per
+// logit one exp2, half a packed bf16 convert and a quarter of a dot2 (the row sum).
 // K and V^T tiles are shared by the 4 waves through LDS in fragment order
 // (double-buffered, one barrier per tile); the bias tile is private to a wave
 // and read straight from global (L2-resident: workgroups are numbered so that
@@ -37,8 +38,12 @@ constexpr int kKeyTile = 64;
 constexpr float kLog2e = 1.4426950408889634f;
 // tile_row: code paths, and the largest per-lane probability sum of a tile (32 values) the
 // optimistic path accepts
-enum { kOptimistic = 0, kClassic = 1, kMasked = 2 };
+enum { kOptimistic = 0, kClassic = 1, kMasked = 2, kOptimisticZero = 3 };
 constexpr float kOptimisticLimit = 1.0e12f;
+constexpr float kLn2 = 0.6931471805599453f;
+// kClassic: a running maximum no larger than this (natural units, all lanes of the wave) is
+// replaced by the reference 0, which makes exp2() of the raw logit the probability
+constexpr float kZeroReferenceLimit = 14.0f;
 
 // Rows of the pair tensor handled by one wave (the bias tile is then loaded once per key
 // tile and reused).  More than one row does not fit the register budget of 2 waves/SIMD.
@@ -174,13 +179,18 @@ __global__ __launch_bounds__(256, 2) void triattn_fwd_kernel(
   // One key tile of one row: logits, online softmax, P.V.  `tb` was fetched one tile ago.
   // Three complete instantiations, so that the rarer paths share no code with - and cannot
   // be speculated into - the common one:
-  //   kOptimistic  the common path.  The softmax reference m_run only has to keep exp() in
+  //   kOptimistic  The softmax reference m_run only has to keep exp() in
   //                range, so it is NOT updated: probabilities are taken against the reference
   //                left by earlier tiles, no tile maximum is formed and O, l are not rescaled.
   //                If a probability sum leaves the safe range (a logit ~28 above the
   //                reference, or no reference yet), nothing has been committed and the tile
   //                is redone by kClassic.  Returns false in that case (same in all lanes).
-  //   kClassic     running maximum, rescale of O and l (first tile, or redo).
+  //   kOptimisticZero  the common path: the same with the reference 0 in all lanes.  q and
+  //                the triangle bias arrive multiplied by log2(e), so the matrix pipe's
+  //                result IS the exponent: one v_exp_f32 per logit and no other arithmetic.
+  //   kClassic     running maximum, rescale of O and l (first tile, or redo).  A maximum of
+  //                modest size is replaced by the reference 0 (any reference is exact as long
+  //                as exp() stays in range), which puts the row on the kOptimisticZero path.
   //   kMasked      tiles with a masked or out-of-range key: the reference's exact fp32
   //                order (q.k + mask_bias) + triangle_bias.
   auto tile_row = [&](auto mode_tag, int buf, int r, V8 (&tb)[2][2], int next_tile) -> bool {
@@ -222,14 +232,15 @@ __global__ __launch_bounds__(256, 2) void triattn_fwd_kernel(
 #pragma unroll
           for (int t = 0; t < 8; ++t) {
             const float mbv = t < 4 ? m0[t & 3] : m1[t & 3];
-            const float v = (s[u][8 * c + t] + mbv) + b[t];
+            // q.k and the bias arrive in log2 units: back to natural ones for this sum
+            const float v = (s[u][8 * c + t] * kLn2 + mbv) + b[t] * kLn2;
             s[u][8 * c + t] = mbv == -INFINITY ? -INFINITY : v;   // key beyond n
           }
         }
     }
 
     float alpha = 1.0f;
-    if constexpr (MODE != kOptimistic) {
+    if constexpr (MODE == kClassic || MODE == kMasked) {
       refill_bias();
       float mx[8];
 #pragma unroll
@@ -238,19 +249,27 @@ __global__ __launch_bounds__(256, 2) void triattn_fwd_kernel(
       float mt = fmaxf(fmaxf(fmaxf(mx[0], mx[1]), fmaxf(mx[2], mx[3])),
                        fmaxf(fmaxf(mx[4], mx[5]), fmaxf(mx[6], mx[7])));
       mt = fmaxf(mt, swap32(mt));
-      const float m_new = fmaxf(m_run[r], mt);        // finite: key0 < n is never excluded
+      if (!MASKED) mt *= kLn2;                        // unmasked logits are in log2 units
+      float m_new = fmaxf(m_run[r], mt);              // finite: key0 < n is never excluded
+      if (!MASKED && __ballot(!(fabsf(m_new) < kZeroReferenceLimit)) == 0ull) m_new = 0.0f;
       alpha = fast_exp2((m_run[r] - m_new) * kLog2e);   // 1 when the max did not move
       m_run[r] = m_new;
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc_o[r][e] *= alpha;
     }
 
-    if constexpr (!MASKED) {
+    if constexpr (MODE == kOptimisticZero) {
+      // reference 0: the logit in log2 units is the exponent
+#pragma unroll
+      for (int u = 0; u < 2; ++u)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) s[u][e] = fast_exp2(s[u][e]);
+    } else if constexpr (!MASKED) {
       const float nml = -m_run[r] * kLog2e;
 #pragma unroll
       for (int u = 0; u < 2; ++u)
 #pragma unroll
-        for (int e = 0; e < 16; ++e) s[u][e] = fast_exp2(fmaf(s[u][e], kLog2e, nml));
+        for (int e = 0; e < 16; ++e) s[u][e] = fast_exp2(s[u][e] + nml);
     } else {
       // (s - m) first: exact when both sit near -1e9
 #pragma unroll
@@ -287,7 +306,7 @@ __global__ __launch_bounds__(256, 2) void triattn_fwd_kernel(
           for (int t = 0; t < 8; ++t) psum += p8[t];
         }
       }
-    if constexpr (MODE == kOptimistic) {
+    if constexpr (MODE == kOptimistic || MODE == kOptimisticZero) {
       // out of the safe range (also catches inf and NaN)?  Nothing committed yet: redo.
       if (__ballot(!(psum < kOptimisticLimit)) != 0ull) return false;
       refill_bias();
@@ -312,7 +331,12 @@ __global__ __launch_bounds__(256, 2) void triattn_fwd_kernel(
         tile_row(std::integral_constant<int, kMasked>{}, buf, r, tb, nt);
       } else {
         bool done = false;
-        if (tile != 0) done = tile_row(std::integral_constant<int, kOptimistic>{}, buf, r, tb, nt);
+        if (tile != 0) {
+          if (__ballot(m_run[r] != 0.0f) == 0ull)
+            done = tile_row(std::integral_constant<int, kOptimisticZero>{}, buf, r, tb, nt);
+          else
+            done = tile_row(std::integral_constant<int, kOptimistic>{}, buf, r, tb, nt);
+        }
         if (!done) tile_row(std::integral_constant<int, kClassic>{}, buf, r, tb, nt);
       }
     }
