@@ -3,6 +3,7 @@ TriangleMultiplication*, TriangleAttention, LayerNorm, Transition,
 AttentionPairBias, PairformerBlock and PairformerStack, backed by hand-written
 gfx950 kernels in libprotenix_amd.so (C ABI: include/protenix_amd.h)."""
 
+from .graph import Graphed
 from .layer_norm import FusedLayerNorm, LayerNorm
 from .pairformer import PairformerBlock, PairformerStack
 from .primitives import Linear, LinearNoBias, Transition
@@ -17,6 +18,7 @@ from .triangular import (
 )
 
 __all__ = [
+    "Graphed",
     "AttentionPairBias", "FusedLayerNorm", "LayerNorm", "Linear", "LinearNoBias",
     "PairformerBlock", "PairformerStack", "Transition", "TriangleAttention",
     "TriangleAttentionEndingNode", "TriangleAttentionStartingNode",

@@ -86,6 +86,10 @@ __global__ __launch_bounds__(256, 2) void triattn_fwd_kernel(
   // queries all lie beyond n re-reads the last query block; nothing of either is stored.
   const T* b_tiles = bias + ((int64_t)h * q_blocks + min(q0 >> 5, q_blocks - 1)) * key_tiles * kAttnTileElems + lane * 8;
   const int qi = min(q0 + ln, n - 1);
+  // Lanes whose query lies beyond n compute on whatever the bias workspace holds there; they
+  // store nothing, and they are kept out of the wave-wide decisions below so that the path a
+  // wave takes (and with it the rounding of its valid queries) never depends on that content.
+  const bool q_ok = q0 + ln < n;
 
   // Q fragments (B operand): lane <-> query, slots <-> d = 16*kk + 8*g + t
   V8 qf[R][2];
@@ -251,7 +255,7 @@ __global__ __launch_bounds__(256, 2) void triattn_fwd_kernel(
       mt = fmaxf(mt, swap32(mt));
       if (!MASKED) mt *= kLn2;                        // unmasked logits are in log2 units
       float m_new = fmaxf(m_run[r], mt);              // finite: key0 < n is never excluded
-      if (!MASKED && __ballot(!(fabsf(m_new) < kZeroReferenceLimit)) == 0ull) m_new = 0.0f;
+      if (!MASKED && __ballot(q_ok && !(fabsf(m_new) < kZeroReferenceLimit)) == 0ull) m_new = 0.0f;
       alpha = fast_exp2((m_run[r] - m_new) * kLog2e);   // 1 when the max did not move
       m_run[r] = m_new;
 #pragma unroll
@@ -308,7 +312,7 @@ __global__ __launch_bounds__(256, 2) void triattn_fwd_kernel(
       }
     if constexpr (MODE == kOptimistic || MODE == kOptimisticZero) {
       // out of the safe range (also catches inf and NaN)?  Nothing committed yet: redo.
-      if (__ballot(!(psum < kOptimisticLimit)) != 0ull) return false;
+      if (__ballot(q_ok && !(psum < kOptimisticLimit)) != 0ull) return false;
       refill_bias();
     }
     l_run[r] = l_run[r] * alpha + psum;
@@ -332,7 +336,7 @@ __global__ __launch_bounds__(256, 2) void triattn_fwd_kernel(
       } else {
         bool done = false;
         if (tile != 0) {
-          if (__ballot(m_run[r] != 0.0f) == 0ull)
+          if (__ballot(q_ok && m_run[r] != 0.0f) == 0ull)
             done = tile_row(std::integral_constant<int, kOptimisticZero>{}, buf, r, tb, nt);
           else
             done = tile_row(std::integral_constant<int, kOptimistic>{}, buf, r, tb, nt);

@@ -16,8 +16,14 @@ import torch.nn as nn
 from . import ops
 
 
-def _forward_only(*tensors: Optional[torch.Tensor]) -> None:
-    if torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in tensors):
+def _forward_only(*tensors: Optional[torch.Tensor], module: Optional[nn.Module] = None) -> None:
+    """Refuses inputs (and, with `module`, parameters) that would need a backward pass.
+    Under torch.no_grad() nothing is inspected: the parameter walk is not free."""
+    if not torch.is_grad_enabled():
+        return
+    if module is not None:
+        tensors = tensors + tuple(module.parameters())
+    if any(t is not None and t.requires_grad for t in tensors):
         raise RuntimeError(
             "protenix_amd kernels are forward-only: call under torch.no_grad() "
             "(backward kernels are not part of this build)")

@@ -109,6 +109,17 @@ def layer_norm(x: torch.Tensor, weight: Optional[torch.Tensor], bias: Optional[t
     return (y, mean, rstd) if return_stats else y
 
 
+# Workspaces are handed to the kernels uninitialised.  With `poison_workspaces` set (tests),
+# they are filled with NaN first: no result may depend on what a workspace held before.
+poison_workspaces = False
+
+
+def _workspace(shape, dtype, device) -> torch.Tensor:
+    if poison_workspaces:
+        return torch.full(shape, float("nan"), dtype=dtype, device=device)
+    return torch.empty(shape, dtype=dtype, device=device)
+
+
 def _mask_for(mask: Optional[torch.Tensor], z: torch.Tensor) -> Optional[torch.Tensor]:
     if mask is None:
         return None
@@ -129,13 +140,13 @@ def triangle_multiplication(z: torch.Tensor, mask: Optional[torch.Tensor], w: di
     mask = _mask_for(mask, z)
     # contraction operands in the library's fragment order (see include/protenix_amd.h)
     n_op = lib.ptx_trimul_operand_elems(n, c_h)
-    a = torch.empty((n_op,), dtype=z.dtype, device=z.device)
-    b = torch.empty((n_op,), dtype=z.dtype, device=z.device)
+    a = _workspace((n_op,), z.dtype, z.device)
+    b = _workspace((n_op,), z.dtype, z.device)
     with torch.cuda.device(z.device):
         _call("trimul_project", lib.ptx_trimul_project, _ptr(z), _ptr(mask), _ptr(w["ln_in_w"]), _ptr(w["ln_in_b"]), _ptr(w["w_ap"]),
             _ptr(w["w_ag"]), _ptr(w["w_bp"]), _ptr(w["w_bg"]), _ptr(a), _ptr(b), n, c_z, c_h, pitch,
             int(incoming), eps, dt, st)
-        x = torch.empty((c_h, n, n), dtype=z.dtype, device=z.device)
+        x = _workspace((c_h, n, n), z.dtype, z.device)
         _call("trimul_contract", lib.ptx_trimul_contract, _ptr(a), _ptr(b), _ptr(x), n, c_h, pitch, dt, st)
         del a, b
         if out is None:
@@ -163,11 +174,11 @@ def triangle_attention(z: torch.Tensor, mask: Optional[torch.Tensor], w: dict, h
     # attention-core layouts (see include/protenix_amd.h): q, gate, output head-major; K, V^T
     # and the triangle bias in fragment-ordered key tiles
     n_kv, n_tb = lib.ptx_triattn_kv_elems(n, heads), lib.ptx_triattn_bias_elems(n, heads)
-    q = torch.empty((heads, n, n, d), dtype=z.dtype, device=dev)
-    g = torch.empty((heads, n, n, d), dtype=z.dtype, device=dev)
-    k = torch.empty((n_kv,), dtype=z.dtype, device=dev)
-    vt = torch.empty((n_kv,), dtype=z.dtype, device=dev)
-    tb = torch.empty((n_tb,), dtype=z.dtype, device=dev)
+    q = _workspace((heads, n, n, d), z.dtype, dev)
+    g = _workspace((heads, n, n, d), z.dtype, dev)
+    k = _workspace((n_kv,), z.dtype, dev)
+    vt = _workspace((n_kv,), z.dtype, dev)
+    tb = _workspace((n_tb,), z.dtype, dev)
     with torch.cuda.device(dev):
         _call("triattn_project", lib.ptx_triattn_project, _ptr(z), _ptr(w["ln_w"]),
               _ptr(w["ln_b"]), _ptr(w["w_q"]), _ptr(w["w_k"]), _ptr(w["w_v"]), _ptr(w["w_g"]),

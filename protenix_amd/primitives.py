@@ -109,7 +109,7 @@ class Transition(nn.Module):
     def forward(self, x: torch.Tensor, _residual_out: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Returns the update; with `_residual_out` (may be x itself) writes
         x + update there instead and returns it."""
-        _forward_only(x, *self.parameters())
+        _forward_only(x, module=self)
         add = _residual_out is not None
         fused = self.c_in in (64, 128) or (self.c_in == 256 and x.dtype == torch.bfloat16)
         if fused and (self.n * self.c_in) % 64 == 0:

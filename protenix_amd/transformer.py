@@ -115,6 +115,6 @@ class AttentionPairBias(nn.Module):
     def forward_with_bias(self, a: torch.Tensor, bias: torch.Tensor) -> torch.Tensor:
         """The single-track part, given bias = pair_bias(z).  Split off so that a
         caller can run it on another stream once the pass over z is done."""
-        _forward_only(a, bias, *self.parameters())
+        _forward_only(a, bias, module=self)
         a = self.layernorm_a(a)
         return self.attention(q_x=a, kv_x=a, attn_bias=bias)

@@ -85,7 +85,7 @@ class TriangleMultiplicativeUpdate(nn.Module):
             raise ValueError(
                 "triangle_multiplicative must be 'cuequivariance' or 'torch', but got "
                 f"{triangle_multiplicative}")
-        _forward_only(z, *self.parameters())
+        _forward_only(z, module=self)
         add_inplace = bool(inplace_safe and _add_with_inplace)
         w = self._weights(z.dtype, z.device)
         src = z if z.is_contiguous() else z.contiguous()
@@ -168,7 +168,7 @@ class TriangleAttention(nn.Module):
 
     def _run(self, x: torch.Tensor, mask: Optional[torch.Tensor], transposed: bool,
              residual_inplace: bool) -> torch.Tensor:
-        _forward_only(x, *self.parameters())
+        _forward_only(x, module=self)
         w = self._weights(x.dtype, x.device)
         src = x if x.is_contiguous() else x.contiguous()
         xb, mb = _per_batch(src, mask)

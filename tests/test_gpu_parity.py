@@ -316,3 +316,28 @@ def test_cz256_fp32_is_refused():
     blk = P.TriangleMultiplicationOutgoing(256, 256).cuda()
     with torch.no_grad(), pytest.raises(RuntimeError, match="unsupported"):
         blk(torch.randn(1, 8, 8, 256, device="cuda"))
+
+
+# ------------------------------------------------------------------ workspaces
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("n,n_pad", [(100, 7), (72, 0), (37, 5)])
+def test_results_do_not_depend_on_workspace_contents(dtype, n, n_pad):
+    """The kernels get their workspaces uninitialised; filled with NaN instead, every module
+    must return bit-identical results (tails beyond N are never read into a result, nor into
+    a decision that changes the rounding of one)."""
+    from protenix_amd import ops
+    z = _z(n, dtype).cuda()
+    mask = pad_mask(n, n_pad, dtype).cuda() if n_pad else None
+    mods = [P.TriangleMultiplicationOutgoing(128, 128), P.TriangleMultiplicationIncoming(128, 128),
+            P.TriangleAttention(128, 32, 4, starting=True), P.TriangleAttention(128, 32, 4, starting=False)]
+    for mod in mods:
+        O.seed_parameters_(mod)
+        mod = mod.to("cuda", dtype).eval()
+        with torch.no_grad():
+            want = mod(z, mask)
+            ops.poison_workspaces = True
+            try:
+                got = mod(z, mask)
+            finally:
+                ops.poison_workspaces = False
+        assert torch.equal(got, want), type(mod).__name__
