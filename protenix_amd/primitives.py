@@ -97,6 +97,7 @@ class Transition(nn.Module):
         self.linear_no_bias_b = LinearNoBias(c_in, n * c_in, initializer="relu")
         self.linear_no_bias = LinearNoBias(n * c_in, c_in, initializer="zeros")
         self._cache = _WeightCache()
+        self._cache_ab = _WeightCache()
 
     def _weights(self, dtype, device) -> dict:
         ps = (self.layernorm1.weight, self.layernorm1.bias, self.linear_no_bias_a.weight,
@@ -115,9 +116,17 @@ class Transition(nn.Module):
         if fused and (self.n * self.c_in) % 64 == 0:
             return ops.transition(x, self._weights(x.dtype, x.device), self.n, add_residual=add,
                                   out=_residual_out)
-        # other widths: HIP LayerNorm + library GEMMs
+        # other widths: HIP LayerNorm + library GEMMs (a and b as one GEMM on the stacked weights)
         y = self.layernorm1(x)
-        h = F.silu(self.linear_no_bias_a(y)) * self.linear_no_bias_b(y)
+        if (not torch.is_grad_enabled() and self.linear_no_bias_a.precision is None
+                and self.linear_no_bias_b.precision is None):
+            ps = (self.linear_no_bias_a.weight, self.linear_no_bias_b.weight)
+            w_ab = self._cache_ab.get(ps, y.dtype, y.device, lambda: torch.cat(
+                [_cv(p, y.dtype, y.device) for p in ps], 0).contiguous())
+            a, b = F.linear(y, w_ab).chunk(2, dim=-1)
+            h = F.silu(a) * b
+        else:
+            h = F.silu(self.linear_no_bias_a(y)) * self.linear_no_bias_b(y)
         u = self.linear_no_bias(h)
         if add:
             return _residual_out.copy_(x + u) if _residual_out is not x else x.add_(u)

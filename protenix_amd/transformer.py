@@ -44,13 +44,37 @@ class Attention(nn.Module):
         self.zero_init = zero_init
         if zero_init:
             nn.init.zeros_(self.linear_o.weight)
+        self._cache_in = _WeightCache()
+
+    def _fused_in(self, dtype, device):
+        """q, k, v and gate projections of one input as a single GEMM: the four weights
+        stacked (and the q bias padded with zeros), built once per weight set."""
+        ps = (self.linear_q.weight, self.linear_q.bias, self.linear_k.weight, self.linear_v.weight,
+              self.linear_g.weight)
+
+        def make():
+            wq, bq, wk, wv, wg = (_cv(p, dtype, device) for p in ps)
+            w = torch.cat([wq, wk, wv, wg], 0).contiguous()
+            b = torch.zeros(w.shape[0], dtype=dtype, device=device)
+            if bq is not None:
+                b[: wq.shape[0]] = bq
+            return w, b
+        return self._cache_in.get(ps, dtype, device, make)
 
     def forward(self, q_x: torch.Tensor, kv_x: torch.Tensor,
                 attn_bias: Optional[torch.Tensor] = None, **_unused) -> torch.Tensor:
         H = self.num_heads
-        q = self.linear_q(q_x).unflatten(-1, (H, -1)).transpose(-2, -3)
-        k = self.linear_k(kv_x).unflatten(-1, (H, -1)).transpose(-2, -3)
-        v = self.linear_v(kv_x).unflatten(-1, (H, -1)).transpose(-2, -3)
+        g_lin = None
+        plain = all(l.precision is None for l in (self.linear_q, self.linear_k, self.linear_v))
+        if (q_x is kv_x and self.linear_g is not None and plain and self.linear_g.precision is None
+                and self.c_q == self.c_k == self.c_v and not torch.is_grad_enabled()):
+            w, b = self._fused_in(q_x.dtype, q_x.device)
+            q, k, v, g_lin = torch.nn.functional.linear(q_x, w, b).chunk(4, dim=-1)
+            q, k, v = (t.unflatten(-1, (H, -1)).transpose(-2, -3) for t in (q, k, v))
+        else:
+            q = self.linear_q(q_x).unflatten(-1, (H, -1)).transpose(-2, -3)
+            k = self.linear_k(kv_x).unflatten(-1, (H, -1)).transpose(-2, -3)
+            v = self.linear_v(kv_x).unflatten(-1, (H, -1)).transpose(-2, -3)
         q = q / math.sqrt(self.c_hidden)
         # logits, softmax and the weighted sum in fp32 (the reference upcasts q, k
         # and the bias and relies on autocast for v; here v is upcast as well)
@@ -63,7 +87,9 @@ class Attention(nn.Module):
         w = torch.softmax(w, dim=-1)
         o = torch.matmul(w, v.float()).to(d).transpose(-2, -3)
         if self.linear_g is not None:
-            o = o * torch.sigmoid(self.linear_g(q_x)).unflatten(-1, (H, -1))
+            if g_lin is None:
+                g_lin = self.linear_g(q_x)
+            o = o * torch.sigmoid(g_lin).unflatten(-1, (H, -1))
         return self.linear_o(o.flatten(-2))
 
 
