@@ -108,6 +108,23 @@ __device__ __forceinline__ void load_to_lds16(const void* gptr, uint32_t lds_bas
                : "v"(gptr), "s"(lds_base)
                : "m0");
 }
+// The same with the address split into a wave-uniform 64-bit base (scalar registers), a
+// 32-bit byte offset per lane and an immediate: no vector ALU work per load.  The immediate
+// is added to the LDS address as well as to the global one.
+template <int IMM>
+__device__ __forceinline__ void load_to_lds16_s(uint64_t sbase, uint32_t voff, uint32_t lds_base) {
+  static_assert(IMM >= 0 && IMM < 4096, "13-bit signed immediate offset");
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1 offset:%3"
+               :
+               : "v"(voff), "s"(sbase), "s"(lds_base), "n"(IMM)
+               : "m0");
+}
+// A 64-bit value that is the same in all lanes, moved to scalar registers.
+__device__ __forceinline__ uint64_t uniform64(uint64_t v) {
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
+  const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+  return ((uint64_t)hi << 32) | lo;
+}
 // The 4-byte form, used to pull cache lines into L2 ahead of time: no register receives the
 // data (a register destination would have to stay reserved until the load returns), it
 // lands in a junk LDS area of 256 bytes at lds_base.
