@@ -104,7 +104,7 @@ PTX_API int ptx_trimul_project(const void* z, const void* mask, const void* ln_w
   PTX_REQUIRE(k_pitch == ptx_key_pitch(n), PTX_ERR_BAD_ARG,
               "trimul_project: k_pitch=%d, expected ptx_key_pitch(%d)=%d", k_pitch, n,
               ptx_key_pitch(n));
-  PTX_REQUIRE(n < 32768, PTX_ERR_UNSUPPORTED, "trimul_project: n=%d too large", n);
+  PTX_REQUIRE(n <= 8192, PTX_ERR_UNSUPPORTED, "trimul_project: n=%d too large (8192 at most)", n);
   if (n == 0) return PTX_OK;
   PTX_REQUIRE(z && w_ap && w_ag && w_bp && w_bg && a && b, PTX_ERR_BAD_ARG,
               "trimul_project: null pointer");
@@ -167,7 +167,7 @@ PTX_API int ptx_triattn_project(const void* z, const void* ln_w, const void* ln_
               kWidthMsg, c_in, heads, d);
   PTX_REQUIRE(key_pitch == ptx_key_pitch(n), PTX_ERR_BAD_ARG,
               "triattn_project: key_pitch=%d, expected %d", key_pitch, ptx_key_pitch(n));
-  PTX_REQUIRE(n < 32768, PTX_ERR_UNSUPPORTED, "triattn_project: n=%d too large", n);
+  PTX_REQUIRE(n <= 8192, PTX_ERR_UNSUPPORTED, "triattn_project: n=%d too large (8192 at most)", n);
   if (n == 0) return PTX_OK;
   PTX_REQUIRE(z && w_q && w_k && w_v && w_g && w_b && q && k && vt && g && tri_bias,
               PTX_ERR_BAD_ARG, "triattn_project: null pointer");

@@ -354,6 +354,38 @@ rowgemm_in_kernel(RowGemmInParams p) {
     cm_j[rb] = pc - cm_i[rb] * (uint32_t)p.n;
   }
 
+  // Element offsets of this lane's vectors inside the fragment-ordered destinations, relative
+  // to the head (K, V^T) or channel block (a, b) the chunk writes: the index arithmetic of
+  // the layouts (common.h) runs once per tile here instead of once per store.  32 bits
+  // suffice: a plane has n * pitch * 32 elements and the entry points bound n by 8192.
+  uint32_t rel_k[RB][C::NPASS], rel_v[RB][C::NPASS], rel_b[RB][C::NPASS], rel_a[RB][C::NPASS];
+  if constexpr (MODE == kTriAttnIn) {
+    const int key_tiles = p.pitch >> 6, q_blocks = (p.n + 31) >> 5;
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+      for (int ps = 0; ps < C::NPASS; ++ps) {
+        int mj, m0;
+        stage_coord<T>(ps, lane, mj, m0);   // K: major = key row, minor = d; V^T, bias: major = channel
+        rel_k[rb][ps] = (uint32_t)attn_k_offset(0, rm_i[rb][ps], rm_j[rb][ps], m0, p.n, key_tiles);
+        rel_v[rb][ps] = (uint32_t)attn_v_offset(0, cm_i[rb], cm_j[rb], mj, p.n, key_tiles);
+        rel_b[rb][ps] = (uint32_t)attn_b_offset(mj, cm_i[rb], cm_j[rb], q_blocks, key_tiles);
+      }
+  }
+  if constexpr (MODE == kTriMulIn) {
+    const int n_rb = (p.n + 31) >> 5, n_ks = p.pitch >> 4;
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+      for (int ps = 0; ps < C::NPASS; ++ps) {
+        int chn, r0;
+        stage_coord<T>(ps, lane, chn, r0);
+        const int i = pi0 + 4 * rb + (r0 >> 3);
+        rel_a[rb][ps] = (uint32_t)(trimul_frag_offset(chn, i >> 5, pk0 >> 4, n_rb, n_ks) +
+                                   ((pk0 >> 3) & 1) * 256 + (i & 31) * 8 + (r0 & 7));
+      }
+  }
+
   if constexpr (!RES && !kDma) {
     fetch(0);
     stash(0);
@@ -451,9 +483,9 @@ rowgemm_in_kernel(RowGemmInParams p) {
     // ------------------------------ epilogues ------------------------------
     if constexpr (MODE == kTriMulIn) {
       // a/b[c][i][k] = mask * sigmoid(gate) * proj ; lane <-> channel, register <-> row
-      T* outp = (T*)p.out[ch / (SL / 2)];
       const int c0 = (ch % (SL / 2)) * 32;
       const int n_rb = (p.n + 31) >> 5, n_ks = p.pitch >> 4;
+      T* outp_c0 = (T*)p.out[ch / (SL / 2)] + trimul_frag_offset(c0, 0, 0, n_rb, n_ks);
       constexpr int GT = NST < RB ? NST : RB;   // result tiles per LDS round trip
 #pragma unroll
       for (int rb0 = 0; rb0 < RB; rb0 += GT) {
@@ -483,10 +515,7 @@ rowgemm_in_kernel(RowGemmInParams p) {
           for (int ps = 0; ps < C::NPASS; ++ps) {
             int chn, r0;
             stage_coord<T>(ps, lane, chn, r0);
-            const int i = pi0 + 4 * rb + (r0 >> 3);
-            const int64_t off = trimul_frag_offset(c0 + chn, i >> 5, pk0 >> 4, n_rb, n_ks) +
-                                ((pk0 >> 3) & 1) * 256 + (i & 31) * 8 + (r0 & 7);
-            *reinterpret_cast<VE_t*>(outp + off) = stage_get_vec<T>(stile(q), chn, r0);
+            *reinterpret_cast<VE_t*>(outp_c0 + rel_a[rb][ps]) = stage_get_vec<T>(stile(q), chn, r0);
           }
         }
       }
@@ -496,6 +525,7 @@ rowgemm_in_kernel(RowGemmInParams p) {
       const int which = ch / (SL / 4);
       const int key_tiles = p.pitch >> 6;
       const int q_blocks = (p.n + 31) >> 5;
+      const int64_t head_plane = (int64_t)p.n * key_tiles * kAttnTileElems;   // K, V^T elements per head
       constexpr int GT = NST < 2 * RB ? NST : 2 * RB;   // result tiles per LDS round trip
 #pragma unroll
       for (int k0 = 0; k0 < 2 * RB; k0 += GT) {
@@ -535,15 +565,13 @@ rowgemm_in_kernel(RowGemmInParams p) {
           } else if (which == 1) {
             // K: staged row-major (major = key row, minor = d); each 16-byte d-chunk goes to
             // its fragment slot
-            T* outp = (T*)p.out[1];
+            T* outp = (T*)p.out[1] + h * head_plane;
 #pragma unroll
             for (int ps = 0; ps < C::NPASS; ++ps) {
               int mj, m0;
               stage_coord<T>(ps, lane, mj, m0);
-              *reinterpret_cast<VE_t*>(
-                  rrow[rb][ps] >= 0
-                      ? outp + attn_k_offset(h, rm_i[rb][ps], rm_j[rb][ps], m0, p.n, key_tiles)
-                      : sink) = stage_get_vec<T>(stg, mj, m0);
+              *reinterpret_cast<VE_t*>(rrow[rb][ps] >= 0 ? outp + rel_k[rb][ps] : sink) =
+                  stage_get_vec<T>(stg, mj, m0);
             }
           } else {
             // V^T (which == 3, major = channel d of head h) and the triangle bias (which == 4,
@@ -558,9 +586,7 @@ rowgemm_in_kernel(RowGemmInParams p) {
               const VE_t v = stage_get_vec<T>(stg, chn, r0);
               T* outp = (T*)p.out[which];
               if (vec_ok) {
-                const int64_t off =
-                    which == 3 ? attn_v_offset(h, cm_i[rb], cm_j[rb], chn, p.n, key_tiles)
-                               : attn_b_offset(chn, cm_i[rb], cm_j[rb], q_blocks, key_tiles);
+                const int64_t off = which == 3 ? h * head_plane + rel_v[rb][ps] : (int64_t)rel_b[rb][ps];
                 *reinterpret_cast<VE_t*>(cm_ok[rb] ? outp + off : sink) = v;
               } else {
                 // (the row is made opaque here: the divisions below do not depend on the
