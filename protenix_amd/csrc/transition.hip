@@ -94,16 +94,21 @@ __global__ __launch_bounds__(256) void transition_fused_kernel(
   const int64_t row0 = ((int64_t)blockIdx.x * 4 + wave) * (RB * 32);
 
   // chunk j (clamped for the address) -> buffer j % NBUF; every wave moves FPW fragments
+  // (address = wave-uniform base in scalar registers + this lane's offset inside a fragment:
+  // no vector ALU work per load)
+  const uint32_t lane_off = lane * 8 * (uint32_t)sizeof(T);
   auto dma_chunk = [&](int j) {
     const int jc = min(j, n_chunks - 1);
     const int buf = j % NBUF;
+    const uint64_t base = uniform64(
+        (uint64_t)(packed + ((int64_t)jc * kTrFrags + wave * FPW) * kFragElems));
 #pragma unroll
     for (int q = 0; q < FPW; ++q) {
       const int frag = wave * FPW + q;
+      const uint64_t fb = base + (uint64_t)q * (kFragElems * sizeof(T));
 #pragma unroll
       for (int pc = 0; pc < PIECES; ++pc)
-        load_to_lds16(packed + ((int64_t)jc * kTrFrags + frag) * kFragElems + lane * 8 + pc * C::VE,
-                      lds_address(&lds_w[buf][frag][pc][0]));
+        load_to_lds16_s<0>(fb, lane_off + 16 * pc, lds_address(&lds_w[buf][frag][pc][0]));
     }
   };
   auto read_frag = [&](int buf, int frag) {
