@@ -341,3 +341,17 @@ def test_results_do_not_depend_on_workspace_contents(dtype, n, n_pad):
             finally:
                 ops.poison_workspaces = False
         assert torch.equal(got, want), type(mod).__name__
+
+
+# ------------------------------------------------------------------ smallest and odd sizes
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("n,n_pad", [(1, 0), (2, 1), (5, 0), (17, 1), (33, 0), (65, 1), (127, 0), (129, 1)])
+def test_block_edge_sizes(dtype, n, n_pad):
+    """One block at sizes around the 32-row / 64-key tile edges, down to a single token."""
+    ref, prod = oracle_and_product(O.PairformerBlock, P.PairformerBlock, dtype=dtype)
+    s, z, pm = O.make_inputs(n, n_pad=n_pad, seed=9 + n, dtype=dtype)
+    pm = pm if n_pad else None
+    with torch.no_grad():
+        s_ref, z_ref = ref(s.float(), z.float(), None if pm is None else pm.float())
+        s_got, z_got = prod(s.cuda(), z.cuda(), None if pm is None else pm.cuda())
+    assert rel_err(z_got, z_ref) <= tol(dtype) and rel_err(s_got, s_ref) <= tol(dtype)
