@@ -38,7 +38,7 @@ __global__ __launch_bounds__(256) void layernorm_fwd_kernel(
   typedef typename VecN<T, VEC>::ftype F;
   constexpr int ROWS_PER_WAVE = (kWave / G) * UNROLL;
   const int lane = threadIdx.x & (kWave - 1);
-  const int wave = threadIdx.x >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int sub = lane % G;   // lane within the row group
   const int grp = lane / G;   // which row of the wave's batch
   const int64_t row0 = ((int64_t)blockIdx.x * (blockDim.x >> 6) + wave) * ROWS_PER_WAVE;

@@ -68,7 +68,7 @@ __global__ __launch_bounds__(256) void nt_gemm_batched_kernel(const T* __restric
   constexpr int KK = G::KK, BK = G::BK, NBUF = G::NBUF, PIECES = G::PIECES, RUNS = G::RUNS;
   // [buffer][operand*8*KK + row block*KK + kk][16-byte piece][lane]
   __shared__ u32x4_t lds_f[NBUF][G::NF][PIECES][kWave];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int ln = lane & 31, g = lane >> 5;
   const int wi = wave >> 1, wj = wave & 1;
 

@@ -149,7 +149,7 @@ rowgemm_in_kernel(RowGemmInParams p) {
   __shared__ __attribute__((aligned(16))) T lds_res[MODE == kTriMulOut ? NW : 1][MODE == kTriMulOut ? RB * 32 : 1][kResPitch];
   __shared__ __attribute__((aligned(16))) T lds_stage[NW][NST][32 * C::PITCH];
   __shared__ __attribute__((aligned(16))) float lds_mask[MODE == kTriMulIn ? NW : 1][RB * 32];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int n = lane & 31, g = lane >> 5;
   T* st = lds_stage[wave][0];
   auto stile = [&](int k) { return lds_stage[wave][k]; };
@@ -722,7 +722,7 @@ __global__ __launch_bounds__(256, 2) void rowgemm_out_kernel(RowGemmOutParams p)
   typedef Cfg<T> C;
   __shared__ V8 lds_w[C::NBUF][2 * kKSteps][kWave];
   __shared__ __attribute__((aligned(16))) T lds_stage[4][32 * C::PITCH];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int64_t row0 = ((int64_t)blockIdx.x * 4 + wave) * (RB * 32);
   const int K = kC * p.n_slab;
   const T* w = (const T*)p.w;

@@ -90,7 +90,7 @@ __global__ __launch_bounds__(256) void transition_fused_kernel(
   static_assert(sizeof(T) * 4 * 32 * C::PITCH <= sizeof(u32x4_t) * kTrFrags * PIECES * kWave,
                 "the staging tiles reuse chunk buffer 0");
 
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int64_t row0 = ((int64_t)blockIdx.x * 4 + wave) * (RB * 32);
 
   // chunk j (clamped for the address) -> buffer j % NBUF; every wave moves FPW fragments

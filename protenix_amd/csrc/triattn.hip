@@ -63,7 +63,7 @@ __global__ __launch_bounds__(256, 2) void triattn_fwd_kernel(
   __shared__ V8 lds_kv[3][R][8][kWave];     // fragments 0-3: K (u,kk); 4-7: V^T (u,s)
   __shared__ __attribute__((aligned(16))) float lds_mb[3][R][kKeyTile];  // mask bias per key
 
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int ln = lane & 31, g = lane >> 5;
 
   // Work item -> (h, row group, query tile), h-major, one contiguous span per XCD
