@@ -185,7 +185,11 @@ rowgemm_in_kernel(RowGemmInParams p) {
     load_to_lds16(w + (int64_t)col * ldw + kk * 16 + 8 * (lane >> 5),
                   lds_address(&lds_w[f_dst][0]));
   };
-  constexpr bool kDma = sizeof(T) == 2 && MODE == kPairBias;   // bf16 pair bias: its single chunk
+  // bf16 without resident weights (the pair bias' single chunk; rows of 256 channels): a ring
+  // of two chunk buffers filled by the same direct-to-LDS loads, one chunk ahead.  The wait
+  // for a chunk counts the stores issued after its loads (see the end of the chunk loop): a
+  // register-staged prefetch would make the compiler drain every store before each chunk.
+  constexpr bool kDma = sizeof(T) == 2 && !RES;
   if constexpr (RES) {
     for (int f = wave; f < IC::NFRAG; f += NW) dma_frag(f, f);
     ring_barrier<0>();
@@ -409,7 +413,16 @@ rowgemm_in_kernel(RowGemmInParams p) {
 #pragma clang loop unroll(disable)
   for (int ch = 0; ch < nch; ++ch) {
     const int buf = (!RES && C::NBUF == 2) ? (ch & 1) : 0;
-    if constexpr (!RES && !kDma) fetch(min(ch + 1, nch - 1));   // unconditional: static load count
+    if constexpr (kDma) {
+      // the other buffer was last read in the previous chunk, which every wave has left
+      if (ch + 1 < nch) {
+#pragma unroll
+        for (int j = 0; j < FPW; ++j)
+          dma_frag((ch + 1) * 2 * SL + wave * FPW + j, (buf ^ 1) * 2 * SL + wave * FPW + j);
+      }
+    } else if constexpr (!RES) {
+      fetch(min(ch + 1, nch - 1));   // unconditional: static load count
+    }
     // first fragment of this chunk's two weight tiles (the resident triangle bias is one tile)
     const int wf0 = RES ? ch * 2 * SL : buf * 2 * SL;
     const int wf1 = wf0 + ((RES && MODE == kTriAttnIn && ch == nch - 1) ? 0 : SL);
@@ -658,7 +671,17 @@ rowgemm_in_kernel(RowGemmInParams p) {
       }
     }
 
-    if constexpr (!RES && !kDma) {
+    if constexpr (kDma) {
+      // The next chunk's weights must have landed: all but the stores this wave issued after
+      // requesting them (a lower bound on that count is what is safe; the triangle bias,
+      // whose store count varies, is the last chunk and has no successor).
+      constexpr int kStores = MODE == kTriMulIn    ? RB * C::NPASS
+                              : MODE == kTriAttnIn ? RB * 2 * C::NPASS
+                              : MODE == kTriMulOut ? RB * C::NPASS
+                                                   : 0;
+      if (MODE != kTriAttnIn || vec_ok) ring_barrier<kStores>();
+      else ring_barrier<0>();   // element-wise V^T stores: no fixed count
+    } else if constexpr (!RES) {
       if (C::NBUF == 1) {
         __syncthreads();      // everyone is done reading the single buffer
         stash(0);
