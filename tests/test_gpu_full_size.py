@@ -181,3 +181,28 @@ def test_block_under_autocast_keeps_fp32_residual_stream():
     assert torch.equal(zc.cpu(), z) and torch.equal(sc.cpu(), s)
     assert rel_err(got_z, want_z) <= TOL_BF16
     assert rel_err(got_s, want_s) <= TOL_BF16
+
+
+@pytest.mark.parametrize("kw,n", [(dict(), 768), (dict(c_z=256, hidden_scale_up=True), 320),
+                                  (dict(c_z=64, c_s=0, num_intermediate_factor=2), 520)])
+def test_block_is_deterministic(kw, n):
+    """No kernel uses atomics or depends on scheduling: repeated runs on the same input are
+    bit-identical (a miscounted wait in one of the hand-synchronised load rings would show up
+    here as a sporadic difference)."""
+    blk = P.PairformerBlock(**kw)
+    O.seed_parameters_(blk)
+    blk = blk.to("cuda", BF16).eval()
+    c_z = kw.get("c_z", 128)
+    g = torch.Generator().manual_seed(11)
+    z = torch.randn(1, n, n, c_z, generator=g).to(BF16).cuda()
+    s = torch.randn(1, n, 384, generator=g).to(BF16).cuda() if kw.get("c_s", 384) else None
+    mask = pad_mask(n, 24, BF16).cuda()
+    outs = []
+    with torch.no_grad():
+        for _ in range(6):
+            s_o, z_o = blk(s, z, mask)
+            outs.append((s_o, z_o))
+    torch.cuda.synchronize()
+    for s_o, z_o in outs[1:]:
+        assert torch.equal(z_o, outs[0][1])
+        assert s_o is None or torch.equal(s_o, outs[0][0])
