@@ -91,6 +91,24 @@ PTX_API int ptx_layernorm_fwd(const void* x, const void* gamma, const void* beta
                       int dtype, void* stream);
 
 /*
+ * LayerNorm backward.  Replaces fast_layer_norm_cuda_v2.backward_{none,with_bias,with_weight,
+ * with_both}_affine (layer_norm_cuda.cpp:159-178; kernels layer_norm_cuda_kernel.cu:395-760,
+ * host :860-990), fp32 arithmetic, with xc = x - mean and gd = gamma * dout:
+ *   dx     = gd * rstd - sum_c(gd) * rstd / cols - xc * sum_c(gd * xc) * rstd^3 / cols
+ *   dgamma = sum_rows dout * xc * rstd          dbeta = sum_rows dout
+ *   dout, x, dx [rows][cols] in `dtype` (dx aliases neither);  mean, rstd fp32 [rows] as
+ *   written by ptx_layernorm_fwd;  gamma [cols] in `dtype` or NULL (= 1);
+ *   dgamma, dbeta [cols] in `dtype`, each may be NULL (not wanted);
+ *   workspace: ptx_layernorm_bwd_workspace_elems(rows, cols) fp32 elements of partial sums,
+ *   needed unless dgamma and dbeta are both NULL.  The sums run in a fixed order: results are
+ *   reproducible bit for bit.  beta does not enter the gradients and is not an argument.
+ */
+PTX_API int64_t ptx_layernorm_bwd_workspace_elems(int64_t rows, int cols);
+PTX_API int ptx_layernorm_bwd(const void* dout, const void* x, const float* mean, const float* rstd,
+                      const void* gamma, void* dx, void* dgamma, void* dbeta, float* workspace,
+                      int64_t rows, int cols, int dtype, void* stream);
+
+/*
  * Triangle multiplication, stage 1 (triangular.py:537-543):
  *   zn = LN(z);  a = mask * sigmoid(W_ag zn) * (W_ap zn);  b likewise,
  * written channel-major so that stage 2 is a plain batched matrix product:

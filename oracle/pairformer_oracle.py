@@ -10,6 +10,8 @@ What pins each function (see tests/test_oracle_*.py):
 
 * ``layer_norm``            -> ``torch.nn.LayerNorm`` + closed forms
                                (constant row -> beta, unit variance rows)
+* ``layer_norm_backward``   -> autograd of ``F.layer_norm`` in fp64, central
+                               differences, dx orthogonal to 1 and to x - mean
 * ``linear``                -> ``torch.nn.functional.linear``
 * triangle multiplication   -> ``torch.einsum`` + a triple-loop brute force on
                                tiny N, token-permutation equivariance,
@@ -60,6 +62,38 @@ def layer_norm(
     w = weight.to(d) if weight is not None else None
     b = bias.to(d) if bias is not None else None
     return F.layer_norm(x, (x.shape[-1],), w, b, eps)
+
+
+def layer_norm_backward(
+    dout: torch.Tensor,
+    x: torch.Tensor,
+    weight: Optional[torch.Tensor],
+    eps: float = 1e-5,
+) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """(dx, dgamma, dbeta) of layer_norm for upstream gradient dout, in the dtype of x.
+
+    Follows the arithmetic of protenix/model/layer_norm/kernel/layer_norm_cuda_kernel.cu:672-716
+    (grad_input = part1 - part2 - part3 in fp32) and :395-470 (parameter gradients: column
+    sums of dout * (x - mean) * invvar and of dout); gamma cast to the gradient's dtype as
+    layer_norm.py:114-176 does.  Arithmetic in fp32 (fp64 for fp64 inputs).
+    """
+    d = x.dtype
+    f = torch.float64 if d == torch.float64 else torch.float32
+    cols = x.shape[-1]
+    xf, df = x.to(f), dout.to(d).to(f)
+    g = weight.to(d).to(f) if weight is not None else torch.ones(cols, dtype=f)
+    mean = xf.mean(-1, keepdim=True)
+    invvar = torch.rsqrt(((xf - mean) ** 2).mean(-1, keepdim=True) + eps)
+    xc = xf - mean
+    gd = g * df
+    part1 = gd * invvar
+    part2 = gd.sum(-1, keepdim=True) * invvar / cols
+    part3 = xc * ((gd * xc).sum(-1, keepdim=True) * invvar * invvar * invvar / cols)
+    dx = part1 - part2 - part3
+    red = tuple(range(x.dim() - 1))
+    dgamma = (df * xc * invvar).sum(red) if red else df * xc * invvar
+    dbeta = df.sum(red) if red else df
+    return dx.to(d), dgamma.to(d), dbeta.to(d)
 
 
 def linear(

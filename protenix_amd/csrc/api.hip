@@ -84,6 +84,29 @@ PTX_API int ptx_layernorm_fwd(const void* x, const void* gamma, const void* beta
   return after_launch("layernorm");
 }
 
+PTX_API int64_t ptx_layernorm_bwd_workspace_elems(int64_t rows, int cols) {
+  return ptx::layernorm_bwd_workspace_elems(rows, cols);
+}
+
+PTX_API int ptx_layernorm_bwd(const void* dout, const void* x, const float* mean, const float* rstd,
+                      const void* gamma, void* dx, void* dgamma, void* dbeta, float* workspace,
+                      int64_t rows, int cols, int dtype, void* stream) {
+  PTX_REQUIRE(dtype_ok(dtype), PTX_ERR_BAD_ARG, "layernorm_bwd: unknown dtype %d", dtype);
+  PTX_REQUIRE(rows >= 0 && cols > 0, PTX_ERR_BAD_ARG, "layernorm_bwd: rows=%lld cols=%d",
+              (long long)rows, cols);
+  PTX_REQUIRE(rows < ((int64_t)1 << 31), PTX_ERR_UNSUPPORTED,
+              "layernorm_bwd: rows=%lld too large", (long long)rows);
+  PTX_REQUIRE(!(dgamma || dbeta) || workspace, PTX_ERR_BAD_ARG,
+              "layernorm_bwd: dgamma / dbeta need the workspace");
+  if (rows == 0 && !dgamma && !dbeta) return PTX_OK;
+  if (rows > 0)
+    PTX_REQUIRE(dout && x && mean && rstd && dx, PTX_ERR_BAD_ARG, "layernorm_bwd: null pointer");
+  PTX_DISPATCH(dtype, ptx::layernorm_bwd<T>((const T*)dout, (const T*)x, mean, rstd,
+                                            (const T*)gamma, (T*)dx, (T*)dgamma, (T*)dbeta,
+                                            workspace, rows, cols, (hipStream_t)stream));
+  return after_launch("layernorm_bwd");
+}
+
 // Pair-row widths the kernels are built for: c_z = 64 or 128 with hidden widths (c_hidden,
 // heads * 32) of 128, or c_z = 256 in bf16 with hidden widths of 256.
 static bool pair_width_ok(int c_z, int hidden, int dtype) {

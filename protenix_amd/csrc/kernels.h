@@ -10,6 +10,13 @@ namespace ptx {
 template <typename T>
 int layernorm_fwd(const T* x, const T* gamma, const T* beta, T* y, float* mean, float* rstd,
                   int64_t rows, int cols, float eps, hipStream_t stream);
+// LayerNorm backward: dx always; dgamma / dbeta when non-null, through `workspace`
+// (layernorm_bwd_workspace_elems fp32 elements).
+int64_t layernorm_bwd_workspace_elems(int64_t rows, int cols);
+template <typename T>
+int layernorm_bwd(const T* dout, const T* x, const float* mean, const float* rstd, const T* gamma,
+                  T* dx, T* dgamma, T* dbeta, float* workspace, int64_t rows, int cols,
+                  hipStream_t stream);
 
 template <typename T>
 int trimul_project(const void* z, const void* mask, const void* ln_w, const void* ln_b,

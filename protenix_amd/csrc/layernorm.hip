@@ -1,4 +1,6 @@
-// LayerNorm forward over the last dimension, HBM-bound.
+// LayerNorm over the last dimension, forward and backward, HBM-bound.
+//
+// Forward:
 //
 // A group of G lanes (G a power of two, 1..64) owns one row: each lane keeps
 // NCHUNK vectors of VEC elements in registers (16-byte loads where alignment
@@ -7,7 +9,10 @@
 // group with xor-shuffles.  A wave issues the loads of UNROLL independent rows
 // per group before touching any of them, to keep enough bytes in flight.
 // Algorithmic traffic: 2 * rows * cols * sizeof(T) bytes.
+#include <algorithm>
+
 #include "common.h"
+#include "kernels.h"
 
 namespace ptx {
 
@@ -199,5 +204,285 @@ template int layernorm_fwd<float>(const float*, const float*, const float*, floa
                                   int64_t, int, float, hipStream_t);
 template int layernorm_fwd<bf16_t>(const bf16_t*, const bf16_t*, const bf16_t*, bf16_t*, float*,
                                    float*, int64_t, int, float, hipStream_t);
+
+// ---------------------------------------------------------------------------
+// Backward.  With xc = x - mean, gd = gamma * dout (gamma = 1 when absent), all in fp32:
+//   dx     = gd * rstd - sum_c(gd) * rstd / cols - xc * sum_c(gd * xc) * rstd^3 / cols
+//   dgamma = sum_rows dout * xc * rstd,   dbeta = sum_rows dout
+// One pass over x and dout serves all three: the rows are laid out over the lanes as in the
+// forward kernel, a wave walks over row batches with a grid stride and keeps its column sums
+// of dgamma / dbeta in registers; at the end every workgroup writes one row of partial sums
+// ([2][parts][cols] fp32, parts = gridDim.x) and a second small kernel adds them up in a
+// fixed order (no atomics: the result does not depend on scheduling).
+// Algorithmic traffic: 3 * rows * cols * sizeof(T) bytes.
+// ---------------------------------------------------------------------------
+constexpr int kLnBwdMaxBlocks = 1024;   // = most rows of partial sums
+
+template <typename T, int VEC, int G, int NCHUNK>
+__global__ __launch_bounds__(256) void layernorm_bwd_kernel(
+    const T* __restrict__ dout, const T* __restrict__ x, const float* __restrict__ mean,
+    const float* __restrict__ rstd, const T* __restrict__ gamma, T* __restrict__ dx,
+    float* __restrict__ part, int64_t rows, int cols) {
+  typedef typename VecN<T, VEC>::type V;
+  typedef typename VecN<T, VEC>::ftype F;
+  constexpr int RPW = kWave / G;   // rows per wave and batch
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int sub = lane % G, grp = lane / G;
+  const float inv_n = 1.0f / (float)cols;
+  const int64_t n_batches = (rows + RPW - 1) / RPW;
+
+  F gm[NCHUNK], dg[NCHUNK], db[NCHUNK];
+#pragma unroll
+  for (int c = 0; c < NCHUNK; ++c) {
+    const int col = (c * G + sub) * VEC;
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+      gm[c][e] = 1.0f;
+      dg[c][e] = 0.0f;
+      db[c][e] = 0.0f;
+    }
+    if (gamma && col < cols) gm[c] = __builtin_convertvector(*reinterpret_cast<const V*>(gamma + col), F);
+  }
+
+  for (int64_t batch = (int64_t)blockIdx.x * 4 + wave; batch < n_batches; batch += (int64_t)gridDim.x * 4) {
+    const int64_t row = batch * RPW + grp;
+    const bool ok = row < rows;
+    const float mu = ok ? mean[row] : 0.0f;
+    const float rs = ok ? rstd[row] : 0.0f;
+    F xc[NCHUNK], dv[NCHUNK];
+#pragma unroll
+    for (int c = 0; c < NCHUNK; ++c) {
+      const int col = (c * G + sub) * VEC;
+      if (ok && col < cols) {
+        xc[c] = __builtin_convertvector(*reinterpret_cast<const V*>(x + row * cols + col), F);
+        dv[c] = __builtin_convertvector(*reinterpret_cast<const V*>(dout + row * cols + col), F);
+      } else {
+        // dout = 0 keeps the padding out of every sum below
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+          xc[c][e] = 0.0f;
+          dv[c][e] = 0.0f;
+        }
+      }
+    }
+    float s1 = 0.0f, s2 = 0.0f;
+#pragma unroll
+    for (int c = 0; c < NCHUNK; ++c)
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) {
+        xc[c][e] -= mu;
+        const float gd = gm[c][e] * dv[c][e];
+        s1 += gd;
+        s2 += gd * xc[c][e];
+      }
+    const float p2 = group_sum<G>(s1) * rs * inv_n;
+    const float p3 = group_sum<G>(s2) * rs * rs * rs * inv_n;
+#pragma unroll
+    for (int c = 0; c < NCHUNK; ++c) {
+      const int col = (c * G + sub) * VEC;
+      F o;
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) {
+        o[e] = gm[c][e] * dv[c][e] * rs - p2 - xc[c][e] * p3;
+        dg[c][e] += dv[c][e] * xc[c][e] * rs;
+        db[c][e] += dv[c][e];
+      }
+      if (ok && col < cols) *reinterpret_cast<V*>(dx + row * cols + col) = __builtin_convertvector(o, V);
+    }
+  }
+
+  if (part) {
+    // wave: lanes that share `sub` hold the same columns of different rows; workgroup: the
+    // four waves through LDS, added in wave order
+    constexpr int WIDTH = G * NCHUNK * VEC;
+    __shared__ float red[2][4][WIDTH];
+#pragma unroll
+    for (int c = 0; c < NCHUNK; ++c) {
+      const int col = (c * G + sub) * VEC;
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) {
+        float a = dg[c][e], b = db[c][e];
+#pragma unroll
+        for (int m = G; m < kWave; m <<= 1) {
+          a += __shfl_xor(a, m, 64);
+          b += __shfl_xor(b, m, 64);
+        }
+        if (grp == 0) {
+          red[0][wave][col + e] = a;
+          red[1][wave][col + e] = b;
+        }
+      }
+    }
+    __syncthreads();
+    const int64_t parts = gridDim.x;
+    for (int col = threadIdx.x; col < cols; col += 256) {
+      part[(int64_t)blockIdx.x * cols + col] =
+          (red[0][0][col] + red[0][1][col]) + (red[0][2][col] + red[0][3][col]);
+      part[(parts + blockIdx.x) * cols + col] =
+          (red[1][0][col] + red[1][1][col]) + (red[1][2][col] + red[1][3][col]);
+    }
+  }
+}
+
+// Rows too long for the register layout: dx with one wave per row (the row is re-read from
+// cache), dgamma / dbeta partial sums with one thread per column over a slice of the rows.
+template <typename T>
+__global__ __launch_bounds__(256) void layernorm_bwd_long_kernel(
+    const T* __restrict__ dout, const T* __restrict__ x, const float* __restrict__ mean,
+    const float* __restrict__ rstd, const T* __restrict__ gamma, T* __restrict__ dx, int64_t rows,
+    int cols) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t row = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const T* xr = x + row * cols;
+  const T* dr = dout + row * cols;
+  const float mu = mean[row], rs = rstd[row];
+  float s1 = 0.0f, s2 = 0.0f;
+  for (int c = lane; c < cols; c += kWave) {
+    const float gd = (gamma ? to_f32(gamma[c]) : 1.0f) * to_f32(dr[c]);
+    s1 += gd;
+    s2 += gd * (to_f32(xr[c]) - mu);
+  }
+  const float p2 = group_sum<64>(s1) * rs / (float)cols;
+  const float p3 = group_sum<64>(s2) * rs * rs * rs / (float)cols;
+  for (int c = lane; c < cols; c += kWave) {
+    const float gd = (gamma ? to_f32(gamma[c]) : 1.0f) * to_f32(dr[c]);
+    dx[row * cols + c] = from_f32<T>(gd * rs - p2 - (to_f32(xr[c]) - mu) * p3);
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void layernorm_bwd_params_kernel(
+    const T* __restrict__ dout, const T* __restrict__ x, const float* __restrict__ mean,
+    const float* __restrict__ rstd, float* __restrict__ part, int64_t rows, int cols) {
+  // grid: (column blocks of 256, parts); part p owns rows p, p + parts, ...
+  const int col = blockIdx.x * 256 + threadIdx.x;
+  const int64_t parts = gridDim.y, p = blockIdx.y;
+  if (col >= cols) return;
+  float a = 0.0f, b = 0.0f;
+  for (int64_t row = p; row < rows; row += parts) {
+    const float d = to_f32(dout[row * cols + col]);
+    a += d * (to_f32(x[row * cols + col]) - mean[row]) * rstd[row];
+    b += d;
+  }
+  part[p * cols + col] = a;
+  part[(parts + p) * cols + col] = b;
+}
+
+// Column sums of the partial rows: 64 columns per workgroup, the parts dealt to 16 waves.
+template <typename T>
+__global__ __launch_bounds__(1024) void layernorm_bwd_reduce_kernel(
+    const float* __restrict__ part, int parts, int cols, T* __restrict__ dgamma,
+    T* __restrict__ dbeta) {
+  constexpr int SL = 16;
+  __shared__ float red[2][SL][kWave];
+  const int cl = threadIdx.x & (kWave - 1), sl = threadIdx.x >> 6;
+  const int col = blockIdx.x * kWave + cl;
+  float a[2] = {0.0f, 0.0f}, b[2] = {0.0f, 0.0f};
+  if (col < cols) {
+    int p = sl;
+    for (; p + SL < parts; p += 2 * SL) {   // two independent chains per sum
+      a[0] += part[(int64_t)p * cols + col];
+      a[1] += part[(int64_t)(p + SL) * cols + col];
+      b[0] += part[((int64_t)parts + p) * cols + col];
+      b[1] += part[((int64_t)parts + p + SL) * cols + col];
+    }
+    if (p < parts) {
+      a[0] += part[(int64_t)p * cols + col];
+      b[0] += part[((int64_t)parts + p) * cols + col];
+    }
+  }
+  red[0][sl][cl] = a[0] + a[1];
+  red[1][sl][cl] = b[0] + b[1];
+  __syncthreads();
+  if (sl == 0 && col < cols) {
+    float sa = 0.0f, sb = 0.0f;
+#pragma unroll
+    for (int w = 0; w < SL; ++w) {
+      sa += red[0][w][cl];
+      sb += red[1][w][cl];
+    }
+    if (dgamma) dgamma[col] = from_f32<T>(sa);
+    if (dbeta) dbeta[col] = from_f32<T>(sb);
+  }
+}
+
+template <typename T, int VEC>
+static int dispatch_ln_bwd_vec(const T* dout, const T* x, const float* mean, const float* rstd,
+                               const T* gamma, T* dx, float* part, int64_t rows, int cols,
+                               hipStream_t stream) {
+  const int nvec = cols / VEC;
+  // returns the number of partial-sum rows written (0: no kernel fits)
+#define PTX_LNB_CASE(G, NC)                                                                    \
+  if (nvec <= (G) * (NC)) {                                                                    \
+    const int64_t batches = (rows + (kWave / (G)) - 1) / (kWave / (G));                        \
+    const int blocks = (int)std::min<int64_t>((batches + 3) / 4, kLnBwdMaxBlocks);             \
+    layernorm_bwd_kernel<T, VEC, G, NC><<<dim3(blocks), dim3(256), 0, stream>>>(               \
+        dout, x, mean, rstd, gamma, dx, part, rows, cols);                                     \
+    return blocks;                                                                             \
+  }
+  PTX_LNB_CASE(1, 1) PTX_LNB_CASE(2, 1) PTX_LNB_CASE(4, 1) PTX_LNB_CASE(8, 1) PTX_LNB_CASE(16, 1)
+  PTX_LNB_CASE(16, 2) PTX_LNB_CASE(16, 3) PTX_LNB_CASE(64, 1) PTX_LNB_CASE(64, 2) PTX_LNB_CASE(64, 4)
+  if constexpr (VEC <= 4) {
+    PTX_LNB_CASE(64, 8)
+  }
+#undef PTX_LNB_CASE
+  return 0;
+}
+
+int64_t layernorm_bwd_workspace_elems(int64_t rows, int cols) {
+  if (rows <= 0 || cols <= 0) return 0;
+  return 2 * (int64_t)kLnBwdMaxBlocks * cols;
+}
+
+template <typename T>
+int layernorm_bwd(const T* dout, const T* x, const float* mean, const float* rstd, const T* gamma,
+                  T* dx, T* dgamma, T* dbeta, float* workspace, int64_t rows, int cols,
+                  hipStream_t stream) {
+  const bool params = dgamma || dbeta;
+  if (rows == 0) {
+    // empty input: the parameter gradients are sums over no rows (written by a kernel, so
+    // that the call can be captured into a HIP graph like every other one)
+    if (params)
+      layernorm_bwd_reduce_kernel<T><<<dim3((cols + kWave - 1) / kWave), dim3(1024), 0, stream>>>(
+          nullptr, 0, cols, dgamma, dbeta);
+    return 0;
+  }
+  float* part = params ? workspace : nullptr;
+  auto aligned = [&](int vec) {
+    const uintptr_t bytes = (uintptr_t)vec * sizeof(T);
+    return cols % vec == 0 && ((uintptr_t)x % bytes) == 0 && ((uintptr_t)dout % bytes) == 0 &&
+           ((uintptr_t)dx % bytes) == 0 && (!gamma || ((uintptr_t)gamma % bytes) == 0);
+  };
+  int parts = 0;
+  if constexpr (sizeof(T) == 2) {
+    if (aligned(8)) parts = dispatch_ln_bwd_vec<T, 8>(dout, x, mean, rstd, gamma, dx, part, rows, cols, stream);
+  }
+  if (!parts && aligned(4)) parts = dispatch_ln_bwd_vec<T, 4>(dout, x, mean, rstd, gamma, dx, part, rows, cols, stream);
+  if (!parts && aligned(2)) parts = dispatch_ln_bwd_vec<T, 2>(dout, x, mean, rstd, gamma, dx, part, rows, cols, stream);
+  if (!parts) parts = dispatch_ln_bwd_vec<T, 1>(dout, x, mean, rstd, gamma, dx, part, rows, cols, stream);
+  if (!parts) {
+    const int64_t blocks = (rows + 3) / 4;
+    layernorm_bwd_long_kernel<T><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(
+        dout, x, mean, rstd, gamma, dx, rows, cols);
+    if (params) {
+      parts = (int)std::min<int64_t>(rows, 256);
+      layernorm_bwd_params_kernel<T><<<dim3((cols + 255) / 256, parts), dim3(256), 0, stream>>>(
+          dout, x, mean, rstd, part, rows, cols);
+    }
+  }
+  if (params)
+    layernorm_bwd_reduce_kernel<T><<<dim3((cols + kWave - 1) / kWave), dim3(1024), 0, stream>>>(
+        part, parts, cols, dgamma, dbeta);
+  return 0;
+}
+
+template int layernorm_bwd<float>(const float*, const float*, const float*, const float*,
+                                  const float*, float*, float*, float*, float*, int64_t, int,
+                                  hipStream_t);
+template int layernorm_bwd<bf16_t>(const bf16_t*, const bf16_t*, const float*, const float*,
+                                   const bf16_t*, bf16_t*, bf16_t*, bf16_t*, float*, int64_t, int,
+                                   hipStream_t);
 
 }  // namespace ptx

@@ -3,7 +3,8 @@
 Mirrors protenix/model/layer_norm/layer_norm.py:190-233 (FusedLayerNorm) and
 the factory protenix/model/triangular/layers.py:246-256: parameters `weight`
 and `bias` (either may be absent), fp32 statistics, gamma/beta cast to the
-input dtype, output in the input dtype.  Forward only.
+input dtype, output in the input dtype.  Forward and backward
+(FusedLayerNormAffineFunction, layer_norm.py:69-187) both run on HIP kernels.
 """
 from __future__ import annotations
 
@@ -27,6 +28,29 @@ def _forward_only(*tensors: Optional[torch.Tensor], module: Optional[nn.Module] 
         raise RuntimeError(
             "protenix_amd kernels are forward-only: call under torch.no_grad() "
             "(backward kernels are not part of this build)")
+
+
+class FusedLayerNormAffineFunction(torch.autograd.Function):
+    """layer_norm.py:69-187: forward keeps the fp32 row statistics for the backward kernel;
+    weight / bias may be None."""
+
+    @staticmethod
+    def forward(ctx, input, weight, bias, normalized_shape, eps):  # noqa: A002
+        ctx.normalized_shape = normalized_shape
+        ctx.eps = eps
+        input_ = input.contiguous()
+        output, mean, invvar = ops.layer_norm(input_, weight, bias, eps, return_stats=True)
+        ctx.save_for_backward(input_, weight, bias, mean, invvar)
+        return output
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        input_, weight_, bias_, mean, invvar = ctx.saved_tensors
+        need = ctx.needs_input_grad
+        grad_input, grad_weight, grad_bias = ops.layer_norm_backward(
+            grad_output, input_, mean, invvar, weight_,
+            need_weight=weight_ is not None and need[1], need_bias=bias_ is not None and need[2])
+        return grad_input if need[0] else None, grad_weight, grad_bias, None, None
 
 
 class FusedLayerNorm(nn.Module):
@@ -58,7 +82,10 @@ class FusedLayerNorm(nn.Module):
         if input.shape[-1] != self.normalized_shape[0]:
             raise RuntimeError(
                 f"expected last dimension {self.normalized_shape[0]}, got {tuple(input.shape)}")
-        _forward_only(input, self.weight, self.bias)
+        if torch.is_grad_enabled() and any(
+                t is not None and t.requires_grad for t in (input, self.weight, self.bias)):
+            return FusedLayerNormAffineFunction.apply(input, self.weight, self.bias,
+                                                      self.normalized_shape, self.eps)
         return ops.layer_norm(input, self.weight, self.bias, self.eps)
 
     def extra_repr(self) -> str:

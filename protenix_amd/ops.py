@@ -109,6 +109,31 @@ def layer_norm(x: torch.Tensor, weight: Optional[torch.Tensor], bias: Optional[t
     return (y, mean, rstd) if return_stats else y
 
 
+def layer_norm_backward(dout: torch.Tensor, x: torch.Tensor, mean: torch.Tensor, rstd: torch.Tensor,
+                        weight: Optional[torch.Tensor], need_weight: bool, need_bias: bool):
+    """Gradients of layer_norm (reference: layer_norm.py:114-187): dx in x's dtype and, when
+    asked for, dweight / dbias [cols] in x's dtype; mean, rstd as returned by
+    layer_norm(..., return_stats=True)."""
+    _dev(x, "input")
+    lib = _lib.load()
+    x = x.contiguous()
+    dout = dout.to(dtype=x.dtype).contiguous()
+    cols = x.shape[-1]
+    rows = x.numel() // cols if cols else 0
+    w = _same(weight, x, "weight")
+    dx = torch.empty_like(x)
+    dw = torch.empty(cols, dtype=x.dtype, device=x.device) if need_weight else None
+    db = torch.empty(cols, dtype=x.dtype, device=x.device) if need_bias else None
+    ws = None
+    if need_weight or need_bias:
+        ws = _workspace((lib.ptx_layernorm_bwd_workspace_elems(max(rows, 1), cols),), torch.float32,
+                        x.device)
+    with torch.cuda.device(x.device):
+        _call("layernorm_bwd", lib.ptx_layernorm_bwd, _ptr(dout), _ptr(x), _ptr(mean), _ptr(rstd),
+              _ptr(w), _ptr(dx), _ptr(dw), _ptr(db), _ptr(ws), rows, cols, _dt(x), _stream())
+    return dx, dw, db
+
+
 # Workspaces are handed to the kernels uninitialised.  With `poison_workspaces` set (tests),
 # they are filled with NaN first: no result may depend on what a workspace held before.
 poison_workspaces = False

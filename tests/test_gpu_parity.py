@@ -7,7 +7,7 @@ import torch
 
 import protenix_amd as P
 from oracle import pairformer_oracle as O
-from tests.util import oracle_and_product, pad_mask, rel_err, tol
+from tests.util import TOL_BF16, oracle_and_product, pad_mask, rel_err, tol
 
 pytestmark = pytest.mark.gpu
 DTYPES = [torch.float32, torch.bfloat16]
@@ -54,6 +54,69 @@ def test_layernorm_stats_and_closed_forms():
     beta = torch.randn(128, device="cuda")
     const = torch.full((9, 128), 4.25, device="cuda")
     assert torch.allclose(ops.layer_norm(const, torch.randn(128, device="cuda"), beta), beta.expand(9, 128), atol=1e-6)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("rows,cols", [(1000, 128), (4099, 128), (70001, 128), (77, 384), (300, 768),
+                                       (33, 64), (64, 449), (19, 100), (5, 7), (3, 4096),
+                                       (2, 5000), (0, 128)])
+@pytest.mark.parametrize("affine", ["both", "none", "scale", "offset"])
+def test_layernorm_backward(dtype, rows, cols, affine):
+    """FusedLayerNorm under autograd: input and parameter gradients from the HIP backward
+    kernels against the oracle's restatement of the reference's backward arithmetic."""
+    g = torch.Generator().manual_seed(rows * 37 + cols)
+    x = (torch.randn(rows, cols, generator=g) * 3 + 1.5).to(dtype)
+    dout = torch.randn(rows, cols, generator=g).to(dtype)
+    ln = P.LayerNorm(cols, create_scale=affine in ("both", "scale"),
+                     create_offset=affine in ("both", "offset"))
+    with torch.no_grad():
+        if ln.weight is not None:
+            ln.weight.copy_(1 + 0.1 * torch.randn(cols, generator=g))
+        if ln.bias is not None:
+            ln.bias.copy_(0.1 * torch.randn(cols, generator=g))
+    ln = ln.to("cuda", dtype)
+    xg = x.cuda().requires_grad_(True)
+    y = ln(xg)
+    y.backward(dout.cuda())
+    assert xg.grad.shape == x.shape and xg.grad.dtype == dtype
+    if rows == 0:
+        for p_ in ln.parameters():
+            assert torch.count_nonzero(p_.grad) == 0
+        return
+    w = ln.weight.detach().cpu() if ln.weight is not None else None
+    dx, dg, db = O.layer_norm_backward(dout.float(), x.float(), None if w is None else w.float())
+    tol = 1e-4 if dtype == torch.float32 else TOL_BF16
+    assert rel_err(xg.grad, dx) <= tol
+    if ln.weight is not None:
+        assert rel_err(ln.weight.grad, dg) <= tol
+    if ln.bias is not None:
+        assert rel_err(ln.bias.grad, db) <= tol
+
+
+def test_layernorm_backward_c_abi_options_and_determinism():
+    """dgamma / dbeta are optional outputs; the partial sums are added in a fixed order."""
+    from protenix_amd import ops
+    x = torch.randn(5000, 128, device="cuda").bfloat16()
+    dout = torch.randn(5000, 128, device="cuda").bfloat16()
+    w = (1 + 0.1 * torch.randn(128, device="cuda")).bfloat16()
+    _, mean, rstd = ops.layer_norm(x, w, None, 1e-5, return_stats=True)
+    ops.poison_workspaces = True
+    try:
+        full = ops.layer_norm_backward(dout, x, mean, rstd, w, True, True)
+        for need_w, need_b in ((False, False), (True, False), (False, True)):
+            dx, dw, db = ops.layer_norm_backward(dout, x, mean, rstd, w, need_w, need_b)
+            assert torch.equal(dx, full[0])
+            assert (dw is None) == (not need_w) and (db is None) == (not need_b)
+            assert dw is None or torch.equal(dw, full[1])
+            assert db is None or torch.equal(db, full[2])
+        again = ops.layer_norm_backward(dout, x, mean, rstd, w, True, True)
+    finally:
+        ops.poison_workspaces = False
+    assert all(torch.equal(a, b) for a, b in zip(full, again))
+    # no gamma: the same as a gamma of ones
+    ones = ops.layer_norm_backward(dout, x, mean, rstd, torch.ones_like(w), True, True)
+    none = ops.layer_norm_backward(dout, x, mean, rstd, None, True, True)
+    assert all(torch.equal(a, b) for a, b in zip(ones, none))
 
 
 # ------------------------------------------------------------------ TriMul

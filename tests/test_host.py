@@ -44,6 +44,11 @@ def test_argument_validation_without_gpu():
     assert b"dtype" in lib.ptx_last_error_string()
     assert lib.ptx_layernorm_fwd(None, None, None, None, None, None, 4, 128, 1e-5, 0, None) == 1
     assert lib.ptx_layernorm_fwd(None, None, None, None, None, None, 0, 128, 1e-5, 0, None) == 0
+    assert lib.ptx_layernorm_bwd(*([None] * 9), 4, 128, 7, None) == 1
+    assert lib.ptx_layernorm_bwd(*([None] * 9), 4, 128, 0, None) == 1      # null pointers
+    assert lib.ptx_layernorm_bwd(*([None] * 9), 0, 128, 0, None) == 0      # nothing to do
+    assert lib.ptx_layernorm_bwd_workspace_elems(1000, 128) >= 2 * 128
+    assert lib.ptx_layernorm_bwd_workspace_elems(0, 128) == 0
     assert lib.ptx_trimul_contract(None, None, None, 8, 128, 63, 1, None) == 1
     assert b"k_pitch" in lib.ptx_last_error_string()
     assert lib.ptx_trimul_project(*([None] * 10), 8, 64, 64, 64, 0, 1e-5, 1, None) == 2
@@ -63,8 +68,11 @@ def test_modules_refuse_cpu_tensors_and_grad():
     ln = P.LayerNorm(128)
     with torch.no_grad(), pytest.raises(RuntimeError, match="GPU tensor"):
         ln(torch.randn(4, 128))
+    with pytest.raises(RuntimeError, match="GPU tensor"):
+        ln(torch.randn(4, 128))          # LayerNorm has a backward; it still needs the GPU
+    tm = P.TriangleMultiplicationOutgoing(128, 128)
     with pytest.raises(RuntimeError, match="forward-only"):
-        ln(torch.randn(4, 128))
+        tm(torch.randn(1, 4, 4, 128))
     blk = P.PairformerBlock()
     with pytest.raises(RuntimeError, match="inference-only"):
         blk(torch.randn(1, 8, 384), torch.randn(1, 8, 8, 128), None)

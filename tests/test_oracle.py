@@ -46,6 +46,53 @@ def test_layer_norm_matches_library_and_closed_forms():
     assert torch.allclose(O.layer_norm(x, None, b), O.layer_norm(x, None, None) + b, atol=1e-12)
 
 
+@pytest.mark.parametrize("affine", [True, False])
+def test_layer_norm_backward_matches_autograd_and_finite_differences(affine):
+    g = torch.Generator().manual_seed(3)
+    x = (torch.randn(2, 9, 24, generator=g, dtype=D64) * 2 + 0.7).requires_grad_(True)
+    w = (1 + 0.3 * torch.randn(24, generator=g, dtype=D64)).requires_grad_(True) if affine else None
+    b = (0.3 * torch.randn(24, generator=g, dtype=D64)).requires_grad_(True) if affine else None
+    dout = torch.randn(2, 9, 24, generator=g, dtype=D64)
+    y = F.layer_norm(x, (24,), w, b, 1e-5)
+    y.backward(dout)
+    dx, dg, db = O.layer_norm_backward(dout, x.detach(), None if w is None else w.detach())
+    assert torch.allclose(dx, x.grad, atol=1e-12)
+    if affine:
+        assert torch.allclose(dg, w.grad, atol=1e-12) and torch.allclose(db, b.grad, atol=1e-12)
+    else:
+        # without gamma the "parameter gradients" are those of an all-ones gamma / zero beta
+        xn = O.layer_norm(x.detach(), None, None)
+        assert torch.allclose(dg, (dout * xn).sum((0, 1)), atol=1e-12)
+        assert torch.allclose(db, dout.sum((0, 1)), atol=1e-12)
+    # central differences on a few coordinates of the scalar <dout, LN(x)>
+    f = lambda t: (dout * O.layer_norm(t, None if w is None else w.detach(),
+                                       None if b is None else b.detach())).sum()
+    x0 = x.detach()
+    for idx in [(0, 0, 0), (1, 4, 7), (1, 8, 23)]:
+        e = torch.zeros_like(x0)
+        e[idx] = 1e-6
+        assert abs((f(x0 + e) - f(x0 - e)).item() / 2e-6 - dx[idx].item()) < 1e-6
+    # the Jacobian of the normalisation annihilates shifts and (up to eps) rescalings of a row
+    assert dx.sum(-1).abs().max() < 1e-12
+    xc = x0 - x0.mean(-1, keepdim=True)
+    var = (xc ** 2).mean(-1)
+    gd = dout * (w.detach() if affine else 1.0)
+    expect = (gd * xc).sum(-1) * 1e-5 * torch.rsqrt(var + 1e-5) ** 3   # vanishes with eps
+    assert torch.allclose((dx * xc).sum(-1), expect, atol=1e-12)
+
+
+def test_layer_norm_backward_bf16_arithmetic_in_fp32():
+    g = torch.Generator().manual_seed(4)
+    x = (torch.randn(50, 128, generator=g) * 3 + 1).bfloat16()
+    dout = torch.randn(50, 128, generator=g).bfloat16()
+    w = 1 + 0.2 * torch.randn(128, generator=g)
+    dx, dg, db = O.layer_norm_backward(dout, x, w)
+    assert dx.dtype == dg.dtype == db.dtype == torch.bfloat16
+    rx, rg, rb = O.layer_norm_backward(dout.double(), x.double(), w.bfloat16().double())
+    for got, ref in ((dx, rx), (dg, rg), (db, rb)):
+        assert (got.double() - ref).abs().max() <= 2 ** -8 * ref.abs().max()
+
+
 def test_layer_norm_bf16_statistics_in_fp32():
     x = (torch.randn(64, 128) * 3 + 10).bfloat16()
     w = torch.randn(128)
@@ -244,7 +291,9 @@ def test_attention_pair_bias_against_sdpa():
     v = (a @ A.linear_v.weight.T).view(1, N, H, d).transpose(1, 2)
     o = F.scaled_dot_product_attention(q, k, v, attn_mask=bias, scale=1.0).transpose(1, 2).reshape(1, N, cs)
     ref = (o * torch.sigmoid(a @ A.linear_g.weight.T)) @ A.linear_o.weight.T
-    assert torch.allclose(m(a=s, s=None, z=z), ref, atol=1e-10)
+    # the oracle, like the reference (primitives.py:233-291), forms logits and softmax in fp32
+    # whatever the input dtype: fp32 rounding is the floor here, a wrong term gives O(1)
+    assert torch.allclose(m(a=s, s=None, z=z), ref, atol=2e-6, rtol=0)
 
 
 # ------------------------------------------------------------- block / stack
