@@ -83,13 +83,6 @@ template <typename T>
 __device__ __forceinline__ void store8(T* p, typename Vec8<T>::type v) {
   *reinterpret_cast<typename Vec8<T>::type*>(p) = v;
 }
-template <typename T>
-__device__ __forceinline__ typename Vec8<T>::type zero8() {
-  typename Vec8<T>::type z;
-#pragma unroll
-  for (int t = 0; t < 8; ++t) z[t] = (T)0.0f;
-  return z;
-}
 
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;
 
@@ -124,15 +117,6 @@ __device__ __forceinline__ uint64_t uniform64(uint64_t v) {
   const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
   const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
   return ((uint64_t)hi << 32) | lo;
-}
-// The 4-byte form, used to pull cache lines into L2 ahead of time: no register receives the
-// data (a register destination would have to stay reserved until the load returns), it
-// lands in a junk LDS area of 256 bytes at lds_base.
-__device__ __forceinline__ void touch_to_lds4(const void* gptr, uint32_t lds_base) {
-  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off"
-               :
-               : "v"(gptr), "s"(lds_base)
-               : "m0");
 }
 #pragma clang diagnostic pop
 // LDS byte address of p, which must be the same for all lanes (it goes to a scalar register)

@@ -1,10 +1,9 @@
-// Row-tile projections with K = 128: every pair-tensor row (one (i,j) position,
-// 128 channels) is normalised in registers and multiplied by small weight
-// matrices on MFMA; gates, masks, SwiGLU and residual adds are applied to the
-// accumulators, and results leave through an LDS transpose as 16-byte, fully
-// coalesced stores.
+// Row-tile projections with K = c_z (64, 128 or 256): every pair-tensor row (one (i,j)
+// position) is normalised in registers and multiplied by small weight matrices on MFMA;
+// gates, masks and residual adds are applied to the accumulators, and results leave through
+// an LDS transpose as 16-byte, fully coalesced stores.
 //
-// A wave owns RB blocks of 32 rows.  A row block lives in registers as 8
+// A wave owns RB blocks of 32 rows.  A row block lives in registers as KS = c_z / 16
 // operand fragments (16-deep K steps, see common.h): lane l holds row l%32,
 // channels 16*kk + 8*(l/32) .. +7.  The same registers serve as the B operand
 // (result: lane <-> row, register <-> output column; used for row-major
@@ -14,11 +13,15 @@
 // written to a per-wave LDS tile [major][minor] with 8-byte stores and read
 // back as vectors of consecutive minors, which is exactly the global layout.
 //
-// Weights are staged through LDS already permuted into fragment order
-// ([fragment][lane] -> conflict-free 16-byte reads), two 32-column tiles per
-// chunk, double-buffered for bf16.  All loads in the hot loops are
-// unconditional (indices are clamped, results of out-of-range rows are simply
-// not stored) so the MFMA loops carry no branches.
+// Weights sit in LDS already permuted into fragment order ([fragment][lane] ->
+// conflict-free 16-byte reads), in chunks of two 32-column tiles.  Three ways to get them
+// there (InCfg below): bf16 with c_z <= 128 loads every chunk of the launch once per
+// workgroup (one 8-wave workgroup per CU, whose waves then walk over row tiles with no
+// workgroup barrier); bf16 with c_z = 256 and the pair-bias projection stream the chunks
+// through a two-slot ring of direct-to-LDS loads; fp32 stages one chunk at a time through
+// registers.  All loads and stores in the hot loops are unconditional (indices are clamped,
+// lanes without a valid row store to a sink) so the MFMA loops carry no branches and the
+// number of memory operations per chunk is a constant the hand-placed waits can count on.
 #include "common.h"
 #include "kernels.h"
 #include "rowtile.h"
@@ -43,7 +46,7 @@ struct RowGemmInParams {
   RowMap mmap;
   int n;                // tokens (n_rows = n*n for pair tensors)
   int pitch;            // row pitch of a, b (TRIMUL_IN) / v^T, triangle bias (TRIATTN_IN)
-  int aux;              // TRIATTN_IN: heads; PAIRBIAS: heads | out_f32 << 8; TRANSITION_IN: n_factor
+  int aux;              // TRIATTN_IN: heads; PAIRBIAS: heads | out_f32 << 8
   float q_scale;        // TRIATTN_IN: log2(e)/sqrt(d)
   // TRIMUL_OUT only
   const void* x2;       // channel-major triangle product [128][n_rows]

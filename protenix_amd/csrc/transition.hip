@@ -1,4 +1,4 @@
-// Transition (SwiGLU feed-forward) on rows of c = 128 (or 64) channels, one kernel:
+// Transition (SwiGLU feed-forward) on rows of c = 128 (or 64; 256 in bf16) channels, one kernel:
 //   out = [x +] W_o ( silu(W_a LN(x)) * (W_b LN(x)) ),   W_a, W_b [c*n_factor][c]
 // (the comments below give the sizes for c = 128).
 // The hidden activations (n_factor * c per row) never leave the chip: a wave

@@ -17,7 +17,7 @@
 // by log2(e) (by the projection kernel), so on the common path the vector ALU executes per
 // logit one exp2, half a packed bf16 convert and a quarter of a dot2 (the row sum).
 // K and V^T tiles are shared by the 4 waves through LDS in fragment order
-// (double-buffered, one barrier per tile); the bias tile is private to a wave
+// (a ring of three tiles, one barrier per tile); the bias tile is private to a wave
 // and read straight from global (L2-resident: workgroups are numbered so that
 // one XCD works on one head at a time).
 //
