@@ -197,14 +197,21 @@ __global__ __launch_bounds__(256, 2) void triattn_fwd_kernel(
   //                as exp() stays in range), which puts the row on the kOptimisticZero path.
   //   kMasked      tiles with a masked or out-of-range key: the reference's exact fp32
   //                order (q.k + mask_bias) + triangle_bias.
-  auto tile_row = [&](auto mode_tag, int buf, int r, V8 (&tb)[2][2], int next_tile) -> bool {
+  // What a path hands to the commit point of its tile: P^T as the B operand of P.V, this lane's
+  // probability sum, and the factor by which O and l shrink first (1 unless the reference moved).
+  struct TileOut {
+    V8 pf[2][2];
+    float psum, alpha;
+  };
+  auto tile_row = [&](auto mode_tag, int buf, int r, V8 (&tb)[2][2], int next_tile,
+                      TileOut& out) -> bool {
     constexpr int MODE = decltype(mode_tag)::value;
     constexpr bool MASKED = MODE == kMasked;
-    // all 8 operand fragments of the tile are requested from LDS up front, so their
-    // latency is paid once per tile instead of once per MFMA
-    V8 kvf[8];
+    // the 4 K fragments of the tile are requested from LDS up front, so their latency is
+    // paid once per tile instead of once per MFMA (the V^T fragments are read at the commit point)
+    V8 kvf[4];
 #pragma unroll
-    for (int f = 0; f < 8; ++f) kvf[f] = lds_kv[buf][r][f][lane];
+    for (int f = 0; f < 4; ++f) kvf[f] = lds_kv[buf][r][f][lane];
     // the bias registers are refilled with the next tile's bias as soon as this tile's has
     // been consumed (after the last row that shares it, and only once the tile is committed)
     auto refill_bias = [&]() {
@@ -258,8 +265,6 @@ __global__ __launch_bounds__(256, 2) void triattn_fwd_kernel(
       if (!MASKED && __ballot(q_ok && !(fabsf(m_new) < kZeroReferenceLimit)) == 0ull) m_new = 0.0f;
       alpha = fast_exp2((m_run[r] - m_new) * kLog2e);   // 1 when the max did not move
       m_run[r] = m_new;
-#pragma unroll
-      for (int e = 0; e < 16; ++e) acc_o[r][e] *= alpha;
     }
 
     if constexpr (MODE == kOptimisticZero) {
@@ -283,7 +288,7 @@ __global__ __launch_bounds__(256, 2) void triattn_fwd_kernel(
     }
     // P as the B operand of P.V; its row sums are taken from the rounded values the matrix
     // pipe will see (bf16: two per v_dot2c_f32_bf16)
-    V8 pf[2][2];
+    V8 (&pf)[2][2] = out.pf;
     float psum = 0.0f;
 #pragma unroll
     for (int u = 0; u < 2; ++u)
@@ -315,13 +320,8 @@ __global__ __launch_bounds__(256, 2) void triattn_fwd_kernel(
       if (__ballot(q_ok && !(psum < kOptimisticLimit)) != 0ull) return false;
       refill_bias();
     }
-    l_run[r] = l_run[r] * alpha + psum;
-
-    // O^T += V^T P^T
-#pragma unroll
-    for (int u = 0; u < 2; ++u)
-#pragma unroll
-      for (int c = 0; c < 2; ++c) mma32(acc_o[r], kvf[4 + u * 2 + c], pf[u][c]);
+    out.psum = psum;
+    out.alpha = alpha;
     return true;
   };
   auto process_tile = [&](int tile, V8 (&tb)[2][2]) {
@@ -331,18 +331,33 @@ __global__ __launch_bounds__(256, 2) void triattn_fwd_kernel(
     for (int r = 0; r < R; ++r) {
       // Does this tile hold a masked or out-of-range key?  Same answer in all waves.
       const float mb_lane = lds_mb[buf][r][lane];
+      TileOut out;
+      bool rescale = true;   // same in all lanes: did the path move the softmax reference?
       if (__ballot(mb_lane != 0.0f) != 0ull) {
-        tile_row(std::integral_constant<int, kMasked>{}, buf, r, tb, nt);
+        tile_row(std::integral_constant<int, kMasked>{}, buf, r, tb, nt, out);
       } else {
         bool done = false;
         if (tile != 0) {
           if (__ballot(q_ok && m_run[r] != 0.0f) == 0ull)
-            done = tile_row(std::integral_constant<int, kOptimisticZero>{}, buf, r, tb, nt);
+            done = tile_row(std::integral_constant<int, kOptimisticZero>{}, buf, r, tb, nt, out);
           else
-            done = tile_row(std::integral_constant<int, kOptimistic>{}, buf, r, tb, nt);
+            done = tile_row(std::integral_constant<int, kOptimistic>{}, buf, r, tb, nt, out);
         }
-        if (!done) tile_row(std::integral_constant<int, kClassic>{}, buf, r, tb, nt);
+        if (!done) tile_row(std::integral_constant<int, kClassic>{}, buf, r, tb, nt, out);
+        else rescale = false;
       }
+      // The one place where O and l change: whatever path produced P, its product with V is
+      // accumulated here (one definition of the accumulator per tile keeps it in place).
+      if (rescale) {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc_o[r][e] *= out.alpha;
+        l_run[r] *= out.alpha;
+      }
+      l_run[r] += out.psum;
+#pragma unroll
+      for (int u = 0; u < 2; ++u)
+#pragma unroll
+        for (int c = 0; c < 2; ++c) mma32(acc_o[r], lds_kv[buf][r][4 + u * 2 + c][lane], out.pf[u][c]);
     }
   };
 
