@@ -151,7 +151,9 @@ __global__ __launch_bounds__(256) void layernorm_fwd_long_kernel(
 template <typename T, int VEC, int G, int NCHUNK>
 static void launch_ln(const T* x, const T* gamma, const T* beta, T* y, float* mean, float* rstd,
                       int64_t rows, int cols, float eps, hipStream_t stream) {
-  constexpr int UNROLL = (NCHUNK * VEC * (int)sizeof(T) <= 16) ? 4 : (NCHUNK <= 2 ? 2 : 1);
+  // (rows in flight per lane group; measured: 16-bit rows of one vector per lane run 30 %
+  // faster with 2 than with 4, 32-bit rows the other way round)
+  constexpr int UNROLL = (NCHUNK * VEC * (int)sizeof(T) <= 16) ? (sizeof(T) == 2 ? 2 : 4) : (NCHUNK <= 2 ? 2 : 1);
   constexpr int ROWS_PER_BLOCK = 4 * (kWave / G) * UNROLL;
   const int64_t blocks = (rows + ROWS_PER_BLOCK - 1) / ROWS_PER_BLOCK;
   layernorm_fwd_kernel<T, VEC, G, NCHUNK, UNROLL>
