@@ -15,8 +15,8 @@
 //
 // Weights are packed once (transition_pack) into MFMA fragment order, chunk by
 // chunk, and stream global -> LDS with direct-to-LDS loads into a ring of
-// chunk buffers shared by the workgroup's 4 waves.  One wave per SIMD (the
-// accumulators and the row fragments take ~370 registers), so the wave is
+// chunk buffers shared by the workgroup's waves.  One or two waves per SIMD (with two row
+// blocks the accumulators and the row fragments take ~370 registers), so the wave is
 // pipelined by hand: while the MFMAs of chunk j's GEMM1 run, the VALU computes
 // the activation of chunk j-1, whose GEMM2 follows; LDS fragment reads are issued
 // one step ahead of their use.
@@ -31,14 +31,20 @@ namespace ptx {
 // NOB = c / 32 output blocks.
 template <typename T, int KS> struct TrCfg {
   // (rows of 256 channels, bf16 only: one row block, and three 48 KB chunk buffers)
-  static constexpr int RB = (sizeof(T) == 2 && KS <= 8) ? 2 : 1;     // row blocks of 32 per wave
+  // Waves per workgroup.  bf16 rows of 128 channels: 8 waves (two per SIMD) of one row block
+  // each.  A single wave issues a vector instruction only every ~9 cycles (two waves: one every
+  // ~5 per SIMD), and the SwiGLU is vector work, so two thin waves beat one fat one by 6 %
+  // although every weight fragment read from LDS then feeds one MFMA instead of two.
+  static constexpr int NW = (sizeof(T) == 2 && KS == 8) ? 8 : 4;
+  static constexpr int RB = (sizeof(T) == 2 && KS <= 8 && NW == 4) ? 2 : 1;     // row blocks of 32 per wave
   static constexpr int NBUF = (sizeof(T) == 2 && KS <= 8) ? 4 : 3;   // chunk buffers in LDS
   static constexpr int D = NBUF - 2;                    // chunks the loads run ahead (two are in use)
   static constexpr int PIECES = (int)sizeof(T) / 2;     // 16-byte pieces per lane and fragment
   static constexpr int NOB = KS / 2;
   // fragments per chunk of 32 hidden: W_a KS K steps, W_b KS, W_o NOB x 2
   static constexpr int FRAGS = 3 * KS;
-  static constexpr int FPW = FRAGS / 4;                 // fragments each wave moves per chunk
+  static constexpr int FPW = FRAGS / NW;                // fragments each wave moves per chunk
+  static_assert(FRAGS % NW == 0, "every wave moves the same number of fragments");
   static constexpr int DMA_PER_CHUNK = FPW * PIECES;
 };
 
@@ -76,7 +82,7 @@ __global__ void transition_pack_kernel(const T* __restrict__ w_a, const T* __res
 }
 
 template <typename T, int KS>
-__global__ __launch_bounds__(256) void transition_fused_kernel(
+__global__ __launch_bounds__((TrCfg<T, KS>::NW * 64)) void transition_fused_kernel(
     const T* x, const T* __restrict__ gamma, const T* __restrict__ beta,
     const T* __restrict__ packed, T* out, int64_t n_rows, int n_chunks, int add_residual,
     float eps) {
@@ -84,14 +90,14 @@ __global__ __launch_bounds__(256) void transition_fused_kernel(
   typedef typename VecE<T>::type VE_t;
   typedef TrCfg<T, KS> G;
   typedef Cfg<T> C;
-  constexpr int RB = G::RB, NBUF = G::NBUF, D = G::D, PIECES = G::PIECES, FPW = G::FPW;
+  constexpr int RB = G::RB, NBUF = G::NBUF, D = G::D, PIECES = G::PIECES, FPW = G::FPW, NW = G::NW;
   constexpr int NOB = G::NOB, kTrFrags = G::FRAGS, kCx = 16 * KS;
   __shared__ u32x4_t lds_w[NBUF][kTrFrags][PIECES][kWave];
-  static_assert(sizeof(T) * 4 * 32 * C::PITCH <= sizeof(u32x4_t) * kTrFrags * PIECES * kWave,
+  static_assert(sizeof(T) * NW * 32 * C::PITCH <= sizeof(u32x4_t) * kTrFrags * PIECES * kWave,
                 "the staging tiles reuse chunk buffer 0");
 
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int64_t row0 = ((int64_t)blockIdx.x * 4 + wave) * (RB * 32);
+  const int64_t row0 = ((int64_t)blockIdx.x * NW + wave) * (RB * 32);
 
   // chunk j (clamped for the address) -> buffer j % NBUF; every wave moves FPW fragments
   // (address = wave-uniform base in scalar registers + this lane's offset inside a fragment:
@@ -296,9 +302,9 @@ template <typename T, int KS>
 static int transition_fwd_ks(const void* x, const void* ln_w, const void* ln_b, const void* packed,
                              void* out, int64_t rows, int n_factor, int add_residual, float eps,
                              hipStream_t stream) {
-  const int64_t rows_per_block = 4 * TrCfg<T, KS>::RB * 32;
+  const int64_t rows_per_block = TrCfg<T, KS>::NW * TrCfg<T, KS>::RB * 32;
   const int64_t blocks = (rows + rows_per_block - 1) / rows_per_block;
-  transition_fused_kernel<T, KS><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(
+  transition_fused_kernel<T, KS><<<dim3((unsigned)blocks), dim3(TrCfg<T, KS>::NW * 64), 0, stream>>>(
       (const T*)x, (const T*)ln_w, (const T*)ln_b, (const T*)packed, (T*)out, rows,
       16 * KS * n_factor / 32, add_residual, eps);
   return 0;
