@@ -251,6 +251,31 @@ def test_block_without_single_track():
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+def test_block_batched_and_noncontiguous_inputs(dtype):
+    """Leading batch dimensions, a non-contiguous pair tensor (a transposed view, as
+    pairformer.py:201 produces it), a boolean-valued mask in another dtype: the caller's
+    tensors are left untouched unless inplace_safe is set."""
+    ref, prod = oracle_and_product(O.PairformerBlock, P.PairformerBlock, dtype=dtype)
+    n = 48
+    g = torch.Generator().manual_seed(99)
+    z = torch.randn(2, n, n, 128, generator=g).to(dtype)
+    s = torch.randn(2, n, 384, generator=g).to(dtype)
+    pm = torch.stack([pad_mask(n, 5)[0], pad_mask(n, 0)[0]])           # fp32, per-sample padding
+    with torch.no_grad():
+        s_ref, z_ref = ref(s.float(), z.float(), pm)
+        z_dev = z.cuda().transpose(1, 2).contiguous().transpose(1, 2)   # same values, strided
+        assert not z_dev.is_contiguous()
+        z_keep = z_dev.clone()
+        s_got, z_got = prod(s.cuda(), z_dev, pm.cuda())
+    assert torch.equal(z_dev, z_keep)
+    assert rel_err(z_got, z_ref) <= tol(dtype) and rel_err(s_got, s_ref) <= tol(dtype)
+    # each sample on its own gives the same answer as inside the batch
+    with torch.no_grad():
+        s1, z1 = prod(s[1:].cuda(), z[1:].cuda(), pm[1:].cuda())
+    assert torch.equal(z1, z_got[1:]) and torch.equal(s1, s_got[1:])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_stack_4_blocks(dtype):
     ref, prod = oracle_and_product(O.PairformerStack, P.PairformerStack, n_blocks=4, dtype=dtype)
     s, z, pm = O.make_inputs(80, n_pad=6, dtype=dtype)
