@@ -2,11 +2,13 @@
 // are never written anywhere.
 //
 // One workgroup (4 waves) owns one (row i, head h) pair and 128 queries; each
-// wave owns 32 queries and walks over the keys in tiles of 64.  Per tile:
-//   S^T[key][query]  = K Q^T + bias     2 x (2 + 2) MFMA (two 32-key halves)
+// wave owns 32 queries and walks over the keys in staged tiles of 64, which it
+// processes as two halves of 32 keys (16 logit registers at a time: four waves
+// fit a SIMD).  Per half:
+//   S^T[key][query]  = K Q^T + bias     2 + 2 MFMA
 //   online softmax along keys = along the registers of a lane (+ one exchange
 //   with the other half-wave), because MFMA puts the query on the lane
-//   O^T[d][query]   += V^T P^T          4 MFMA, P^T taken straight from the S^T
+//   O^T[d][query]   += V^T P^T          2 MFMA, P^T taken straight from the S^T
 //   accumulators with no shuffle
 // MFMA row m of half u is mapped to key 32*((m>>2)&1) + 16*u + 4*(m>>3) + (m&3),
 // which makes register r of half-wave g hold key 32*g + 16*u + r: 16 consecutive
@@ -36,7 +38,7 @@ namespace ptx {
 constexpr int kD = 32;          // head dim
 constexpr int kKeyTile = 64;
 constexpr float kLog2e = 1.4426950408889634f;
-// tile_row: code paths, and the largest per-lane probability sum of a tile (32 values) the
+// half_row: code paths, and the largest per-lane probability sum of a half tile (16 values) the
 // optimistic path accepts
 enum { kOptimistic = 0, kClassic = 1, kMasked = 2, kOptimisticZero = 3 };
 constexpr float kOptimisticLimit = 1.0e12f;
@@ -45,14 +47,12 @@ constexpr float kLn2 = 0.6931471805599453f;
 // replaced by the reference 0, which makes exp2() of the raw logit the probability
 constexpr float kZeroReferenceLimit = 14.0f;
 
-// Rows of the pair tensor handled by one wave (the bias tile is then loaded once per key
-// tile and reused).  More than one row does not fit the register budget of 2 waves/SIMD.
-#ifndef PTX_ATTN_ROWS
+// Rows of the pair tensor handled by one wave: one (more would share the bias tile, but do not
+// fit the register budget).
 #define PTX_ATTN_ROWS 1
-#endif
 
 template <typename T, int R>
-__global__ __launch_bounds__(256, 2) void triattn_fwd_kernel(
+__global__ __launch_bounds__(256, (sizeof(T) == 2 ? 4 : 2)) void triattn_fwd_kernel(
     const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ vt,
     const T* gate, const T* __restrict__ bias, const T* __restrict__ mask,
     T* o, int n, int heads, int key_pitch, int mask_transposed, float inf,
@@ -180,14 +180,14 @@ __global__ __launch_bounds__(256, 2) void triattn_fwd_kernel(
     l_run[r] = 0.0f;
   }
 
-  // One key tile of one row: logits, online softmax, P.V.  `tb` was fetched one tile ago.
-  // Three complete instantiations, so that the rarer paths share no code with - and cannot
-  // be speculated into - the common one:
+  // One half of a key tile: logits, online softmax, P^T.  `tb` was fetched one tile ago.
+  // Complete instantiations, so that the rarer paths share no code with - and cannot be
+  // speculated into - the common one:
   //   kOptimistic  The softmax reference m_run only has to keep exp() in
   //                range, so it is NOT updated: probabilities are taken against the reference
   //                left by earlier tiles, no tile maximum is formed and O, l are not rescaled.
   //                If a probability sum leaves the safe range (a logit ~28 above the
-  //                reference, or no reference yet), nothing has been committed and the tile
+  //                reference, or no reference yet), nothing has been committed and the half
   //                is redone by kClassic.  Returns false in that case (same in all lanes).
   //   kOptimisticZero  the common path: the same with the reference 0 in all lanes.  q and
   //                the triangle bias arrive multiplied by log2(e), so the matrix pipe's
@@ -197,170 +197,135 @@ __global__ __launch_bounds__(256, 2) void triattn_fwd_kernel(
   //                as exp() stays in range), which puts the row on the kOptimisticZero path.
   //   kMasked      tiles with a masked or out-of-range key: the reference's exact fp32
   //                order (q.k + mask_bias) + triangle_bias.
-  // What a path hands to the commit point of its tile: P^T as the B operand of P.V, this lane's
-  // probability sum, and the factor by which O and l shrink first (1 unless the reference moved).
-  struct TileOut {
-    V8 pf[2][2];
+  // A path works on one 32-key half u of the staged tile (keys 32g + 16u + 0..15 of half-wave
+  // g): 16 logit registers instead of 32, which lets four waves share a SIMD (a wave issues a
+  // vector instruction only every ~9 cycles; it takes several to keep the vector unit busy).
+  // What a path hands to the commit point of its half: P^T as the B operand of P.V, this
+  // lane's probability sum, and the factor by which O and l shrink first (1 unless the
+  // reference moved).
+  struct HalfOut {
+    V8 pf[2];
     float psum, alpha;
   };
-  auto tile_row = [&](auto mode_tag, int buf, int r, V8 (&tb)[2][2], int next_tile,
-                      TileOut& out) -> bool {
+  auto half_row = [&](auto mode_tag, int buf, int u, V8 (&tbh)[2], HalfOut& out) -> bool {
     constexpr int MODE = decltype(mode_tag)::value;
     constexpr bool MASKED = MODE == kMasked;
-    // the 4 K fragments of the tile are requested from LDS up front, so their latency is
-    // paid once per tile instead of once per MFMA (the V^T fragments are read at the commit point)
-    V8 kvf[4];
+    V8 kf[2];
 #pragma unroll
-    for (int f = 0; f < 4; ++f) kvf[f] = lds_kv[buf][r][f][lane];
-    // the bias registers are refilled with the next tile's bias as soon as this tile's has
-    // been consumed (after the last row that shares it, and only once the tile is committed)
-    auto refill_bias = [&]() {
-      if (r == R - 1) fetch_bias(next_tile, tb);
-    };
-    f32x16 s[2];
+    for (int kk = 0; kk < 2; ++kk) kf[kk] = lds_kv[buf][0][u * 2 + kk][lane];
+    f32x16 s;
 #pragma unroll
-    for (int u = 0; u < 2; ++u) {
+    for (int e = 0; e < 16; ++e) s[e] = 0.0f;
 #pragma unroll
-      for (int e = 0; e < 16; ++e) s[u][e] = 0.0f;
-#pragma unroll
-      for (int kk = 0; kk < 2; ++kk) mma32(s[u], kvf[u * 2 + kk], qf[r][kk]);
-    }
+    for (int kk = 0; kk < 2; ++kk) mma32(s, kf[kk], qf[0][kk]);
     if constexpr (!MASKED) {
-      // bias on the matrix pipe: S^T += Sel * Bias
 #pragma unroll
-      for (int u = 0; u < 2; ++u)
-#pragma unroll
-        for (int c = 0; c < 2; ++c) mma32(s[u], sel[c], tb[u][c]);
+      for (int c = 0; c < 2; ++c) mma32(s, sel[c], tbh[c]);
     } else {
-      // exact reference order in fp32: (q.k + mask_bias) + triangle_bias
 #pragma unroll
-      for (int u = 0; u < 2; ++u)
+      for (int c = 0; c < 2; ++c) {
+        const f32x8 b = to_f32(tbh[c]);
+        const f32x4 m0 = *reinterpret_cast<const f32x4*>(&lds_mb[buf][0][32 * g + 16 * u + 8 * c]);
+        const f32x4 m1 = *reinterpret_cast<const f32x4*>(&lds_mb[buf][0][32 * g + 16 * u + 8 * c + 4]);
 #pragma unroll
-        for (int c = 0; c < 2; ++c) {
-          const f32x8 b = to_f32(tb[u][c]);
-          const f32x4 m0 = *reinterpret_cast<const f32x4*>(&lds_mb[buf][r][32 * g + 16 * u + 8 * c]);
-          const f32x4 m1 = *reinterpret_cast<const f32x4*>(&lds_mb[buf][r][32 * g + 16 * u + 8 * c + 4]);
-#pragma unroll
-          for (int t = 0; t < 8; ++t) {
-            const float mbv = t < 4 ? m0[t & 3] : m1[t & 3];
-            // q.k and the bias arrive in log2 units: back to natural ones for this sum
-            const float v = (s[u][8 * c + t] * kLn2 + mbv) + b[t] * kLn2;
-            s[u][8 * c + t] = mbv == -INFINITY ? -INFINITY : v;   // key beyond n
-          }
+        for (int t = 0; t < 8; ++t) {
+          const float mbv = t < 4 ? m0[t & 3] : m1[t & 3];
+          const float v = (s[8 * c + t] * kLn2 + mbv) + b[t] * kLn2;
+          s[8 * c + t] = mbv == -INFINITY ? -INFINITY : v;
         }
+      }
     }
-
     float alpha = 1.0f;
     if constexpr (MODE == kClassic || MODE == kMasked) {
-      refill_bias();
       float mx[8];
 #pragma unroll
-      for (int j = 0; j < 8; ++j)
-        mx[j] = fmaxf(fmaxf(s[0][2 * j], s[0][2 * j + 1]), fmaxf(s[1][2 * j], s[1][2 * j + 1]));
+      for (int j = 0; j < 8; ++j) mx[j] = fmaxf(s[2 * j], s[2 * j + 1]);
       float mt = fmaxf(fmaxf(fmaxf(mx[0], mx[1]), fmaxf(mx[2], mx[3])),
                        fmaxf(fmaxf(mx[4], mx[5]), fmaxf(mx[6], mx[7])));
       mt = fmaxf(mt, swap32(mt));
-      if (!MASKED) mt *= kLn2;                        // unmasked logits are in log2 units
-      float m_new = fmaxf(m_run[r], mt);              // finite: key0 < n is never excluded
+      if (!MASKED) mt *= kLn2;
+      // (a half whose keys all lie beyond n has mt = -inf: the reference stays where it is)
+      float m_new = fmaxf(m_run[0], mt);
       if (!MASKED && __ballot(q_ok && !(fabsf(m_new) < kZeroReferenceLimit)) == 0ull) m_new = 0.0f;
-      alpha = fast_exp2((m_run[r] - m_new) * kLog2e);   // 1 when the max did not move
-      m_run[r] = m_new;
+      alpha = m_new == -INFINITY ? 1.0f : fast_exp2((m_run[0] - m_new) * kLog2e);
+      m_run[0] = m_new;
     }
-
     if constexpr (MODE == kOptimisticZero) {
-      // reference 0: the logit in log2 units is the exponent
 #pragma unroll
-      for (int u = 0; u < 2; ++u)
-#pragma unroll
-        for (int e = 0; e < 16; ++e) s[u][e] = fast_exp2(s[u][e]);
+      for (int e = 0; e < 16; ++e) s[e] = fast_exp2(s[e]);
     } else if constexpr (!MASKED) {
-      const float nml = -m_run[r] * kLog2e;
+      const float nml = -m_run[0] * kLog2e;
 #pragma unroll
-      for (int u = 0; u < 2; ++u)
-#pragma unroll
-        for (int e = 0; e < 16; ++e) s[u][e] = fast_exp2(s[u][e] + nml);
+      for (int e = 0; e < 16; ++e) s[e] = fast_exp2(s[e] + nml);
     } else {
-      // (s - m) first: exact when both sit near -1e9
 #pragma unroll
-      for (int u = 0; u < 2; ++u)
-#pragma unroll
-        for (int e = 0; e < 16; ++e) s[u][e] = fast_exp2((s[u][e] - m_run[r]) * kLog2e);
+      for (int e = 0; e < 16; ++e)
+        s[e] = m_run[0] == -INFINITY ? 0.0f : fast_exp2((s[e] - m_run[0]) * kLog2e);
     }
-    // P as the B operand of P.V; its row sums are taken from the rounded values the matrix
-    // pipe will see (bf16: two per v_dot2c_f32_bf16)
-    V8 (&pf)[2][2] = out.pf;
     float psum = 0.0f;
 #pragma unroll
-    for (int u = 0; u < 2; ++u)
+    for (int c = 0; c < 2; ++c) {
+      f32x8 p8;
 #pragma unroll
-      for (int c = 0; c < 2; ++c) {
-        f32x8 p8;
+      for (int t = 0; t < 8; ++t) p8[t] = s[8 * c + t];
+      out.pf[c] = from_f32<T>(p8);
+      if constexpr (sizeof(T) == 2) {
+        typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
+        bf16x2_t ones;
+        ones[0] = (__bf16)1.0f;
+        ones[1] = (__bf16)1.0f;
 #pragma unroll
-        for (int t = 0; t < 8; ++t) p8[t] = s[u][8 * c + t];
-        pf[u][c] = from_f32<T>(p8);
-        if constexpr (sizeof(T) == 2) {
-          typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
-          bf16x2_t ones;
-          ones[0] = (__bf16)1.0f;
-          ones[1] = (__bf16)1.0f;
-#pragma unroll
-          for (int t = 0; t < 4; ++t) {
-            bf16x2_t pr;
-            pr[0] = pf[u][c][2 * t];
-            pr[1] = pf[u][c][2 * t + 1];
-            psum = __builtin_amdgcn_fdot2_f32_bf16(pr, ones, psum, false);
-          }
-        } else {
-#pragma unroll
-          for (int t = 0; t < 8; ++t) psum += p8[t];
+        for (int t = 0; t < 4; ++t) {
+          bf16x2_t pr;
+          pr[0] = out.pf[c][2 * t];
+          pr[1] = out.pf[c][2 * t + 1];
+          psum = __builtin_amdgcn_fdot2_f32_bf16(pr, ones, psum, false);
         }
+      } else {
+#pragma unroll
+        for (int t = 0; t < 8; ++t) psum += p8[t];
       }
+    }
     if constexpr (MODE == kOptimistic || MODE == kOptimisticZero) {
-      // out of the safe range (also catches inf and NaN)?  Nothing committed yet: redo.
       if (__ballot(q_ok && !(psum < kOptimisticLimit)) != 0ull) return false;
-      refill_bias();
     }
     out.psum = psum;
     out.alpha = alpha;
     return true;
   };
   auto process_tile = [&](int tile, V8 (&tb)[2][2]) {
+    static_assert(R == 1, "the register budget of four waves per SIMD holds one row per wave");
     const int buf = tile % 3;
-    const int nt = tile + 1;
+    const float mb_lane = lds_mb[buf][0][lane];
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
-      // Does this tile hold a masked or out-of-range key?  Same answer in all waves.
-      const float mb_lane = lds_mb[buf][r][lane];
-      TileOut out;
-      bool rescale = true;   // same in all lanes: did the path move the softmax reference?
-      if (__ballot(mb_lane != 0.0f) != 0ull) {
-        tile_row(std::integral_constant<int, kMasked>{}, buf, r, tb, nt, out);
+    for (int u = 0; u < 2; ++u) {
+      HalfOut out;
+      bool rescale = true;
+      // this half's keys are those of lanes with bit 4 == u
+      if (__ballot(mb_lane != 0.0f && ((lane >> 4) & 1) == u) != 0ull) {
+        half_row(std::integral_constant<int, kMasked>{}, buf, u, tb[u], out);
       } else {
         bool done = false;
-        if (tile != 0) {
-          if (__ballot(q_ok && m_run[r] != 0.0f) == 0ull)
-            done = tile_row(std::integral_constant<int, kOptimisticZero>{}, buf, r, tb, nt, out);
+        if (tile != 0 || u != 0) {
+          if (__ballot(q_ok && m_run[0] != 0.0f) == 0ull)
+            done = half_row(std::integral_constant<int, kOptimisticZero>{}, buf, u, tb[u], out);
           else
-            done = tile_row(std::integral_constant<int, kOptimistic>{}, buf, r, tb, nt, out);
+            done = half_row(std::integral_constant<int, kOptimistic>{}, buf, u, tb[u], out);
         }
-        if (!done) tile_row(std::integral_constant<int, kClassic>{}, buf, r, tb, nt, out);
+        if (!done) half_row(std::integral_constant<int, kClassic>{}, buf, u, tb[u], out);
         else rescale = false;
       }
-      // The one place where O and l change: whatever path produced P, its product with V is
-      // accumulated here (one definition of the accumulator per tile keeps it in place).
       if (rescale) {
 #pragma unroll
-        for (int e = 0; e < 16; ++e) acc_o[r][e] *= out.alpha;
-        l_run[r] *= out.alpha;
+        for (int e = 0; e < 16; ++e) acc_o[0][e] *= out.alpha;
+        l_run[0] *= out.alpha;
       }
-      l_run[r] += out.psum;
+      l_run[0] += out.psum;
 #pragma unroll
-      for (int u = 0; u < 2; ++u)
-#pragma unroll
-        for (int c = 0; c < 2; ++c) mma32(acc_o[r], lds_kv[buf][r][4 + u * 2 + c][lane], out.pf[u][c]);
+      for (int c = 0; c < 2; ++c) mma32(acc_o[0], lds_kv[buf][0][4 + u * 2 + c][lane], out.pf[c]);
     }
+    fetch_bias(tile + 1, tb);
   };
-
   // Tile t+2 travels global -> registers -> LDS while tile t is processed; the bias tile of
   // t+1 is requested into the bias registers once tile t has consumed them.
   V8 tbias[2][2];
