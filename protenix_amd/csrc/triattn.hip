@@ -123,6 +123,11 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? 4 : 2)) void triattn_fwd_ker
   // for memory sits in the issue path.
   V8 pre[2 * R];
   T pre_mv;
+  // mask value of key kc for this wave's row: m_base[kc * m_stride] (stride 0: no mask, any
+  // valid address - the value is discarded)
+  const int m_row = min(i0 + min(wave, R - 1), n - 1);
+  const unsigned m_stride = has_mask ? (mask_transposed ? n : 1) : 0;
+  const T* m_base = mask_or_dummy + (has_mask ? (mask_transposed ? (int64_t)m_row : (int64_t)m_row * n) : 0);
   auto fetch = [&](int tile) {
     const int64_t atile = min(tile, n_tiles - 1);
 #pragma unroll
@@ -134,9 +139,7 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? 4 : 2)) void triattn_fwd_ker
     }
     // wave w < R publishes the mask bias of row i0 + w; all waves load (uniform load count)
     const int kc = min(tile * kKeyTile + lane, n - 1);
-    const int row = min(i0 + min(wave, R - 1), n - 1);
-    const int64_t mi = mask_transposed ? (int64_t)kc * n + row : (int64_t)row * n + kc;
-    pre_mv = mask_or_dummy[has_mask ? mi : 0];
+    pre_mv = m_base[__umul24(kc, m_stride)];   // both below 2^15
   };
   auto stash = [&](int tile) {
     const int buf = tile % 3;
