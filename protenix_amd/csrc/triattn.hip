@@ -13,11 +13,10 @@
 // MFMA row m of half u is mapped to key 32*((m>>2)&1) + 16*u + 4*(m>>3) + (m&3),
 // which makes register r of half-wave g hold key 32*g + 16*u + r: 16 consecutive
 // keys -> 16-byte bias loads, and 8 consecutive keys per P.V operand slot group.
-// The triangle bias never touches the vector ALU: its raw bf16 registers are the
-// B operand of an MFMA whose A operand is the constant 0/1 matrix that undoes the
-// key permutation, accumulating straight into S^T.  q and the bias are stored multiplied
-// by log2(e) (by the projection kernel), so on the common path the vector ALU executes per
-// logit one exp2, half a packed bf16 convert and a quarter of a dot2 (the row sum).
+// The triangle bias is the initial value of the S^T accumulators (converted to fp32 if it
+// is stored in 16 bits).  q and the bias are stored multiplied by log2(e) (by the projection
+// kernel), so on the common path the vector ALU executes per logit one conversion, one exp2,
+// half a packed bf16 convert and half a dot2 (the row sum).
 // K and V^T tiles are shared by the 4 waves through LDS in fragment order
 // (a ring of three tiles, one barrier per tile); the bias tile is private to a wave
 // and read straight from global (L2-resident: workgroups are numbered so that
@@ -99,17 +98,6 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? 4 : 2)) void triattn_fwd_ker
     qrow[r] = (((int64_t)h * n + min(i0 + r, n - 1)) * n + qi) * kD;
 #pragma unroll
     for (int kk = 0; kk < 2; ++kk) qf[r][kk] = load8<T>(q + qrow[r] + 16 * kk + 8 * g);
-  }
-
-  // Constant operand sel[s]: A matrix with sel[m][slot (g,t)] = 1 iff key(m) is the key behind
-  // slot (g,t) of step s, i.e. g == (m>>2)&1 and 8s+t == 4*(m>>3) + (m&3).
-  V8 sel[2];
-  {
-    const int g_m = (ln >> 2) & 1, r_m = 4 * (ln >> 3) + (ln & 3);
-#pragma unroll
-    for (int sgrp = 0; sgrp < 2; ++sgrp)
-#pragma unroll
-      for (int t = 0; t < 8; ++t) sel[sgrp][t] = (T)((g == g_m && 8 * sgrp + t == r_m) ? 1.0f : 0.0f);
   }
 
   // ---- cooperative tile loader: 8*R fragments per key tile, 2*R per wave ----
@@ -217,14 +205,19 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? 4 : 2)) void triattn_fwd_ker
 #pragma unroll
     for (int kk = 0; kk < 2; ++kk) kf[kk] = lds_kv[buf][0][u * 2 + kk][lane];
     f32x16 s;
+    if constexpr (!MASKED) {
+      // S^T starts from the bias, the C operand of the first product: register e of this lane
+      // <-> element e of its 16 stored values (16-bit: one conversion per logit, which with
+      // four waves per SIMD costs less than adding the bias on the matrix pipe)
+      const f32x8 b0 = to_f32(tbh[0]), b1 = to_f32(tbh[1]);
+      s = __builtin_shufflevector(b0, b1, 0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15);
+    } else {
 #pragma unroll
-    for (int e = 0; e < 16; ++e) s[e] = 0.0f;
+      for (int e = 0; e < 16; ++e) s[e] = 0.0f;
+    }
 #pragma unroll
     for (int kk = 0; kk < 2; ++kk) mma32(s, kf[kk], qf[0][kk]);
-    if constexpr (!MASKED) {
-#pragma unroll
-      for (int c = 0; c < 2; ++c) mma32(s, sel[c], tbh[c]);
-    } else {
+    if constexpr (MASKED) {
 #pragma unroll
       for (int c = 0; c < 2; ++c) {
         const f32x8 b = to_f32(tbh[c]);
