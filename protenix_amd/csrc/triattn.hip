@@ -342,6 +342,12 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? 4 : 2)) void triattn_fwd_ker
 
   // ---- normalise, gate, store: lane <-> query, register e <-> d = acc_row(e, g) ----
   // o may alias gate: every gate load is issued before the first store.
+  // (the row offsets are formed again from a laundered query index: kept across the key loop
+  // they cost two registers of a budget that has none to spare)
+  int qi_again = qi;
+  asm volatile("" : "+v"(qi_again));
+#pragma unroll
+  for (int r = 0; r < R; ++r) qrow[r] = (((int64_t)h * n + min(i0 + r, n - 1)) * n + qi_again) * kD;
   f32x4 gv[R][4];
 #pragma unroll
   for (int r = 0; r < R; ++r)
