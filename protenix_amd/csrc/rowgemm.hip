@@ -152,6 +152,13 @@ rowgemm_in_kernel(RowGemmInParams p) {
   __shared__ __attribute__((aligned(16))) T lds_res[MODE == kTriMulOut ? NW : 1][MODE == kTriMulOut ? RB * 32 : 1][kResPitch];
   __shared__ __attribute__((aligned(16))) T lds_stage[NW][NST][32 * C::PITCH];
   __shared__ __attribute__((aligned(16))) float lds_mask[MODE == kTriMulIn ? NW : 1][RB * 32];
+  // LayerNorm weight and bias (absent: 1 and 0) as fp32, converted once per workgroup: read
+  // from global memory they cost every row tile as many load instructions as the tile's own
+  // rows and, in 16 bits, a conversion per value and tile.  Only where the fp32 copies fit the
+  // register budget: in the triangle-multiplication kernels the wider operands spill more
+  // than the conversions cost, and those keep reading the parameters from global memory.
+  constexpr bool kLdsAffine = MODE == kTriAttnIn || MODE == kPairBias;
+  __shared__ __attribute__((aligned(16))) float lds_affine[2][kLdsAffine ? kCz : 1];
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int n = lane & 31, g = lane >> 5;
   T* st = lds_stage[wave][0];
@@ -159,6 +166,14 @@ rowgemm_in_kernel(RowGemmInParams p) {
   const bool vec_ok = (p.n % C::VE) == 0;   // channel-major vectors stay inside one plane row
   T* const sink = reinterpret_cast<T*>(g_store_sink) + lane * C::VE;
   constexpr int nch = IC::NCH;
+
+  if constexpr (kLdsAffine) {
+    for (int c = threadIdx.x; c < kCz; c += NW * kWave) {
+      lds_affine[0][c] = p.gamma ? to_f32(((const T*)p.gamma)[c]) : 1.0f;
+      lds_affine[1][c] = p.beta ? to_f32(((const T*)p.beta)[c]) : 0.0f;
+    }
+    __syncthreads();
+  }
 
   // Work units ("wave tiles").  kTriMulIn works on 2-D patches of the pair tensor instead of
   // runs of logical rows: four waves cover 16*RB outer indices x 8 inner indices, a row block
@@ -250,8 +265,8 @@ rowgemm_in_kernel(RowGemmInParams p) {
     load_rows_at<T, RB, true>(xf, (const T*)p.x, off, gamma, beta, p.eps, lane);
   } else if constexpr (MODE == kTriMulOut) {
     RowFrags<T, RB, KS> zraw;
-    load_rows<T, RB, false>(zraw, (const T*)p.x, p.xmap, row0, p.n_rows, nullptr, nullptr, 0.0f,
-                            lane);
+    load_rows<T, RB, false>(zraw, (const T*)p.x, p.xmap, row0, p.n_rows, (const T*)nullptr,
+                            (const T*)nullptr, 0.0f, lane);
     wave_lds_sync();   // the previous tile's residual reads are done
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb) {
@@ -261,7 +276,11 @@ rowgemm_in_kernel(RowGemmInParams p) {
       normalize_raw<T>(zraw.f[rb], gamma, beta, p.eps, g, xf.f[rb]);
     }
   } else {
-    load_rows<T, RB, true>(xf, (const T*)p.x, p.xmap, row0, p.n_rows, gamma, beta, p.eps, lane);
+    if constexpr (kLdsAffine)
+      load_rows<T, RB, true, KS, float, false>(xf, (const T*)p.x, p.xmap, row0, p.n_rows, lds_affine[0],
+                                               lds_affine[1], p.eps, lane);
+    else
+      load_rows<T, RB, true>(xf, (const T*)p.x, p.xmap, row0, p.n_rows, gamma, beta, p.eps, lane);
   }
 
   // kTriMulOut: second fragment set = LayerNorm_out of the channel-major triangle product,
@@ -799,8 +818,8 @@ __global__ __launch_bounds__(256, 2) void rowgemm_out_kernel(RowGemmOutParams p)
                                   16 * (kk & 1) + 8 * g_);
       }
     } else {
-      load_rows<T, RB, false>(af, (const T*)p.a + slab * kC, amap, row0, p.n_rows, nullptr,
-                              nullptr, 0.0f, lane);
+      load_rows<T, RB, false>(af, (const T*)p.a + slab * kC, amap, row0, p.n_rows,
+                              (const T*)nullptr, (const T*)nullptr, 0.0f, lane);
     }
 #pragma unroll
     for (int half = 0; half < NH; ++half) {

@@ -55,12 +55,14 @@ template <typename T> __device__ __forceinline__ const T* default_beta() {
 // Mean / rstd of a row of 16*KS channels spread over the two half-wave lanes that hold it,
 // then gamma/beta (either may be null); result rounded to T like the reference's
 // LayerNorm output.
-template <typename T, int KS>
-__device__ __forceinline__ void normalize_row(f32x8 (&v)[KS], const T* __restrict__ gamma,
-                                              const T* __restrict__ beta, float eps, int g,
+// gamma / beta are read as type P: T from global memory (null: the stand-ins above), or float
+// from a copy the caller keeps in LDS (P = float, DEFAULTS = false: never null).
+template <typename T, int KS, typename P = T, bool DEFAULTS = true>
+__device__ __forceinline__ void normalize_row(f32x8 (&v)[KS], const P* __restrict__ gamma,
+                                              const P* __restrict__ beta, float eps, int g,
                                               typename Vec8<T>::type (&out)[KS]) {
-  const T* gp = (gamma ? gamma : default_gamma<T>()) + 8 * g;
-  const T* bp = (beta ? beta : default_beta<T>()) + 8 * g;
+  const P* gp = (DEFAULTS && !gamma ? default_gamma<P>() : gamma) + 8 * g;
+  const P* bp = (DEFAULTS && !beta ? default_beta<P>() : beta) + 8 * g;
   float s = 0.0f;
 #pragma unroll
   for (int kk = 0; kk < KS; ++kk)
@@ -81,7 +83,7 @@ __device__ __forceinline__ void normalize_row(f32x8 (&v)[KS], const T* __restric
 #pragma unroll
   for (int kk = 0; kk < KS; ++kk) {
     // (no branch around these loads, so the compiler may issue them as early as registers allow)
-    const f32x8 gmf = to_f32(load8<T>(gp + 16 * kk)), btf = to_f32(load8<T>(bp + 16 * kk));
+    const f32x8 gmf = to_f32(load8<P>(gp + 16 * kk)), btf = to_f32(load8<P>(bp + 16 * kk));
     f32x8 o;
 #pragma unroll
     for (int t = 0; t < 8; ++t) o[t] = (v[kk][t] - mean) * rstd * gmf[t] + btf[t];
@@ -91,13 +93,13 @@ __device__ __forceinline__ void normalize_row(f32x8 (&v)[KS], const T* __restric
 
 // The same LayerNorm straight from the stored fragments, converting on the fly in each of
 // its three passes: no fp32 copy of the row is kept, for callers short of registers.
-template <typename T, int KS>
+template <typename T, int KS, typename P = T, bool DEFAULTS = true>
 __device__ __forceinline__ void normalize_raw(const typename Vec8<T>::type (&raw)[KS],
-                                              const T* __restrict__ gamma,
-                                              const T* __restrict__ beta, float eps, int g,
+                                              const P* __restrict__ gamma,
+                                              const P* __restrict__ beta, float eps, int g,
                                               typename Vec8<T>::type (&out)[KS]) {
-  const T* gp = (gamma ? gamma : default_gamma<T>()) + 8 * g;
-  const T* bp = (beta ? beta : default_beta<T>()) + 8 * g;
+  const P* gp = (DEFAULTS && !gamma ? default_gamma<P>() : gamma) + 8 * g;
+  const P* bp = (DEFAULTS && !beta ? default_beta<P>() : beta) + 8 * g;
   float s = 0.0f;
 #pragma unroll
   for (int kk = 0; kk < KS; ++kk) {
@@ -122,7 +124,7 @@ __device__ __forceinline__ void normalize_raw(const typename Vec8<T>::type (&raw
 #pragma unroll
   for (int kk = 0; kk < KS; ++kk) {
     const f32x8 v = to_f32(raw[kk]);
-    const f32x8 gmf = to_f32(load8<T>(gp + 16 * kk)), btf = to_f32(load8<T>(bp + 16 * kk));
+    const f32x8 gmf = to_f32(load8<P>(gp + 16 * kk)), btf = to_f32(load8<P>(bp + 16 * kk));
     f32x8 o;
 #pragma unroll
     for (int t = 0; t < 8; ++t) o[t] = (v[t] - mean) * rstd * gmf[t] + btf[t];
@@ -132,10 +134,10 @@ __device__ __forceinline__ void normalize_raw(const typename Vec8<T>::type (&raw
 
 // Load RB row blocks whose lane rows start at element offsets off[rb] (+ 8*g added here)
 // and, if LN, normalise them.
-template <typename T, int RB, bool LN, int KS>
+template <typename T, int RB, bool LN, int KS, typename P = T, bool DEFAULTS = true>
 __device__ __forceinline__ void load_rows_at(RowFrags<T, RB, KS>& out, const T* __restrict__ x,
-                                             const int64_t (&off)[RB], const T* __restrict__ gamma,
-                                             const T* __restrict__ beta, float eps, int lane) {
+                                             const int64_t (&off)[RB], const P* __restrict__ gamma,
+                                             const P* __restrict__ beta, float eps, int lane) {
   const int g = lane >> 5;
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
@@ -147,17 +149,17 @@ __device__ __forceinline__ void load_rows_at(RowFrags<T, RB, KS>& out, const T* 
       f32x8 v[KS];
 #pragma unroll
       for (int kk = 0; kk < KS; ++kk) v[kk] = to_f32(load8<T>(rp + 16 * kk));
-      normalize_row<T>(v, gamma, beta, eps, g, out.f[rb]);
+      normalize_row<T, KS, P, DEFAULTS>(v, gamma, beta, eps, g, out.f[rb]);
     }
   }
 }
 
 // Load RB*32 consecutive logical rows starting at row0 (rows >= n_rows re-read the last
 // valid row; their results are never stored).
-template <typename T, int RB, bool LN, int KS>
+template <typename T, int RB, bool LN, int KS, typename P = T, bool DEFAULTS = true>
 __device__ __forceinline__ void load_rows(RowFrags<T, RB, KS>& out, const T* __restrict__ x,
                                           const RowMap& map, int64_t row0, int64_t n_rows,
-                                          const T* __restrict__ gamma, const T* __restrict__ beta,
+                                          const P* __restrict__ gamma, const P* __restrict__ beta,
                                           float eps, int lane) {
   int64_t off[RB];
 #pragma unroll
@@ -166,7 +168,7 @@ __device__ __forceinline__ void load_rows(RowFrags<T, RB, KS>& out, const T* __r
     p = p < n_rows ? p : n_rows - 1;
     off[rb] = map(p);
   }
-  load_rows_at<T, RB, LN, KS>(out, x, off, gamma, beta, eps, lane);
+  load_rows_at<T, RB, LN, KS, P, DEFAULTS>(out, x, off, gamma, beta, eps, lane);
 }
 
 // One weight fragment: 32 output columns x 16 K values, lane -> (column l%32,
