@@ -131,7 +131,10 @@ template <typename T, int MODE, int KS> struct InCfg {
   static constexpr int MIN_WG = (RES || KS > 8) ? 1 : 2;
 };
 
-template <typename T, int RB, int MODE, int KS>
+// VEC: n is a multiple of the 16-byte vector length, so channel-major vectors stay inside one
+// plane row (the element-wise fallback for other n is a kernel of its own: compiled into the
+// same one, its code and its registers weigh on the path every production shape takes).
+template <typename T, int RB, int MODE, int KS, bool VEC>
 __global__ __launch_bounds__((InCfg<T, MODE, KS>::NW * 64), (InCfg<T, MODE, KS>::MIN_WG)) void
 rowgemm_in_kernel(RowGemmInParams p) {
   typedef typename Vec8<T>::type V8;
@@ -163,7 +166,7 @@ rowgemm_in_kernel(RowGemmInParams p) {
   const int n = lane & 31, g = lane >> 5;
   T* st = lds_stage[wave][0];
   auto stile = [&](int k) { return lds_stage[wave][k]; };
-  const bool vec_ok = (p.n % C::VE) == 0;   // channel-major vectors stay inside one plane row
+  constexpr bool vec_ok = VEC;
   T* const sink = reinterpret_cast<T*>(g_store_sink) + lane * C::VE;
   constexpr int nch = IC::NCH;
 
@@ -301,7 +304,7 @@ rowgemm_in_kernel(RowGemmInParams p) {
           stage_coord<T>(ps, lane, chn, r0);
           const int64_t pr = row0 + rb * 32 + r0;
           const T* src = x2 + (int64_t)(32 * cg + chn) * p.n_rows;
-          if (vec_ok) {
+          if constexpr (vec_ok) {
             const int64_t pc = pr + C::VE <= p.n_rows ? pr : 0;
             vec[cg][ps] = *reinterpret_cast<const VE_t*>(src + pc);
           } else {
@@ -620,7 +623,7 @@ rowgemm_in_kernel(RowGemmInParams p) {
               if (which == 4 && chn >= p.aux) continue;
               const VE_t v = stage_get_vec<T>(stg, chn, r0);
               T* outp = (T*)p.out[which];
-              if (vec_ok) {
+              if constexpr (vec_ok) {
                 const int64_t off = which == 3 ? h * head_plane + rel_v[rb][ps] : (int64_t)rel_b[rb][ps];
                 *reinterpret_cast<VE_t*>(cm_ok[rb] ? outp + off : sink) = v;
               } else {
@@ -739,7 +742,13 @@ int launch_rowgemm_in(const RowGemmInParams& p, hipStream_t stream) {
   if (tiles == 0) return 0;
   int64_t blocks = (tiles + 3) / 4;
   if (IC::RES) blocks = std::min<int64_t>((tiles + IC::NW - 1) / IC::NW, device_cu_count());
-  rowgemm_in_kernel<T, RB, MODE, KS><<<dim3((unsigned)blocks), dim3(IC::NW * 64), 0, stream>>>(p);
+  // (only the modes with channel-major vector stores have an element-wise variant)
+  constexpr bool kHasScalarPath = MODE == kTriAttnIn || MODE == kTriMulOut;
+  if (!kHasScalarPath || p.n % Cfg<T>::VE == 0)
+    rowgemm_in_kernel<T, RB, MODE, KS, true><<<dim3((unsigned)blocks), dim3(IC::NW * 64), 0, stream>>>(p);
+  else
+    rowgemm_in_kernel<T, RB, MODE, KS, (kHasScalarPath ? false : true)>
+        <<<dim3((unsigned)blocks), dim3(IC::NW * 64), 0, stream>>>(p);
   return 0;
 }
 
