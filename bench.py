@@ -33,7 +33,7 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on this benchmark and calibrated against a plain
 # elementwise kernel of known size (profiles/trunk_n768_bf16_hbm_traffic.txt):
 # 603780 KiB fetched + 147456 KiB written.  Algorithmic: 594432 + 147456 KiB.
-TRIATTN_FWD_TRAFFIC_BYTES_N768 = (604165 + 147461) * 1024
+TRIATTN_FWD_TRAFFIC_BYTES_N768 = (604154 + 147460) * 1024
 
 # Algorithmic work per launch at N tokens, c = 128, bf16 (2 bytes):
 #   flops for the MFMA-bound kernels, bytes for the HBM-bound ones.
