@@ -50,8 +50,10 @@ constexpr float kZeroReferenceLimit = 14.0f;
 // fit the register budget).
 #define PTX_ATTN_ROWS 1
 
-template <typename T, int R>
-__global__ __launch_bounds__(256, (sizeof(T) == 2 ? 4 : 2)) void triattn_fwd_kernel(
+// NWQ waves per workgroup (4 or 8), each with 32 queries: the workgroup's waves share the staged
+// K / V^T tiles, so with 8 every wave moves one fragment per tile instead of two.
+template <typename T, int R, int NWQ>
+__global__ __launch_bounds__((NWQ * 64), (sizeof(T) == 2 ? 16 / NWQ : 2)) void triattn_fwd_kernel(
     const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ vt,
     const T* gate, const T* __restrict__ bias, const T* __restrict__ mask,
     T* o, int n, int heads, int key_pitch, int mask_transposed, float inf,
@@ -74,7 +76,7 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? 4 : 2)) void triattn_fwd_ker
   const int i0 = (int)((item / n_qtiles) % n_rowgroups) * R;   // first of this workgroup's R rows
   const int h = (int)(item / ((int64_t)n_qtiles * n_rowgroups));
 
-  const int q0 = (qt * 4 + wave) * 32;   // first query of this wave
+  const int q0 = (qt * NWQ + wave) * 32;   // first query of this wave
   const int key_tiles = key_pitch >> 6;
   const int q_blocks = (n + 31) >> 5;
   const int n_tiles = (n + kKeyTile - 1) / kKeyTile;
@@ -109,7 +111,8 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? 4 : 2)) void triattn_fwd_ker
   // fetch() only issues loads; everything that consumes a loaded value (mask -> additive
   // bias, zeroing of V^T beyond n) happens in stash(), one tile of work later, so no wait
   // for memory sits in the issue path.
-  V8 pre[2 * R];
+  constexpr int FPW = 8 * R / NWQ;   // fragments each wave moves per tile
+  V8 pre[FPW];
   T pre_mv;
   // mask value of key kc for this wave's row: m_base[kc * m_stride] (stride 0: no mask, any
   // valid address - the value is discarded)
@@ -119,8 +122,8 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? 4 : 2)) void triattn_fwd_ker
   auto fetch = [&](int tile) {
     const int64_t atile = min(tile, n_tiles - 1);
 #pragma unroll
-    for (int j = 0; j < 2 * R; ++j) {
-      const int fid = wave * 2 * R + j;            // row = fid / 8, fragment = fid % 8
+    for (int j = 0; j < FPW; ++j) {
+      const int fid = wave * FPW + j;              // row = fid / 8, fragment = fid % 8
       const int r = fid >> 3, f = fid & 7;
       const int64_t rowtiles = ((int64_t)h * n + min(i0 + r, n - 1)) * key_tiles + atile;
       pre[j] = load8<T>((f < 4 ? k : vt) + rowtiles * kAttnTileElems + (f & 3) * 512 + lane * 8);
@@ -134,8 +137,8 @@ __global__ __launch_bounds__(256, (sizeof(T) == 2 ? 4 : 2)) void triattn_fwd_ker
     const int key0 = tile * kKeyTile;
     const bool tail = key0 + kKeyTile > n;   // uniform
 #pragma unroll
-    for (int j = 0; j < 2 * R; ++j) {
-      const int fid = wave * 2 * R + j;
+    for (int j = 0; j < FPW; ++j) {
+      const int fid = wave * FPW + j;
       const int f = fid & 7;
       V8 v = pre[j];
       if (tail && f >= 4) {
@@ -378,13 +381,22 @@ int triattn_fwd(const T* q, const T* k, const T* vt, const T* g, const T* tri_bi
                 hipStream_t stream) {
   if (n == 0) return 0;
   constexpr int R = PTX_ATTN_ROWS;
-  const int n_qtiles = (n + 127) / 128;
+  // 8-wave workgroups for long rows (measured: +2 % at n = 768, even at 1024, -2.6 % at 1536,
+  // -2.2 % at 2048), where their 256 queries divide n or n is large enough for the idle waves
+  // of the last one not to matter
+  const bool wide = sizeof(T) == 2 && ((n % 256 == 0 && n >= 1536) || n >= 2048);
+  const int n_qtiles = wide ? (n + 255) / 256 : (n + 127) / 128;
   const int n_rowgroups = (n + R - 1) / R;
   const int64_t total = (int64_t)heads * n_rowgroups * n_qtiles;
   const int64_t per_xcd = (total + 7) / 8;
-  triattn_fwd_kernel<T, R><<<dim3((unsigned)(per_xcd * 8)), dim3(256), 0, stream>>>(
-      q, k, vt, g, tri_bias, mask, o, n, heads, key_pitch, mask_transposed, inf, n_qtiles,
-      n_rowgroups, total);
+  if (wide)
+    triattn_fwd_kernel<T, R, 8><<<dim3((unsigned)(per_xcd * 8)), dim3(512), 0, stream>>>(
+        q, k, vt, g, tri_bias, mask, o, n, heads, key_pitch, mask_transposed, inf, n_qtiles,
+        n_rowgroups, total);
+  else
+    triattn_fwd_kernel<T, R, 4><<<dim3((unsigned)(per_xcd * 8)), dim3(256), 0, stream>>>(
+        q, k, vt, g, tri_bias, mask, o, n, heads, key_pitch, mask_transposed, inf, n_qtiles,
+        n_rowgroups, total);
   return 0;
 }
 
