@@ -29,6 +29,19 @@ def test_config2_triattn_start_n384_pad32():
     assert rel_err(got, want) <= TOL_BF16
 
 
+def test_triattn_n1536_pad40_wide_workgroups():
+    """From 1536 tokens on the attention core runs 8-wave workgroups (256 queries share the
+    staged key tiles): oracle parity at the smallest such size, ending node, padded."""
+    ref, prod = oracle_and_product(O.TriangleAttention, P.TriangleAttention, 128, 32, 4,
+                                   starting=False, dtype=BF16)
+    n = 1536
+    z, mask = _z(n, seed=77), pad_mask(n, 40, BF16)
+    with torch.no_grad():
+        want = ref(z.float(), mask.float(), chunk_size=32)
+        got = prod(z.cuda(), mask.cuda())
+    assert rel_err(got, want) <= TOL_BF16
+
+
 @pytest.mark.parametrize("cls", ["TriangleMultiplicationOutgoing", "TriangleMultiplicationIncoming"])
 def test_config3_trimul_n768_pad48(cls):
     """TriangleMultiplication outgoing / incoming, bf16, N = 768, 48 trailing padded tokens."""
