@@ -109,6 +109,22 @@ PTX_API int ptx_layernorm_bwd(const void* dout, const void* x, const float* mean
                       int64_t rows, int cols, int dtype, void* stream);
 
 /*
+ * ptx_layernorm_bwd without a workspace argument and without any allocation.  No counterpart
+ * in the reference; it is for callers that cannot allocate device memory (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc).  The partial sums of
+ * dgamma / dbeta live in a buffer built into the library (8 MiB per GPU, kept until the
+ * process ends), which bounds the row length: cols <= 1024, else PTX_ERR_UNSUPPORTED.  Same
+ * kernels, same summation order and therefore the same bits as ptx_layernorm_bwd.  The
+ * buffer's device address is looked up on the first call on each device (call once outside
+ * graph capture); the device of `stream` must be the current device.  All calls on one GPU
+ * share the buffer: calls that overlap there (different streams or threads) race - serialise
+ * them.  Nothing needs clearing between calls: a launch writes every partial row it reads.
+ */
+PTX_API int ptx_layernorm_bwd_static(const void* dout, const void* x, const float* mean,
+                      const float* rstd, const void* gamma, void* dx, void* dgamma, void* dbeta,
+                      int64_t rows, int cols, int dtype, void* stream);
+
+/*
  * Triangle multiplication, stage 1 (triangular.py:537-543):
  *   zn = LN(z);  a = mask * sigmoid(W_ag zn) * (W_ap zn);  b likewise,
  * written channel-major so that stage 2 is a plain batched matrix product:

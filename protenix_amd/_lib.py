@@ -32,6 +32,7 @@ SIGNATURES = {
     "ptx_layernorm_fwd": (_i, [_p, _p, _p, _p, _p, _p, _l, _i, _f, _i, _p]),
     "ptx_layernorm_bwd_workspace_elems": (_l, [_l, _i]),
     "ptx_layernorm_bwd": (_i, [_p] * 9 + [_l, _i, _i, _p]),
+    "ptx_layernorm_bwd_static": (_i, [_p] * 8 + [_l, _i, _i, _p]),
     "ptx_trimul_project": (_i, [_p] * 10 + [_i, _i, _i, _i, _i, _f, _i, _p]),
     "ptx_trimul_contract": (_i, [_p, _p, _p, _i, _i, _i, _i, _p]),
     "ptx_trimul_output": (_i, [_p] * 9 + [_i, _i, _i, _i, _f, _i, _p]),

@@ -3,6 +3,8 @@
 #include <stdarg.h>
 #include <stdio.h>
 
+#include <mutex>
+
 #include "../../include/protenix_amd.h"
 #include "common.h"
 #include "kernels.h"
@@ -47,6 +49,39 @@ bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
       CALL;                              \
     }                                    \
   } while (0)
+
+// Partial sums of ptx_layernorm_bwd_static: 2 x 1024 rows of fp32 partial column sums for rows
+// of at most kStaticLnCols columns (8 MiB per GPU, held until the process ends).  In host
+// code the array's name is only a handle; the device address comes from hipGetSymbolAddress,
+// once per device, and is what the kernels receive.
+constexpr int kStaticLnCols = 1024;
+constexpr int kStaticLnParts = 1024;   // = the most partial rows layernorm_bwd ever writes
+constexpr int kMaxDevices = 64;
+static __device__ __align__(256) float scratch[2 * kStaticLnParts * kStaticLnCols];
+float* g_scratch_ptr[kMaxDevices] = {};
+std::mutex g_scratch_lock;
+
+// Device address of `scratch` on the current device (nullptr + error text on failure).
+float* scratch_on_current_device() {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    fail(PTX_ERR_LAUNCH, "layernorm_bwd_static: hipGetDevice: %s (device %d)",
+         hipGetErrorString(e), dev);
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> hold(g_scratch_lock);
+  if (!g_scratch_ptr[dev]) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p) {
+      fail(PTX_ERR_LAUNCH, "layernorm_bwd_static: hipGetSymbolAddress: %s", hipGetErrorString(e));
+      return nullptr;
+    }
+    g_scratch_ptr[dev] = (float*)p;
+  }
+  return g_scratch_ptr[dev];
+}
 
 }  // namespace
 
@@ -105,6 +140,25 @@ PTX_API int ptx_layernorm_bwd(const void* dout, const void* x, const float* mean
                                             (const T*)gamma, (T*)dx, (T*)dgamma, (T*)dbeta,
                                             workspace, rows, cols, (hipStream_t)stream));
   return after_launch("layernorm_bwd");
+}
+
+PTX_API int ptx_layernorm_bwd_static(const void* dout, const void* x, const float* mean,
+                                     const float* rstd, const void* gamma, void* dx, void* dgamma,
+                                     void* dbeta, int64_t rows, int cols, int dtype, void* stream) {
+  PTX_REQUIRE(cols <= kStaticLnCols, PTX_ERR_UNSUPPORTED,
+              "layernorm_bwd_static: cols=%d exceeds the built-in scratch (%d columns at most); "
+              "use ptx_layernorm_bwd with a workspace",
+              cols, kStaticLnCols);
+  PTX_REQUIRE(cols > 0 && ptx::layernorm_bwd_workspace_elems(1, cols) <=
+                              (int64_t)2 * kStaticLnParts * kStaticLnCols,
+              PTX_ERR_BAD_ARG, "layernorm_bwd_static: cols=%d", cols);
+  float* ws = nullptr;
+  if (dgamma || dbeta) {
+    ws = scratch_on_current_device();
+    if (!ws) return PTX_ERR_LAUNCH;
+  }
+  return ptx_layernorm_bwd(dout, x, mean, rstd, gamma, dx, dgamma, dbeta, ws, rows, cols, dtype,
+                           stream);
 }
 
 // Pair-row widths the kernels are built for: c_z = 64 or 128 with hidden widths (c_hidden,
