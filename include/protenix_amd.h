@@ -34,10 +34,21 @@
 extern "C" {
 #endif
 
-#define PTX_ABI_VERSION 1
+#define PTX_ABI_VERSION 2
 #define PTX_API __attribute__((visibility("default")))
 
-enum ptx_dtype { PTX_F32 = 0, PTX_BF16 = 1 };
+/*
+ * PTX_MIXED: bf16 arithmetic on an fp32 residual stream, the way the reference runs
+ * inference (fp32 parameters and activations under torch.autocast(bfloat16),
+ * runner/inference.py:214-234): the pair tensor the call reads (z, x of the transition) and
+ * the `out` it adds its update to are fp32; weights, masks, workspaces and every other tensor
+ * are bf16.  Rows are normalised in fp32 and rounded to bf16 for the matrix products; the
+ * update is rounded to bf16 and added to the fp32 row.  Accepted by the entry points that
+ * touch the residual stream (rows of 64 or 128 channels); the others (ptx_trimul_contract,
+ * ptx_triattn_fwd, ptx_transition_pack) treat it as PTX_BF16, so one code serves a whole
+ * update; the LayerNorm entry points refuse it.
+ */
+enum ptx_dtype { PTX_F32 = 0, PTX_BF16 = 1, PTX_MIXED = 2 };
 
 enum ptx_status {
   PTX_OK = 0,

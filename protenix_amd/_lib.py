@@ -13,8 +13,8 @@ import threading
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libprotenix_amd.so")
 
-PTX_F32, PTX_BF16 = 0, 1
-ABI_VERSION = 1
+PTX_F32, PTX_BF16, PTX_MIXED = 0, 1, 2
+ABI_VERSION = 2
 
 _p = ctypes.c_void_p
 _i = ctypes.c_int

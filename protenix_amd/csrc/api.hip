@@ -29,6 +29,8 @@ int after_launch(const char* what) {
 }
 
 bool dtype_ok(int dtype) { return dtype == PTX_F32 || dtype == PTX_BF16; }
+// entry points that read or write the residual stream also take PTX_MIXED
+bool dtype_ok_z(int dtype) { return dtype_ok(dtype) || dtype == PTX_MIXED; }
 
 size_t esize(int dtype) { return dtype == PTX_BF16 ? 2 : 4; }
 
@@ -82,6 +84,24 @@ float* scratch_on_current_device() {
   }
   return g_scratch_ptr[dev];
 }
+
+// T = arithmetic type, TZ = storage type of the residual stream (see PTX_MIXED)
+#define PTX_DISPATCH_Z(dtype, CALL)      \
+  do {                                   \
+    if ((dtype) == PTX_BF16) {           \
+      typedef ptx::bf16_t T;             \
+      typedef ptx::bf16_t TZ;            \
+      CALL;                              \
+    } else if ((dtype) == PTX_MIXED) {   \
+      typedef ptx::bf16_t T;             \
+      typedef float TZ;                  \
+      CALL;                              \
+    } else {                             \
+      typedef float T;                   \
+      typedef float TZ;                  \
+      CALL;                              \
+    }                                    \
+  } while (0)
 
 }  // namespace
 
@@ -165,7 +185,7 @@ PTX_API int ptx_layernorm_bwd_static(const void* dout, const void* x, const floa
 // heads * 32) of 128, or c_z = 256 in bf16 with hidden widths of 256.
 static bool pair_width_ok(int c_z, int hidden, int dtype) {
   if (c_z == 64 || c_z == 128) return hidden == 128;
-  return c_z == 256 && hidden == 256 && dtype == PTX_BF16;
+  return c_z == 256 && hidden == 256 && dtype == PTX_BF16;   // (not PTX_MIXED)
 }
 static const char* const kWidthMsg =
     "only c_z = 64 / 128 with hidden width 128, or c_z = 256 with hidden width 256 in bf16, is built";
@@ -174,7 +194,7 @@ PTX_API int ptx_trimul_project(const void* z, const void* mask, const void* ln_w
                        const void* w_ap, const void* w_ag, const void* w_bp, const void* w_bg,
                        void* a, void* b, int n, int c_z, int c_hidden, int k_pitch, int incoming,
                        float eps, int dtype, void* stream) {
-  PTX_REQUIRE(dtype_ok(dtype), PTX_ERR_BAD_ARG, "trimul_project: unknown dtype %d", dtype);
+  PTX_REQUIRE(dtype_ok_z(dtype), PTX_ERR_BAD_ARG, "trimul_project: unknown dtype %d", dtype);
   PTX_REQUIRE(n >= 0, PTX_ERR_BAD_ARG, "trimul_project: n=%d", n);
   PTX_REQUIRE(pair_width_ok(c_z, c_hidden, dtype), PTX_ERR_UNSUPPORTED,
               "trimul_project: %s (got c_z=%d c_hidden=%d)", kWidthMsg, c_z, c_hidden);
@@ -189,13 +209,14 @@ PTX_API int ptx_trimul_project(const void* z, const void* mask, const void* ln_w
                   aligned16(w_bg) && aligned16(a) && aligned16(b) && (!ln_w || aligned16(ln_w)) &&
                   (!ln_b || aligned16(ln_b)),
               PTX_ERR_BAD_ARG, "trimul_project: pointers must be 16-byte aligned");
-  PTX_DISPATCH(dtype, ptx::trimul_project<T>(z, mask, ln_w, ln_b, w_ap, w_ag, w_bp, w_bg, a, b, n,
+  PTX_DISPATCH_Z(dtype, (ptx::trimul_project<T, TZ>)(z, mask, ln_w, ln_b, w_ap, w_ag, w_bp, w_bg, a, b, n,
                                              c_z, k_pitch, incoming, eps, (hipStream_t)stream));
   return after_launch("trimul_project");
 }
 
 PTX_API int ptx_trimul_contract(const void* a, const void* b, void* x, int n, int c, int k_pitch, int dtype,
                         void* stream) {
+  if (dtype == PTX_MIXED) dtype = PTX_BF16;   // no residual-stream tensor here
   PTX_REQUIRE(dtype_ok(dtype), PTX_ERR_BAD_ARG, "trimul_contract: unknown dtype %d", dtype);
   PTX_REQUIRE(n >= 0 && c >= 0, PTX_ERR_BAD_ARG, "trimul_contract: n=%d c=%d", n, c);
   PTX_REQUIRE(k_pitch == ptx_key_pitch(n), PTX_ERR_BAD_ARG,
@@ -214,7 +235,7 @@ PTX_API int ptx_trimul_output(const void* x, const void* z, const void* ln_in_w,
                       const void* ln_out_w, const void* ln_out_b, const void* w_z,
                       const void* w_g, void* out, int n, int c_z, int c_hidden, int add_residual,
                       float eps, int dtype, void* stream) {
-  PTX_REQUIRE(dtype_ok(dtype), PTX_ERR_BAD_ARG, "trimul_output: unknown dtype %d", dtype);
+  PTX_REQUIRE(dtype_ok_z(dtype), PTX_ERR_BAD_ARG, "trimul_output: unknown dtype %d", dtype);
   PTX_REQUIRE(n >= 0, PTX_ERR_BAD_ARG, "trimul_output: n=%d", n);
   PTX_REQUIRE(pair_width_ok(c_z, c_hidden, dtype), PTX_ERR_UNSUPPORTED,
               "trimul_output: %s (got c_z=%d c_hidden=%d)", kWidthMsg, c_z, c_hidden);
@@ -227,7 +248,7 @@ PTX_API int ptx_trimul_output(const void* x, const void* z, const void* ln_in_w,
                   (!ln_in_w || aligned16(ln_in_w)) &&
                   (!ln_in_b || aligned16(ln_in_b)),
               PTX_ERR_BAD_ARG, "trimul_output: pointers must be 16-byte aligned");
-  PTX_DISPATCH(dtype, ptx::trimul_output<T>(x, z, ln_in_w, ln_in_b, ln_out_w, ln_out_b, w_z, w_g,
+  PTX_DISPATCH_Z(dtype, (ptx::trimul_output<T, TZ>)(x, z, ln_in_w, ln_in_b, ln_out_w, ln_out_b, w_z, w_g,
                                             out, n, c_z, add_residual, eps, (hipStream_t)stream));
   return after_launch("trimul_output");
 }
@@ -237,7 +258,7 @@ PTX_API int ptx_triattn_project(const void* z, const void* ln_w, const void* ln_
                         void* q, void* k, void* vt, void* g, void* tri_bias, int n, int c_in,
                         int heads, int d, int key_pitch, int transposed, float eps, int dtype,
                         void* stream) {
-  PTX_REQUIRE(dtype_ok(dtype), PTX_ERR_BAD_ARG, "triattn_project: unknown dtype %d", dtype);
+  PTX_REQUIRE(dtype_ok_z(dtype), PTX_ERR_BAD_ARG, "triattn_project: unknown dtype %d", dtype);
   PTX_REQUIRE(n >= 0, PTX_ERR_BAD_ARG, "triattn_project: n=%d", n);
   PTX_REQUIRE(d == 32 && heads > 0 && heads <= 8 && pair_width_ok(c_in, heads * 32, dtype),
               PTX_ERR_UNSUPPORTED, "triattn_project: %s, head dim 32 (got c_in=%d heads=%d d=%d)",
@@ -254,7 +275,7 @@ PTX_API int ptx_triattn_project(const void* z, const void* ln_w, const void* ln_
                   (!ln_w || aligned16(ln_w)) &&
                   (!ln_b || aligned16(ln_b)),
               PTX_ERR_BAD_ARG, "triattn_project: pointers must be 16-byte aligned");
-  PTX_DISPATCH(dtype, ptx::triattn_project<T>(z, ln_w, ln_b, w_q, w_k, w_v, w_g, w_b, q, k, vt, g,
+  PTX_DISPATCH_Z(dtype, (ptx::triattn_project<T, TZ>)(z, ln_w, ln_b, w_q, w_k, w_v, w_g, w_b, q, k, vt, g,
                                               tri_bias, n, c_in, heads, d, key_pitch, transposed, eps,
                                               (hipStream_t)stream));
   return after_launch("triattn_project");
@@ -263,6 +284,7 @@ PTX_API int ptx_triattn_project(const void* z, const void* ln_w, const void* ln_
 PTX_API int ptx_triattn_fwd(const void* q, const void* k, const void* vt, const void* g,
                     const void* tri_bias, const void* mask, void* o, int n, int heads, int d,
                     int key_pitch, int mask_transposed, float inf, int dtype, void* stream) {
+  if (dtype == PTX_MIXED) dtype = PTX_BF16;   // no residual-stream tensor here
   PTX_REQUIRE(dtype_ok(dtype), PTX_ERR_BAD_ARG, "triattn_fwd: unknown dtype %d", dtype);
   PTX_REQUIRE(n >= 0 && heads >= 0, PTX_ERR_BAD_ARG, "triattn_fwd: n=%d heads=%d", n, heads);
   PTX_REQUIRE(d == 32, PTX_ERR_UNSUPPORTED, "triattn_fwd: only head dim 32 is built (got %d)", d);
@@ -282,7 +304,7 @@ PTX_API int ptx_triattn_fwd(const void* q, const void* k, const void* vt, const 
 
 PTX_API int ptx_triattn_output(const void* o, const void* w_o, const void* z, void* out, int n, int c_in,
                        int transposed, int add_residual, int dtype, void* stream) {
-  PTX_REQUIRE(dtype_ok(dtype), PTX_ERR_BAD_ARG, "triattn_output: unknown dtype %d", dtype);
+  PTX_REQUIRE(dtype_ok_z(dtype), PTX_ERR_BAD_ARG, "triattn_output: unknown dtype %d", dtype);
   PTX_REQUIRE(n >= 0, PTX_ERR_BAD_ARG, "triattn_output: n=%d", n);
   PTX_REQUIRE(pair_width_ok(c_in, c_in == 256 ? 256 : 128, dtype), PTX_ERR_UNSUPPORTED,
               "triattn_output: %s (got c_in=%d)", kWidthMsg, c_in);
@@ -293,7 +315,7 @@ PTX_API int ptx_triattn_output(const void* o, const void* w_o, const void* z, vo
   PTX_REQUIRE(aligned16(o) && aligned16(w_o) && aligned16(out) && (!z || aligned16(z)),
               PTX_ERR_BAD_ARG,
               "triattn_output: pointers must be 16-byte aligned");
-  PTX_DISPATCH(dtype, ptx::triattn_output<T>(o, w_o, z, out, n, c_in, transposed, add_residual,
+  PTX_DISPATCH_Z(dtype, (ptx::triattn_output<T, TZ>)(o, w_o, z, out, n, c_in, transposed, add_residual,
                                              (hipStream_t)stream));
   return after_launch("triattn_output");
 }
@@ -305,6 +327,7 @@ PTX_API int64_t ptx_transition_packed_elems(int c, int n_factor) {
 
 PTX_API int ptx_transition_pack(const void* w_a, const void* w_b, const void* w_o, void* packed, int c,
                         int n_factor, int dtype, void* stream) {
+  if (dtype == PTX_MIXED) dtype = PTX_BF16;   // no residual-stream tensor here
   PTX_REQUIRE(dtype_ok(dtype), PTX_ERR_BAD_ARG, "transition_pack: unknown dtype %d", dtype);
   PTX_REQUIRE(n_factor > 0, PTX_ERR_BAD_ARG, "transition_pack: n_factor=%d", n_factor);
   PTX_REQUIRE(c == 128 || c == 64 || (c == 256 && dtype == PTX_BF16), PTX_ERR_UNSUPPORTED,
@@ -323,11 +346,11 @@ PTX_API int ptx_transition_pack(const void* w_a, const void* w_b, const void* w_
 PTX_API int ptx_transition_fwd(const void* x, const void* ln_w, const void* ln_b, const void* packed,
                        void* out, int64_t rows, int c, int n_factor, int add_residual, float eps,
                        int dtype, void* stream) {
-  PTX_REQUIRE(dtype_ok(dtype), PTX_ERR_BAD_ARG, "transition: unknown dtype %d", dtype);
+  PTX_REQUIRE(dtype_ok_z(dtype), PTX_ERR_BAD_ARG, "transition: unknown dtype %d", dtype);
   PTX_REQUIRE(rows >= 0 && n_factor > 0, PTX_ERR_BAD_ARG, "transition: rows=%lld n_factor=%d",
               (long long)rows, n_factor);
   PTX_REQUIRE(c == 128 || c == 64 || (c == 256 && dtype == PTX_BF16), PTX_ERR_UNSUPPORTED,
-              "transition: only c = 64, 128, or 256 in bf16, is built (got %d)", c);
+              "transition: only c = 64, 128, or 256 in bf16 (not mixed), is built (got %d)", c);
   PTX_REQUIRE((n_factor * c) % 64 == 0, PTX_ERR_UNSUPPORTED,
               "transition: the hidden width %d is not a multiple of 64", n_factor * c);
   PTX_REQUIRE(n_factor <= 64, PTX_ERR_UNSUPPORTED, "transition: n_factor=%d too large", n_factor);
@@ -338,7 +361,7 @@ PTX_API int ptx_transition_fwd(const void* x, const void* ln_w, const void* ln_b
   PTX_REQUIRE(aligned16(x) && aligned16(packed) && aligned16(out) && (!ln_w || aligned16(ln_w)) &&
                   (!ln_b || aligned16(ln_b)),
               PTX_ERR_BAD_ARG, "transition: pointers must be 16-byte aligned");
-  PTX_DISPATCH(dtype, ptx::transition_fwd<T>(x, ln_w, ln_b, packed, out, rows, c, n_factor,
+  PTX_DISPATCH_Z(dtype, (ptx::transition_fwd<T, TZ>)(x, ln_w, ln_b, packed, out, rows, c, n_factor,
                                              add_residual, eps, (hipStream_t)stream));
   return after_launch("transition");
 }
@@ -346,7 +369,7 @@ PTX_API int ptx_transition_fwd(const void* x, const void* ln_w, const void* ln_b
 PTX_API int ptx_pair_bias_fwd(const void* z, const void* ln_w, const void* ln_b, const void* w, void* bias,
                       int n, int c_z, int heads, int out_f32, float eps, int dtype,
                       void* stream) {
-  PTX_REQUIRE(dtype_ok(dtype), PTX_ERR_BAD_ARG, "pair_bias: unknown dtype %d", dtype);
+  PTX_REQUIRE(dtype_ok_z(dtype), PTX_ERR_BAD_ARG, "pair_bias: unknown dtype %d", dtype);
   PTX_REQUIRE(n >= 0, PTX_ERR_BAD_ARG, "pair_bias: n=%d", n);
   PTX_REQUIRE(c_z == 128 || (c_z == 256 && dtype == PTX_BF16), PTX_ERR_UNSUPPORTED,
               "pair_bias: only c_z = 128, or 256 in bf16, is built (got %d)", c_z);
@@ -358,7 +381,7 @@ PTX_API int ptx_pair_bias_fwd(const void* z, const void* ln_w, const void* ln_b,
   PTX_REQUIRE(aligned16(z) && aligned16(w) && aligned16(bias) && (!ln_w || aligned16(ln_w)) &&
                   (!ln_b || aligned16(ln_b)),
               PTX_ERR_BAD_ARG, "pair_bias: pointers must be 16-byte aligned");
-  PTX_DISPATCH(dtype, ptx::pair_bias_fwd<T>(z, ln_w, ln_b, w, bias, n, c_z, heads, out_f32, eps,
+  PTX_DISPATCH_Z(dtype, (ptx::pair_bias_fwd<T, TZ>)(z, ln_w, ln_b, w, bias, n, c_z, heads, out_f32, eps,
                                             (hipStream_t)stream));
   return after_launch("pair_bias");
 }

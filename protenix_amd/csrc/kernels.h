@@ -7,6 +7,9 @@
 
 namespace ptx {
 
+// T: arithmetic / weight / workspace type.  TZ (where present): storage type of the pair
+// tensor rows the kernel reads (z, x) and of the residual stream it writes (out): T, or float
+// with T = bf16 (the fp32 residual stream of autocast inference; rows of 64 or 128 channels).
 template <typename T>
 int layernorm_fwd(const T* x, const T* gamma, const T* beta, T* y, float* mean, float* rstd,
                   int64_t rows, int cols, float eps, hipStream_t stream);
@@ -18,32 +21,32 @@ int layernorm_bwd(const T* dout, const T* x, const float* mean, const float* rst
                   T* dx, T* dgamma, T* dbeta, float* workspace, int64_t rows, int cols,
                   hipStream_t stream);
 
-template <typename T>
+template <typename T, typename TZ = T>
 int trimul_project(const void* z, const void* mask, const void* ln_w, const void* ln_b,
                    const void* w_ap, const void* w_ag, const void* w_bp, const void* w_bg, void* a,
                    void* b, int n, int c_z, int k_pitch, int incoming, float eps,
                    hipStream_t stream);
-template <typename T>
+template <typename T, typename TZ = T>
 int trimul_output(const void* x, const void* z, const void* ln_in_w, const void* ln_in_b,
                   const void* ln_out_w, const void* ln_out_b, const void* w_z, const void* w_g,
                   void* out, int n, int c_z, int add_residual, float eps, hipStream_t stream);
-template <typename T>
+template <typename T, typename TZ = T>
 int triattn_project(const void* z, const void* ln_w, const void* ln_b, const void* w_q,
                     const void* w_k, const void* w_v, const void* w_g, const void* w_b, void* q,
                     void* k, void* vt, void* g, void* tri_bias, int n, int c_z, int heads, int d,
                     int key_pitch, int transposed, float eps, hipStream_t stream);
-template <typename T>
+template <typename T, typename TZ = T>
 int triattn_output(const void* o, const void* w_o, const void* z, void* out, int n, int c_z,
                    int transposed, int add_residual, hipStream_t stream);
 // transition weights -> fragment-ordered chunks of 32 hidden (3 * n_factor*c * c elements)
 template <typename T>
 int transition_pack(const void* w_a, const void* w_b, const void* w_o, void* packed, int c,
                     int n_factor, hipStream_t stream);
-template <typename T>
+template <typename T, typename TZ = T>
 int transition_fwd(const void* x, const void* ln_w, const void* ln_b, const void* packed,
                    void* out, int64_t rows, int c, int n_factor, int add_residual, float eps,
                    hipStream_t stream);
-template <typename T>
+template <typename T, typename TZ = T>
 int pair_bias_fwd(const void* z, const void* ln_w, const void* ln_b, const void* w, void* bias,
                   int n, int c_z, int heads, int out_f32, float eps, hipStream_t stream);
 

@@ -134,13 +134,23 @@ template <typename T, int MODE, int KS> struct InCfg {
 // VEC: n is a multiple of the 16-byte vector length, so channel-major vectors stay inside one
 // plane row (the element-wise fallback for other n is a kernel of its own: compiled into the
 // same one, its code and its registers weigh on the path every production shape takes).
-template <typename T, int RB, int MODE, int KS, bool VEC>
+// TZ: storage type of the pair tensor (p.x and, for kTriMulOut, the output).  TZ = float with
+// T = bf16 is the fp32 residual stream of the reference's autocast inference: rows are read
+// as fp32, normalised in fp32 and rounded to T for the matrix products; kTriMulOut adds its
+// T-rounded update to the fp32 row.
+template <typename T, int RB, int MODE, int KS, bool VEC, typename TZ = T>
 __global__ __launch_bounds__((InCfg<T, MODE, KS>::NW * 64), (InCfg<T, MODE, KS>::MIN_WG)) void
 rowgemm_in_kernel(RowGemmInParams p) {
   typedef typename Vec8<T>::type V8;
   typedef typename VecE<T>::type VE_t;
   typedef Cfg<T> C;
+  typedef Cfg<TZ> CZ;
   typedef InCfg<T, MODE, KS> IC;
+  constexpr bool MIXED = !std::is_same<T, TZ>::value;
+  static_assert(!MIXED || (sizeof(T) == 2 && sizeof(TZ) == 4 && KS <= 8),
+                "mixed storage: bf16 arithmetic on fp32 rows of at most 128 channels");
+  // kTriMulOut on an fp32 residual stream keeps the raw rows in registers (see below)
+  constexpr bool kRegRes = MIXED && MODE == kTriMulOut;
   constexpr bool RES = IC::RES;
   constexpr int NW = IC::NW, SL = IC::SL, FPW = IC::FPW;
   __shared__ V8 lds_w[IC::NFRAG][kWave];
@@ -152,7 +162,10 @@ rowgemm_in_kernel(RowGemmInParams p) {
   // HBM at the end costs a full extra pass: by then they have left the L2)
   constexpr int kCz = 16 * KS;   // channels of a pair-tensor row
   constexpr int kResPitch = kCz + 16 / (int)sizeof(T);
-  __shared__ __attribute__((aligned(16))) T lds_res[MODE == kTriMulOut ? NW : 1][MODE == kTriMulOut ? RB * 32 : 1][kResPitch];
+  constexpr bool kLdsRes = MODE == kTriMulOut && !kRegRes;
+  __shared__ __attribute__((aligned(16))) T lds_res[kLdsRes ? NW : 1][kLdsRes ? RB * 32 : 1][kLdsRes ? kResPitch : 8];
+  // kRegRes: staging tile of the fp32 output rows (one 32 x 32 tile per wave)
+  __shared__ __attribute__((aligned(16))) TZ lds_stage_z[kRegRes ? NW : 1][kRegRes ? 32 * CZ::PITCH : 4];
   __shared__ __attribute__((aligned(16))) T lds_stage[NW][NST][32 * C::PITCH];
   __shared__ __attribute__((aligned(16))) float lds_mask[MODE == kTriMulIn ? NW : 1][RB * 32];
   // LayerNorm weight and bias (absent: 1 and 0) as fp32, converted once per workgroup: read
@@ -202,7 +215,12 @@ rowgemm_in_kernel(RowGemmInParams p) {
     const int kk = f_src % SL;
     chunk_tile<T, MODE, KS>(p, f_src / (2 * SL), (f_src / SL) & 1, w, n_out, col0, ldw, ksteps);
     if (kk >= ksteps) return;   // narrow rows: the slot stays unused
-    const int col = min(col0 + (lane & 31), n_out - 1);   // as load_wfrag
+    // kRegRes: output column of MFMA row m is permuted so that the accumulator registers of
+    // a lane cover the same 8-channel runs as its fragments of the z row: register r of
+    // half-wave g <-> column 16*(r>>3) + 8*g + (r&7) of the chunk's 32
+    int m = lane & 31;
+    if constexpr (kRegRes) m = 16 * (m >> 4) + 8 * ((m >> 2) & 1) + 4 * ((m >> 3) & 1) + (m & 3);
+    const int col = min(col0 + m, n_out - 1);   // as load_wfrag
     load_to_lds16(w + (int64_t)col * ldw + kk * 16 + 8 * (lane >> 5),
                   lds_address(&lds_w[f_dst][0]));
   };
@@ -258,6 +276,7 @@ rowgemm_in_kernel(RowGemmInParams p) {
     if constexpr (RES) asm volatile("" : "+s"(gamma), "+s"(beta), "+s"(gamma2), "+s"(beta2));
 
   RowFrags<T, RB, KS> xf;
+  f32x8 zres[kRegRes ? RB : 1][kRegRes ? KS : 1];
   if constexpr (MODE == kTriMulIn) {
     int64_t off[RB];
 #pragma unroll
@@ -265,7 +284,20 @@ rowgemm_in_kernel(RowGemmInParams p) {
       const int i = min(pi0 + 4 * rb + (n >> 3), p.n - 1), k = min(pk0 + (n & 7), p.n - 1);
       off[rb] = (int64_t)i * p.xmap.stride_outer + (int64_t)k * p.xmap.stride_inner;
     }
-    load_rows_at<T, RB, true>(xf, (const T*)p.x, off, gamma, beta, p.eps, lane);
+    load_rows_at<T, RB, true>(xf, (const TZ*)p.x, off, gamma, beta, p.eps, lane);
+  } else if constexpr (kRegRes) {
+    // raw fp32 rows stay in registers for the residual add: lane (row n, half g) holds
+    // channels 16*kk + 8*g .. +7, which the permuted weight columns make the very channels
+    // its accumulator registers stand for
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) {
+      int64_t pr = row0 + rb * 32 + n;
+      pr = pr < p.n_rows ? pr : p.n_rows - 1;
+      const TZ* rp = (const TZ*)p.x + p.xmap(pr) + 8 * g;
+#pragma unroll
+      for (int kk = 0; kk < KS; ++kk) zres[rb][kk] = load8<TZ>(rp + 16 * kk);
+      normalize_row<T, KS>(zres[rb], gamma, beta, p.eps, g, xf.f[rb]);
+    }
   } else if constexpr (MODE == kTriMulOut) {
     RowFrags<T, RB, KS> zraw;
     load_rows<T, RB, false>(zraw, (const T*)p.x, p.xmap, row0, p.n_rows, (const T*)nullptr,
@@ -280,10 +312,10 @@ rowgemm_in_kernel(RowGemmInParams p) {
     }
   } else {
     if constexpr (kLdsAffine)
-      load_rows<T, RB, true, KS, float, false>(xf, (const T*)p.x, p.xmap, row0, p.n_rows, lds_affine[0],
+      load_rows<T, RB, true, KS, float, false>(xf, (const TZ*)p.x, p.xmap, row0, p.n_rows, lds_affine[0],
                                                lds_affine[1], p.eps, lane);
     else
-      load_rows<T, RB, true>(xf, (const T*)p.x, p.xmap, row0, p.n_rows, gamma, beta, p.eps, lane);
+      load_rows<T, RB, true>(xf, (const TZ*)p.x, p.xmap, row0, p.n_rows, gamma, beta, p.eps, lane);
   }
 
   // kTriMulOut: second fragment set = LayerNorm_out of the channel-major triangle product,
@@ -369,6 +401,19 @@ rowgemm_in_kernel(RowGemmInParams p) {
       rm_i[rb][ps] = pc / (uint32_t)p.n;
       rm_j[rb][ps] = pc - rm_i[rb][ps] * (uint32_t)p.n;
     }
+  // kRegRes: the rows this lane stores in the read-back passes of the fp32 staging tile
+  int64_t rrow_z[kRegRes ? RB : 1][kRegRes ? CZ::NPASS : 1];
+  if constexpr (kRegRes) {
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+      for (int ps = 0; ps < CZ::NPASS; ++ps) {
+        int mj, m0;
+        stage_coord<TZ>(ps, lane, mj, m0);
+        const int64_t pr = row0 + rb * 32 + mj;
+        rrow_z[rb][ps] = pr < p.n_rows ? pr : -1;
+      }
+  }
   // Channel-major destinations: the VE consecutive logical rows this lane stores (the same
   // in every read-back pass), as (outer, inner) of the pair tensor; all address divisions
   // happen here, once, outside the chunk loop.
@@ -434,9 +479,9 @@ rowgemm_in_kernel(RowGemmInParams p) {
       *reinterpret_cast<VE_t*>(rrow[rb][ps] >= 0 ? outp + off : sink) = v;
     }
   };
-  // (not unrolled: unrolled, the compiler hoists every chunk's loads to the top and spills them)
-#pragma clang loop unroll(disable)
-  for (int ch = 0; ch < nch; ++ch) {
+  // (not unrolled: unrolled, the compiler hoists every chunk's loads to the top and spills them.
+  // kRegRes indexes the register copy of the rows by chunk and has to be unrolled.)
+  auto chunk_body = [&](int ch) {
     const int buf = (!RES && C::NBUF == 2) ? (ch & 1) : 0;
     if constexpr (kDma) {
       // the other buffer was last read in the previous chunk, which every wave has left
@@ -453,7 +498,7 @@ rowgemm_in_kernel(RowGemmInParams p) {
     const int wf1 = wf0 + ((RES && MODE == kTriAttnIn && ch == nch - 1) ? 0 : SL);
     // kTriMulOut: the residual vectors of this chunk's columns, from the wave's LDS copy of z
     VE_t resv[RB][C::NPASS];
-    if constexpr (MODE == kTriMulOut) {
+    if constexpr (kLdsRes) {
 #pragma unroll
       for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
@@ -681,6 +726,39 @@ rowgemm_in_kernel(RowGemmInParams p) {
     } else {
       // kTriMulOut: out[p][col] = [z +] (W_z LN_out(x)) * sigmoid(W_g LN_in(z)), row-major.
       // out may alias z: the residual comes from the copy of z made before any store.
+      if constexpr (kRegRes) {
+        TZ* stz = lds_stage_z[wave];
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) {
+          wave_lds_sync();
+#pragma unroll
+          for (int k2 = 0; k2 < 2; ++k2) {
+            f32x8 o;
+#pragma unroll
+            for (int t = 0; t < 8; ++t) {
+              const int r = 8 * k2 + t;
+              // linear_z output rounded to T, times the gate, rounded to T: the update
+              const float u = to_f32(from_f32<T>(to_f32(from_f32<T>(acc[rb][0][r])) *
+                                                 sigmoidf_fast(acc[rb][1][r])));
+              o[t] = p.add_residual ? zres[rb][2 * ch + k2][t] + u : u;
+            }
+            // row n of the tile, columns 16*k2 + 8*g .. +7 (8-byte LDS stores)
+            f32x2* dst = reinterpret_cast<f32x2*>(stz + n * CZ::PITCH + 16 * k2 + 8 * g);
+#pragma unroll
+            for (int h2 = 0; h2 < 4; ++h2) dst[h2] = f32x2{o[2 * h2], o[2 * h2 + 1]};
+          }
+          wave_lds_sync();
+#pragma unroll
+          for (int ps = 0; ps < CZ::NPASS; ++ps) {
+            int mj, m0;
+            stage_coord<TZ>(ps, lane, mj, m0);
+            const typename VecE<TZ>::type v = stage_get_vec<TZ>(stz, mj, m0);
+            TZ* dstp = (TZ*)p.out[0] + rrow_z[rb][ps] * kCz + ch * 32 + m0;
+            *reinterpret_cast<typename VecE<TZ>::type*>(
+                rrow_z[rb][ps] >= 0 ? dstp : reinterpret_cast<TZ*>(g_store_sink) + lane * CZ::VE) = v;
+          }
+        }
+      } else {
 #pragma unroll
       for (int rb = 0; rb < RB; ++rb) {
         float vals[16];
@@ -693,6 +771,7 @@ rowgemm_in_kernel(RowGemmInParams p) {
         stage_put<T>(st, vals, lane);
         wave_lds_sync();
         store_row_major(st, (T*)p.out[0], kCz, ch * 32, rb, p.add_residual ? resv[rb] : nullptr);
+      }
       }
     }
 
@@ -713,6 +792,13 @@ rowgemm_in_kernel(RowGemmInParams p) {
       }
       __syncthreads();
     }
+  };
+  if constexpr (kRegRes) {
+#pragma unroll
+    for (int ch = 0; ch < nch; ++ch) chunk_body(ch);
+  } else {
+#pragma clang loop unroll(disable)
+    for (int ch = 0; ch < nch; ++ch) chunk_body(ch);
   }
     if (!RES) break;
     tile += tile_step;
@@ -733,7 +819,7 @@ static int device_cu_count() {
   return cache[dev];
 }
 
-template <typename T, int MODE, int KS>
+template <typename T, int MODE, int KS, typename TZ = T>
 int launch_rowgemm_in(const RowGemmInParams& p, hipStream_t stream) {
   typedef InCfg<T, MODE, KS> IC;
   constexpr int RB = (sizeof(T) == 2 && MODE != kTriMulOut && KS <= 8) ? 2 : 1;
@@ -745,9 +831,9 @@ int launch_rowgemm_in(const RowGemmInParams& p, hipStream_t stream) {
   // (only the modes with channel-major vector stores have an element-wise variant)
   constexpr bool kHasScalarPath = MODE == kTriAttnIn || MODE == kTriMulOut;
   if (!kHasScalarPath || p.n % Cfg<T>::VE == 0)
-    rowgemm_in_kernel<T, RB, MODE, KS, true><<<dim3((unsigned)blocks), dim3(IC::NW * 64), 0, stream>>>(p);
+    rowgemm_in_kernel<T, RB, MODE, KS, true, TZ><<<dim3((unsigned)blocks), dim3(IC::NW * 64), 0, stream>>>(p);
   else
-    rowgemm_in_kernel<T, RB, MODE, KS, (kHasScalarPath ? false : true)>
+    rowgemm_in_kernel<T, RB, MODE, KS, (kHasScalarPath ? false : true), TZ>
         <<<dim3((unsigned)blocks), dim3(IC::NW * 64), 0, stream>>>(p);
   return 0;
 }
@@ -768,19 +854,22 @@ struct RowGemmOutParams {
   int64_t n_rows;
 };
 
-// NOB = output column blocks of 32 (c_z / 32).
-template <typename T, int RB, int NOB>
+// NOB = output column blocks of 32 (c_z / 32).  TZ: storage type of res and out (float with
+// T = bf16: the T-rounded product is added to an fp32 residual stream).
+template <typename T, int RB, int NOB, typename TZ = T>
 __global__ __launch_bounds__(256, 2) void rowgemm_out_kernel(RowGemmOutParams p) {
   typedef typename Vec8<T>::type V8;
-  typedef typename VecE<T>::type VE_t;
-  typedef Cfg<T> C;
-  __shared__ V8 lds_w[C::NBUF][2 * kKSteps][kWave];
-  __shared__ __attribute__((aligned(16))) T lds_stage[4][32 * C::PITCH];
+  typedef typename VecE<TZ>::type VE_t;
+  typedef Cfg<T> CW;    // weight ring
+  typedef Cfg<TZ> C;    // staging tile and stores
+  constexpr bool MIXED = !std::is_same<T, TZ>::value;
+  __shared__ V8 lds_w[CW::NBUF][2 * kKSteps][kWave];
+  __shared__ __attribute__((aligned(16))) TZ lds_stage[4][32 * C::PITCH];
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int64_t row0 = ((int64_t)blockIdx.x * 4 + wave) * (RB * 32);
   const int K = kC * p.n_slab;
   const T* w = (const T*)p.w;
-  T* st = lds_stage[wave];
+  TZ* st = lds_stage[wave];
 
   f32x16 acc[RB][NOB];
 #pragma unroll
@@ -833,7 +922,7 @@ __global__ __launch_bounds__(256, 2) void rowgemm_out_kernel(RowGemmOutParams p)
 #pragma unroll
     for (int half = 0; half < NH; ++half) {
       const int ch = NH * slab + half;
-      const int buf = C::NBUF == 2 ? (ch & 1) : 0;
+      const int buf = CW::NBUF == 2 ? (ch & 1) : 0;
       fetch(min(ch + 1, nch - 1));
 #pragma unroll
       for (int kk = 0; kk < kKSteps; ++kk) {
@@ -846,8 +935,8 @@ __global__ __launch_bounds__(256, 2) void rowgemm_out_kernel(RowGemmOutParams p)
           mma32(acc[rb][2 * half + 1], w1, af.f[rb][kk]);
         }
       }
-      if (C::NBUF == 1) __syncthreads();
-      stash(C::NBUF == 2 ? (buf ^ 1) : 0);
+      if (CW::NBUF == 1) __syncthreads();
+      stash(CW::NBUF == 2 ? (buf ^ 1) : 0);
       __syncthreads();
     }
   }
@@ -855,8 +944,8 @@ __global__ __launch_bounds__(256, 2) void rowgemm_out_kernel(RowGemmOutParams p)
   // out may alias res: a lane reads the residual vectors it is about to overwrite.  They
   // are all requested up front: next to their stores each would cost a serialised memory
   // round trip, since no load can move above the previous (possibly aliasing) store.
-  T* outp = (T*)p.out;
-  const T* resp = (const T*)p.res;
+  TZ* outp = (TZ*)p.out;
+  const TZ* resp = (const TZ*)p.res;
   int64_t obase[RB][C::NPASS];
   VE_t resv[RB][NOB][C::NPASS];
 #pragma unroll
@@ -864,7 +953,7 @@ __global__ __launch_bounds__(256, 2) void rowgemm_out_kernel(RowGemmOutParams p)
 #pragma unroll
     for (int ps = 0; ps < C::NPASS; ++ps) {
       int mj, m0;
-      stage_coord<T>(ps, lane, mj, m0);
+      stage_coord<TZ>(ps, lane, mj, m0);
       const int64_t pr = row0 + rb * 32 + mj;
       obase[rb][ps] = pr < p.n_rows ? p.omap(pr) + m0 : -1;
     }
@@ -884,17 +973,18 @@ __global__ __launch_bounds__(256, 2) void rowgemm_out_kernel(RowGemmOutParams p)
     for (int t = 0; t < NOB; ++t) {
       float vals[16];
 #pragma unroll
-      for (int r = 0; r < 16; ++r) vals[r] = acc[rb][t][r];
+      for (int r = 0; r < 16; ++r)   // (mixed: the product is rounded to T before it is added)
+        vals[r] = MIXED ? to_f32(from_f32<T>(acc[rb][t][r])) : acc[rb][t][r];
       wave_lds_sync();
-      stage_put<T>(st, vals, lane);
+      stage_put<TZ>(st, vals, lane);
       wave_lds_sync();
 #pragma unroll
       for (int ps = 0; ps < C::NPASS; ++ps) {
         int mj, m0;
-        stage_coord<T>(ps, lane, mj, m0);
+        stage_coord<TZ>(ps, lane, mj, m0);
         if (obase[rb][ps] >= 0) {
-          VE_t v = stage_get_vec<T>(st, mj, m0);
-          if (resp) v = add_vec<T>(v, resv[rb][t][ps]);
+          VE_t v = stage_get_vec<TZ>(st, mj, m0);
+          if (resp) v = add_vec<TZ>(v, resv[rb][t][ps]);
           *reinterpret_cast<VE_t*>(outp + obase[rb][ps] + t * 32) = v;
         }
       }
@@ -902,13 +992,14 @@ __global__ __launch_bounds__(256, 2) void rowgemm_out_kernel(RowGemmOutParams p)
   }
 }
 
-template <typename T, int NOB>
+template <typename T, int NOB, typename TZ = T>
 int launch_rowgemm_out(const RowGemmOutParams& p, hipStream_t stream) {
-  constexpr int RB = (sizeof(T) == 2 && NOB <= 4) ? 2 : 1;
+  // (an fp32 residual stream doubles the residual vectors a lane holds: one row block then)
+  constexpr int RB = (sizeof(T) == 2 && sizeof(TZ) == 2 && NOB <= 4) ? 2 : 1;
   const int64_t rows_per_block = 4 * RB * 32;
   const int64_t blocks = (p.n_rows + rows_per_block - 1) / rows_per_block;
   if (blocks == 0) return 0;
-  rowgemm_out_kernel<T, RB, NOB><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(p);
+  rowgemm_out_kernel<T, RB, NOB, TZ><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(p);
   return 0;
 }
 
@@ -923,7 +1014,7 @@ static RowMap pair_map(int n, int c, bool transposed) {
   return m;
 }
 
-template <typename T>
+template <typename T, typename TZ>
 int trimul_project(const void* z, const void* mask, const void* ln_w, const void* ln_b,
                    const void* w_ap, const void* w_ag, const void* w_bp, const void* w_bg, void* a,
                    void* b, int n, int c_z, int k_pitch, int incoming, float eps,
@@ -941,15 +1032,15 @@ int trimul_project(const void* z, const void* mask, const void* ln_w, const void
   p.mmap = pair_map(n, 1, incoming != 0);
   p.n = n;
   p.pitch = k_pitch;
-  if (c_z == 64) return launch_rowgemm_in<T, kTriMulIn, 4>(p, stream);
+  if (c_z == 64) return launch_rowgemm_in<T, kTriMulIn, 4, TZ>(p, stream);
   if (c_z == 256) {
-    if constexpr (sizeof(T) == 2) return launch_rowgemm_in<T, kTriMulIn, 16>(p, stream);
+    if constexpr (sizeof(T) == 2 && sizeof(TZ) == 2) return launch_rowgemm_in<T, kTriMulIn, 16>(p, stream);
     else return -1;   // 256-channel rows are built for bf16 only (refused by the caller)
   }
-  return launch_rowgemm_in<T, kTriMulIn, 8>(p, stream);
+  return launch_rowgemm_in<T, kTriMulIn, 8, TZ>(p, stream);
 }
 
-template <typename T>
+template <typename T, typename TZ>
 int trimul_output(const void* x, const void* z, const void* ln_in_w, const void* ln_in_b,
                   const void* ln_out_w, const void* ln_out_b, const void* w_z, const void* w_g,
                   void* out, int n, int c_z, int add_residual, float eps, hipStream_t stream) {
@@ -967,15 +1058,15 @@ int trimul_output(const void* x, const void* z, const void* ln_in_w, const void*
   p.gamma2 = ln_out_w;
   p.beta2 = ln_out_b;
   p.add_residual = add_residual;
-  if (c_z == 64) return launch_rowgemm_in<T, kTriMulOut, 4>(p, stream);
+  if (c_z == 64) return launch_rowgemm_in<T, kTriMulOut, 4, TZ>(p, stream);
   if (c_z == 256) {
-    if constexpr (sizeof(T) == 2) return launch_rowgemm_in<T, kTriMulOut, 16>(p, stream);
+    if constexpr (sizeof(T) == 2 && sizeof(TZ) == 2) return launch_rowgemm_in<T, kTriMulOut, 16>(p, stream);
     else return -1;   // 256-channel rows are built for bf16 only (refused by the caller)
   }
-  return launch_rowgemm_in<T, kTriMulOut, 8>(p, stream);
+  return launch_rowgemm_in<T, kTriMulOut, 8, TZ>(p, stream);
 }
 
-template <typename T>
+template <typename T, typename TZ>
 int triattn_project(const void* z, const void* ln_w, const void* ln_b, const void* w_q,
                     const void* w_k, const void* w_v, const void* w_g, const void* w_b, void* q,
                     void* k, void* vt, void* g, void* tri_bias, int n, int c_z, int heads, int d,
@@ -993,15 +1084,15 @@ int triattn_project(const void* z, const void* ln_w, const void* ln_b, const voi
   p.aux = heads;
   p.pitch = key_pitch;
   p.q_scale = 1.4426950408889634f / sqrtf((float)d);   // log2(e) / sqrt(d), see triattn.hip
-  if (c_z == 64) return launch_rowgemm_in<T, kTriAttnIn, 4>(p, stream);
+  if (c_z == 64) return launch_rowgemm_in<T, kTriAttnIn, 4, TZ>(p, stream);
   if (c_z == 256) {
-    if constexpr (sizeof(T) == 2) return launch_rowgemm_in<T, kTriAttnIn, 16>(p, stream);
+    if constexpr (sizeof(T) == 2 && sizeof(TZ) == 2) return launch_rowgemm_in<T, kTriAttnIn, 16>(p, stream);
     else return -1;   // 256-channel rows are built for bf16 only (refused by the caller)
   }
-  return launch_rowgemm_in<T, kTriAttnIn, 8>(p, stream);
+  return launch_rowgemm_in<T, kTriAttnIn, 8, TZ>(p, stream);
 }
 
-template <typename T>
+template <typename T, typename TZ>
 int triattn_output(const void* o, const void* w_o, const void* z, void* out, int n, int c_z,
                    int transposed, int add_residual, hipStream_t stream) {
   RowGemmOutParams p = {};
@@ -1013,15 +1104,15 @@ int triattn_output(const void* o, const void* w_o, const void* z, void* out, int
   p.out = out;
   p.omap = pair_map(n, c_z, transposed != 0);
   p.n_rows = (int64_t)n * n;
-  if (c_z == 64) return launch_rowgemm_out<T, 2>(p, stream);
+  if (c_z == 64) return launch_rowgemm_out<T, 2, TZ>(p, stream);
   if (c_z == 256) {
-    if constexpr (sizeof(T) == 2) return launch_rowgemm_out<T, 8>(p, stream);
+    if constexpr (sizeof(T) == 2 && sizeof(TZ) == 2) return launch_rowgemm_out<T, 8>(p, stream);
     else return -1;
   }
-  return launch_rowgemm_out<T, 4>(p, stream);
+  return launch_rowgemm_out<T, 4, TZ>(p, stream);
 }
 
-template <typename T>
+template <typename T, typename TZ>
 int pair_bias_fwd(const void* z, const void* ln_w, const void* ln_b, const void* w, void* bias,
                   int n, int c_z, int heads, int out_f32, float eps, hipStream_t stream) {
   RowGemmInParams p = {};
@@ -1036,29 +1127,30 @@ int pair_bias_fwd(const void* z, const void* ln_w, const void* ln_b, const void*
   p.n = n;
   p.aux = heads | (out_f32 ? 0x100 : 0);
   if (c_z == 256) {
-    if constexpr (sizeof(T) == 2) return launch_rowgemm_in<T, kPairBias, 16>(p, stream);
+    if constexpr (sizeof(T) == 2 && sizeof(TZ) == 2) return launch_rowgemm_in<T, kPairBias, 16>(p, stream);
     else return -1;
   }
-  return launch_rowgemm_in<T, kPairBias, 8>(p, stream);
+  return launch_rowgemm_in<T, kPairBias, 8, TZ>(p, stream);
 }
 
-#define PTX_INSTANTIATE(T)                                                                          \
-  template int trimul_project<T>(const void*, const void*, const void*, const void*, const void*,  \
-                                 const void*, const void*, const void*, void*, void*, int, int,    \
-                                 int, int, float, hipStream_t);                                    \
-  template int trimul_output<T>(const void*, const void*, const void*, const void*, const void*,   \
-                                const void*, const void*, const void*, void*, int, int, int,       \
-                                float, hipStream_t);                                               \
-  template int triattn_project<T>(const void*, const void*, const void*, const void*, const void*, \
-                                  const void*, const void*, const void*, void*, void*, void*,      \
-                                  void*, void*, int, int, int, int, int, int, float,               \
-                                  hipStream_t);                                                    \
-  template int triattn_output<T>(const void*, const void*, const void*, void*, int, int, int, int, \
-                                 hipStream_t);                                                     \
-  template int pair_bias_fwd<T>(const void*, const void*, const void*, const void*, void*, int,    \
-                                int, int, int, float, hipStream_t);
-PTX_INSTANTIATE(float)
-PTX_INSTANTIATE(bf16_t)
+#define PTX_INSTANTIATE(T, TZ)                                                                      \
+  template int trimul_project<T, TZ>(const void*, const void*, const void*, const void*,           \
+                                     const void*, const void*, const void*, const void*, void*,    \
+                                     void*, int, int, int, int, float, hipStream_t);               \
+  template int trimul_output<T, TZ>(const void*, const void*, const void*, const void*,            \
+                                    const void*, const void*, const void*, const void*, void*,     \
+                                    int, int, int, float, hipStream_t);                            \
+  template int triattn_project<T, TZ>(const void*, const void*, const void*, const void*,          \
+                                      const void*, const void*, const void*, const void*, void*,   \
+                                      void*, void*, void*, void*, int, int, int, int, int, int,    \
+                                      float, hipStream_t);                                         \
+  template int triattn_output<T, TZ>(const void*, const void*, const void*, void*, int, int, int,  \
+                                     int, hipStream_t);                                            \
+  template int pair_bias_fwd<T, TZ>(const void*, const void*, const void*, const void*, void*,     \
+                                    int, int, int, int, float, hipStream_t);
+PTX_INSTANTIATE(float, float)
+PTX_INSTANTIATE(bf16_t, bf16_t)
+PTX_INSTANTIATE(bf16_t, float)
 #undef PTX_INSTANTIATE
 
 }  // namespace ptx

@@ -134,21 +134,24 @@ __device__ __forceinline__ void normalize_raw(const typename Vec8<T>::type (&raw
 
 // Load RB row blocks whose lane rows start at element offsets off[rb] (+ 8*g added here)
 // and, if LN, normalise them.
-template <typename T, int RB, bool LN, int KS, typename P = T, bool DEFAULTS = true>
-__device__ __forceinline__ void load_rows_at(RowFrags<T, RB, KS>& out, const T* __restrict__ x,
+// TZ: storage type of the rows (T, or float for an fp32 residual stream normalised and
+// rounded to T here; LN only).
+template <typename T, int RB, bool LN, int KS, typename P = T, bool DEFAULTS = true, typename TZ = T>
+__device__ __forceinline__ void load_rows_at(RowFrags<T, RB, KS>& out, const TZ* __restrict__ x,
                                              const int64_t (&off)[RB], const P* __restrict__ gamma,
                                              const P* __restrict__ beta, float eps, int lane) {
+  static_assert(LN || sizeof(TZ) == sizeof(T), "rows of another type are converted by the LayerNorm");
   const int g = lane >> 5;
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
-    const T* rp = x + off[rb] + 8 * g;
-    if (!LN) {
+    const TZ* rp = x + off[rb] + 8 * g;
+    if constexpr (!LN) {
 #pragma unroll
-      for (int kk = 0; kk < KS; ++kk) out.f[rb][kk] = load8<T>(rp + 16 * kk);
+      for (int kk = 0; kk < KS; ++kk) out.f[rb][kk] = load8<T>((const T*)rp + 16 * kk);
     } else {
       f32x8 v[KS];
 #pragma unroll
-      for (int kk = 0; kk < KS; ++kk) v[kk] = to_f32(load8<T>(rp + 16 * kk));
+      for (int kk = 0; kk < KS; ++kk) v[kk] = to_f32(load8<TZ>(rp + 16 * kk));
       normalize_row<T, KS, P, DEFAULTS>(v, gamma, beta, eps, g, out.f[rb]);
     }
   }
@@ -156,8 +159,8 @@ __device__ __forceinline__ void load_rows_at(RowFrags<T, RB, KS>& out, const T* 
 
 // Load RB*32 consecutive logical rows starting at row0 (rows >= n_rows re-read the last
 // valid row; their results are never stored).
-template <typename T, int RB, bool LN, int KS, typename P = T, bool DEFAULTS = true>
-__device__ __forceinline__ void load_rows(RowFrags<T, RB, KS>& out, const T* __restrict__ x,
+template <typename T, int RB, bool LN, int KS, typename P = T, bool DEFAULTS = true, typename TZ = T>
+__device__ __forceinline__ void load_rows(RowFrags<T, RB, KS>& out, const TZ* __restrict__ x,
                                           const RowMap& map, int64_t row0, int64_t n_rows,
                                           const P* __restrict__ gamma, const P* __restrict__ beta,
                                           float eps, int lane) {
@@ -168,7 +171,7 @@ __device__ __forceinline__ void load_rows(RowFrags<T, RB, KS>& out, const T* __r
     p = p < n_rows ? p : n_rows - 1;
     off[rb] = map(p);
   }
-  load_rows_at<T, RB, LN, KS, P, DEFAULTS>(out, x, off, gamma, beta, eps, lane);
+  load_rows_at<T, RB, LN, KS, P, DEFAULTS, TZ>(out, x, off, gamma, beta, eps, lane);
 }
 
 // One weight fragment: 32 output columns x 16 K values, lane -> (column l%32,

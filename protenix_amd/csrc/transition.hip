@@ -81,20 +81,23 @@ __global__ void transition_pack_kernel(const T* __restrict__ w_a, const T* __res
   store8<T>(packed + (int64_t)idx * 8, v);
 }
 
-template <typename T, int KS>
+// TZ: storage type of x and out (float with T = bf16: rows of an fp32 residual stream are
+// normalised in fp32 and rounded to T; the T-rounded update is added to the fp32 row).
+template <typename T, int KS, typename TZ = T>
 __global__ __launch_bounds__((TrCfg<T, KS>::NW * 64)) void transition_fused_kernel(
-    const T* x, const T* __restrict__ gamma, const T* __restrict__ beta,
-    const T* __restrict__ packed, T* out, int64_t n_rows, int n_chunks, int add_residual,
+    const TZ* x, const T* __restrict__ gamma, const T* __restrict__ beta,
+    const T* __restrict__ packed, TZ* out, int64_t n_rows, int n_chunks, int add_residual,
     float eps) {
   typedef typename Vec8<T>::type V8;
-  typedef typename VecE<T>::type VE_t;
+  typedef typename VecE<TZ>::type VE_t;
   typedef TrCfg<T, KS> G;
-  typedef Cfg<T> C;
+  typedef Cfg<TZ> C;   // staging tile and stores
+  constexpr bool MIXED = !std::is_same<T, TZ>::value;
   constexpr int RB = G::RB, NBUF = G::NBUF, D = G::D, PIECES = G::PIECES, FPW = G::FPW, NW = G::NW;
   constexpr int NOB = G::NOB, kTrFrags = G::FRAGS, kCx = 16 * KS;
   __shared__ u32x4_t lds_w[NBUF][kTrFrags][PIECES][kWave];
-  static_assert(sizeof(T) * NW * 32 * C::PITCH <= sizeof(u32x4_t) * kTrFrags * PIECES * kWave,
-                "the staging tiles reuse chunk buffer 0");
+  static_assert(sizeof(TZ) * NW * 32 * C::PITCH <= sizeof(u32x4_t) * (NBUF - 1) * kTrFrags * PIECES * kWave,
+                "the staging tiles reuse the chunk buffers");
 
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int64_t row0 = ((int64_t)blockIdx.x * NW + wave) * (RB * 32);
@@ -232,7 +235,7 @@ __global__ __launch_bounds__((TrCfg<T, KS>::NW * 64)) void transition_fused_kern
 #pragma unroll
     for (int ps = 0; ps < C::NPASS; ++ps) {
       int mj, m0;
-      stage_coord<T>(ps, lane, mj, m0);
+      stage_coord<TZ>(ps, lane, mj, m0);
       const int64_t pr = row0 + rb * 32 + mj;
       obase[rb][ps] = pr < n_rows ? pr * kCx + m0 : -1;
     }
@@ -251,27 +254,28 @@ __global__ __launch_bounds__((TrCfg<T, KS>::NW * 64)) void transition_fused_kern
   for (int kk = 0; kk < KS; ++kk) act_part(kk, ab1);
   gemm2((n_chunks - 1) % NBUF, read_frag((n_chunks - 1) % NBUF, 2 * KS));
 
-  // ---- epilogue: out rows through the per-wave staging tile (reuses chunk buffer 0 once
+  // ---- epilogue: out rows through the per-wave staging tile (reuses the chunk buffers once
   // every wave is past its last fragment read and all loads have landed) ----
   ring_barrier<0>();
-  T* st = reinterpret_cast<T*>(&lds_w[0][0][0][0]) + wave * (32 * C::PITCH);
+  TZ* st = reinterpret_cast<TZ*>(&lds_w[0][0][0][0]) + wave * (32 * C::PITCH);
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
 #pragma unroll
     for (int ob = 0; ob < NOB; ++ob) {
       float vals[16];
 #pragma unroll
-      for (int r = 0; r < 16; ++r) vals[r] = acc_o[rb][ob][r];
+      for (int r = 0; r < 16; ++r)   // (mixed: the update is rounded to T before it is added)
+        vals[r] = MIXED ? to_f32(from_f32<T>(acc_o[rb][ob][r])) : acc_o[rb][ob][r];
       wave_lds_sync();
-      stage_put<T>(st, vals, lane);
+      stage_put<TZ>(st, vals, lane);
       wave_lds_sync();
 #pragma unroll
       for (int ps = 0; ps < C::NPASS; ++ps) {
         int mj, m0;
-        stage_coord<T>(ps, lane, mj, m0);
+        stage_coord<TZ>(ps, lane, mj, m0);
         if (obase[rb][ps] >= 0) {
-          VE_t v = stage_get_vec<T>(st, mj, m0);
-          if (add_residual) v = add_vec<T>(v, resv[rb][ob][ps]);
+          VE_t v = stage_get_vec<TZ>(st, mj, m0);
+          if (add_residual) v = add_vec<TZ>(v, resv[rb][ob][ps]);
           *reinterpret_cast<VE_t*>(out + obase[rb][ps] + ob * 32) = v;
         }
       }
@@ -298,35 +302,35 @@ int transition_pack(const void* w_a, const void* w_b, const void* w_o, void* pac
   return transition_pack_ks<T, 8>(w_a, w_b, w_o, packed, n_factor, stream);
 }
 
-template <typename T, int KS>
+template <typename T, int KS, typename TZ>
 static int transition_fwd_ks(const void* x, const void* ln_w, const void* ln_b, const void* packed,
                              void* out, int64_t rows, int n_factor, int add_residual, float eps,
                              hipStream_t stream) {
   const int64_t rows_per_block = TrCfg<T, KS>::NW * TrCfg<T, KS>::RB * 32;
   const int64_t blocks = (rows + rows_per_block - 1) / rows_per_block;
-  transition_fused_kernel<T, KS><<<dim3((unsigned)blocks), dim3(TrCfg<T, KS>::NW * 64), 0, stream>>>(
-      (const T*)x, (const T*)ln_w, (const T*)ln_b, (const T*)packed, (T*)out, rows,
+  transition_fused_kernel<T, KS, TZ><<<dim3((unsigned)blocks), dim3(TrCfg<T, KS>::NW * 64), 0, stream>>>(
+      (const TZ*)x, (const T*)ln_w, (const T*)ln_b, (const T*)packed, (TZ*)out, rows,
       16 * KS * n_factor / 32, add_residual, eps);
   return 0;
 }
 
-template <typename T>
+template <typename T, typename TZ>
 int transition_fwd(const void* x, const void* ln_w, const void* ln_b, const void* packed,
                    void* out, int64_t rows, int c, int n_factor, int add_residual, float eps,
                    hipStream_t stream) {
   if (rows == 0) return 0;
   if (c == 64)
-    return transition_fwd_ks<T, 4>(x, ln_w, ln_b, packed, out, rows, n_factor, add_residual, eps,
+    return transition_fwd_ks<T, 4, TZ>(x, ln_w, ln_b, packed, out, rows, n_factor, add_residual, eps,
                                    stream);
   if (c == 256) {
     // bf16 only: an fp32 chunk of weights (96 KB) leaves no room for a ring in LDS
-    if constexpr (sizeof(T) == 2)
-      return transition_fwd_ks<T, 16>(x, ln_w, ln_b, packed, out, rows, n_factor, add_residual,
+    if constexpr (sizeof(T) == 2 && sizeof(TZ) == 2)
+      return transition_fwd_ks<T, 16, TZ>(x, ln_w, ln_b, packed, out, rows, n_factor, add_residual,
                                       eps, stream);
     else
       return -1;
   }
-  return transition_fwd_ks<T, 8>(x, ln_w, ln_b, packed, out, rows, n_factor, add_residual, eps,
+  return transition_fwd_ks<T, 8, TZ>(x, ln_w, ln_b, packed, out, rows, n_factor, add_residual, eps,
                                  stream);
 }
 
@@ -334,9 +338,11 @@ template int transition_pack<float>(const void*, const void*, const void*, void*
                                     hipStream_t);
 template int transition_pack<bf16_t>(const void*, const void*, const void*, void*, int, int,
                                      hipStream_t);
-template int transition_fwd<float>(const void*, const void*, const void*, const void*, void*,
-                                   int64_t, int, int, int, float, hipStream_t);
-template int transition_fwd<bf16_t>(const void*, const void*, const void*, const void*, void*,
-                                    int64_t, int, int, int, float, hipStream_t);
+template int transition_fwd<float, float>(const void*, const void*, const void*, const void*,
+                                          void*, int64_t, int, int, int, float, hipStream_t);
+template int transition_fwd<bf16_t, bf16_t>(const void*, const void*, const void*, const void*,
+                                            void*, int64_t, int, int, int, float, hipStream_t);
+template int transition_fwd<bf16_t, float>(const void*, const void*, const void*, const void*,
+                                           void*, int64_t, int, int, int, float, hipStream_t);
 
 }  // namespace ptx

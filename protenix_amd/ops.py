@@ -18,6 +18,17 @@ def _dt(t: torch.Tensor) -> int:
         raise RuntimeError(f"protenix_amd kernels take float32 or bfloat16 tensors, got {t.dtype}")
 
 
+def _dt_stream(z: torch.Tensor, compute: torch.dtype) -> int:
+    """dtype code of a call whose residual-stream tensors (z, x, out) are `z` and whose
+    weights and workspaces are `compute`: PTX_MIXED for fp32 rows with bf16 arithmetic."""
+    if z.dtype == compute:
+        return _dt(z)
+    if z.dtype == torch.float32 and compute == torch.bfloat16:
+        return _lib.PTX_MIXED
+    raise RuntimeError(f"protenix_amd: rows in {z.dtype} with weights in {compute} are not supported "
+                       "(same dtype, or float32 rows with bfloat16 weights)")
+
+
 def _dev(t: torch.Tensor, name: str) -> None:
     if not t.is_cuda:
         raise RuntimeError(
@@ -64,6 +75,16 @@ def _same(t: Optional[torch.Tensor], like: torch.Tensor, name: str) -> Optional[
     if t.dtype != like.dtype or t.device != like.device:
         t = t.to(device=like.device, dtype=like.dtype)
     return t.contiguous()
+
+
+def compute_dtype(x: torch.Tensor) -> torch.dtype:
+    """dtype the kernels' arithmetic, weights and workspaces take for rows `x`: x's own, or
+    bfloat16 for float32 rows of at most 128 channels under torch.autocast(bfloat16) - the
+    fused fp32-residual-stream mode (PTX_MIXED of the C ABI)."""
+    ac = autocast_compute_dtype(x)
+    if ac == torch.bfloat16 and x.shape[-1] in (64, 128):
+        return ac
+    return x.dtype
 
 
 def autocast_compute_dtype(x: torch.Tensor) -> Optional[torch.dtype]:
@@ -145,10 +166,11 @@ def _workspace(shape, dtype, device) -> torch.Tensor:
     return torch.empty(shape, dtype=dtype, device=device)
 
 
-def _mask_for(mask: Optional[torch.Tensor], z: torch.Tensor) -> Optional[torch.Tensor]:
+def _mask_for(mask: Optional[torch.Tensor], z: torch.Tensor,
+              dtype: Optional[torch.dtype] = None) -> Optional[torch.Tensor]:
     if mask is None:
         return None
-    return mask.to(device=z.device, dtype=z.dtype).contiguous()
+    return mask.to(device=z.device, dtype=dtype or z.dtype).contiguous()
 
 
 def triangle_multiplication(z: torch.Tensor, mask: Optional[torch.Tensor], w: dict, incoming: bool,
@@ -160,18 +182,19 @@ def triangle_multiplication(z: torch.Tensor, mask: Optional[torch.Tensor], w: di
     lib = _lib.load()
     n, c_z = z.shape[0], z.shape[-1]
     c_h = w["w_ap"].shape[0]
-    dt, st = _dt(z), _stream()
+    cd = w["w_ap"].dtype            # arithmetic / workspace dtype; z may be fp32 beside bf16 weights
+    dt, st = _dt_stream(z, cd), _stream()
     pitch = key_pitch(n)
-    mask = _mask_for(mask, z)
+    mask = _mask_for(mask, z, cd)
     # contraction operands in the library's fragment order (see include/protenix_amd.h)
     n_op = lib.ptx_trimul_operand_elems(n, c_h)
-    a = _workspace((n_op,), z.dtype, z.device)
-    b = _workspace((n_op,), z.dtype, z.device)
+    a = _workspace((n_op,), cd, z.device)
+    b = _workspace((n_op,), cd, z.device)
     with torch.cuda.device(z.device):
         _call("trimul_project", lib.ptx_trimul_project, _ptr(z), _ptr(mask), _ptr(w["ln_in_w"]), _ptr(w["ln_in_b"]), _ptr(w["w_ap"]),
             _ptr(w["w_ag"]), _ptr(w["w_bp"]), _ptr(w["w_bg"]), _ptr(a), _ptr(b), n, c_z, c_h, pitch,
             int(incoming), eps, dt, st)
-        x = _workspace((c_h, n, n), z.dtype, z.device)
+        x = _workspace((c_h, n, n), cd, z.device)
         _call("trimul_contract", lib.ptx_trimul_contract, _ptr(a), _ptr(b), _ptr(x), n, c_h, pitch, dt, st)
         del a, b
         if out is None:
@@ -192,18 +215,19 @@ def triangle_attention(z: torch.Tensor, mask: Optional[torch.Tensor], w: dict, h
     _dev(z, "z")
     lib = _lib.load()
     n, c = z.shape[0], z.shape[-1]
-    dt, st = _dt(z), _stream()
+    cd = w["w_q"].dtype
+    dt, st = _dt_stream(z, cd), _stream()
     pitch = key_pitch(n)
-    mask = _mask_for(mask, z)
+    mask = _mask_for(mask, z, cd)
     dev = z.device
     # attention-core layouts (see include/protenix_amd.h): q, gate, output head-major; K, V^T
     # and the triangle bias in fragment-ordered key tiles
     n_kv, n_tb = lib.ptx_triattn_kv_elems(n, heads), lib.ptx_triattn_bias_elems(n, heads)
-    q = _workspace((heads, n, n, d), z.dtype, dev)
-    g = _workspace((heads, n, n, d), z.dtype, dev)
-    k = _workspace((n_kv,), z.dtype, dev)
-    vt = _workspace((n_kv,), z.dtype, dev)
-    tb = _workspace((n_tb,), z.dtype, dev)
+    q = _workspace((heads, n, n, d), cd, dev)
+    g = _workspace((heads, n, n, d), cd, dev)
+    k = _workspace((n_kv,), cd, dev)
+    vt = _workspace((n_kv,), cd, dev)
+    tb = _workspace((n_tb,), cd, dev)
     with torch.cuda.device(dev):
         _call("triattn_project", lib.ptx_triattn_project, _ptr(z), _ptr(w["ln_w"]),
               _ptr(w["ln_b"]), _ptr(w["w_q"]), _ptr(w["w_k"]), _ptr(w["w_v"]), _ptr(w["w_g"]),
@@ -246,7 +270,7 @@ def transition(x: torch.Tensor, w: dict, n_factor: int, add_residual: bool,
     if not x2.is_contiguous():
         x2 = x2.contiguous()
     rows = x2.shape[0]
-    dt, st = _dt(x), _stream()
+    dt, st = _dt_stream(x, w["packed"].dtype), _stream()
     if out is None:
         out = torch.empty_like(x2)
     o2 = out.view(-1, c)
@@ -263,8 +287,8 @@ def pair_bias(z: torch.Tensor, ln_w: Optional[torch.Tensor], ln_b: Optional[torc
     lib = _lib.load()
     n, c = z.shape[0], z.shape[-1]
     heads = w.shape[0]
-    out = torch.empty((heads, n, n), dtype=torch.float32 if out_f32 else z.dtype, device=z.device)
+    out = torch.empty((heads, n, n), dtype=torch.float32 if out_f32 else w.dtype, device=z.device)
     with torch.cuda.device(z.device):
         _call("pair_bias", lib.ptx_pair_bias_fwd, _ptr(z), _ptr(ln_w), _ptr(ln_b), _ptr(w), _ptr(out), n, c,
-                                         heads, int(out_f32), eps, _dt(z), _stream())
+                                         heads, int(out_f32), eps, _dt_stream(z, w.dtype), _stream())
     return out

@@ -112,10 +112,14 @@ class Transition(nn.Module):
         x + update there instead and returns it."""
         _forward_only(x, module=self)
         add = _residual_out is not None
+        cd = ops.compute_dtype(x)     # bf16 for fp32 rows of <= 128 channels under bf16 autocast
         fused = self.c_in in (64, 128) or (self.c_in == 256 and x.dtype == torch.bfloat16)
         if fused and (self.n * self.c_in) % 64 == 0:
-            return ops.transition(x, self._weights(x.dtype, x.device), self.n, add_residual=add,
-                                  out=_residual_out)
+            out = ops.transition(x, self._weights(cd, x.device), self.n, add_residual=add,
+                                 out=_residual_out)
+            # (an update computed on fp32 rows under autocast holds bf16 values: returned in
+            # the autocast dtype, like the reference's last linear)
+            return out if (add or cd == x.dtype) else out.to(cd)
         # other widths: HIP LayerNorm + library GEMMs (a and b as one GEMM on the stacked weights)
         y = self.layernorm1(x)
         if (not torch.is_grad_enabled() and self.linear_no_bias_a.precision is None

@@ -79,13 +79,16 @@ class Attention(nn.Module):
         # logits, softmax and the weighted sum in fp32 (the reference upcasts q, k
         # and the bias and relies on autocast for v; here v is upcast as well)
         d = q.dtype
-        w = torch.matmul(q.float(), k.float().transpose(-1, -2))
-        if attn_bias is not None:
-            if attn_bias.dim() != w.dim():
-                attn_bias = attn_bias.unsqueeze(-3)
-            w = w + attn_bias.float()
-        w = torch.softmax(w, dim=-1)
-        o = torch.matmul(w, v.float()).to(d).transpose(-2, -3)
+        # (shielded from autocast, which would run both products in its own dtype again - as
+        # the reference shields its non-SDPA branch, primitives.py:269)
+        with torch.autocast("cuda", enabled=False):
+            w = torch.matmul(q.float(), k.float().transpose(-1, -2))
+            if attn_bias is not None:
+                if attn_bias.dim() != w.dim():
+                    attn_bias = attn_bias.unsqueeze(-3)
+                w = w + attn_bias.float()
+            w = torch.softmax(w, dim=-1)
+            o = torch.matmul(w, v.float()).to(d).transpose(-2, -3)
         if self.linear_g is not None:
             if g_lin is None:
                 g_lin = self.linear_g(q_x)
@@ -122,8 +125,9 @@ class AttentionPairBias(nn.Module):
         """[*, N, N, c_z] -> fp32 [*, heads, N, N] = permute(linear(LN(z)))
         (transformer.py:191-194)."""
         ps = (self.layernorm_z.weight, self.layernorm_z.bias, self.linear_nobias_z.weight)
-        ln_w, ln_b, w = self._cache.get(ps, z.dtype, z.device,
-                                        lambda: tuple(_cv(p, z.dtype, z.device) for p in ps))
+        cd = ops.compute_dtype(z)     # bf16 for fp32 rows of 128 channels under bf16 autocast
+        ln_w, ln_b, w = self._cache.get(ps, cd, z.device,
+                                        lambda: tuple(_cv(p, cd, z.device) for p in ps))
         n, c = z.shape[-2], z.shape[-1]
         zb = z.contiguous().reshape(-1, n, n, c)
         out = torch.stack([ops.pair_bias(zb[i], ln_w, ln_b, w, out_f32=True)

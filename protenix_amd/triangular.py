@@ -29,6 +29,20 @@ def OpenfoldLinear(in_dim: int, out_dim: int, bias: bool = True, init: str = "de
     return Linear(in_dim, out_dim, bias=bias, initializer=init)
 
 
+def _stream_and_compute_dtype(z: torch.Tensor, c_z: int):
+    """(rows to hand to the kernels, arithmetic dtype, dtype to cast a returned update to).
+    fp32 rows under torch.autocast(bfloat16): rows of 64 / 128 channels stay fp32 and the
+    kernels run bf16 arithmetic on them (the fused fp32 residual stream); wider rows are
+    rounded to the autocast dtype first."""
+    ac = ops.autocast_compute_dtype(z)
+    if ac is None:
+        return z, z.dtype, None
+    cd = ops.compute_dtype(z)
+    if cd == z.dtype:          # no fused kernel for this width / autocast dtype
+        return z.to(ac), ac, None
+    return z, cd, cd
+
+
 def _per_batch(z: torch.Tensor, mask: Optional[torch.Tensor]):
     """[*, N, N, C] -> list of ([N, N, C], [N, N] or None) sharing storage with z."""
     if z.dim() < 3:
@@ -87,7 +101,12 @@ class TriangleMultiplicativeUpdate(nn.Module):
                 f"{triangle_multiplicative}")
         _forward_only(z, module=self)
         add_inplace = bool(inplace_safe and _add_with_inplace)
-        w = self._weights(z.dtype, z.device)
+        z_in = z
+        z, cd, cast_back = _stream_and_compute_dtype(z, self.c_z)
+        if z is not z_in and add_inplace:
+            # rows rounded for the kernels: the update is added to the caller's own rows
+            return z_in.add_(self.forward(z_in, mask=mask))
+        w = self._weights(cd, z.device)
         src = z if z.is_contiguous() else z.contiguous()
         zb, mb = _per_batch(src, mask)
         out = src if add_inplace else torch.empty_like(src)
@@ -99,7 +118,9 @@ class TriangleMultiplicativeUpdate(nn.Module):
         if add_inplace and out is not z:
             z.copy_(out)
             return z
-        return out
+        # (an update computed on fp32 rows under autocast holds bf16 values: returned as the
+        # autocast dtype, like the reference's linear_z output)
+        return out.to(cast_back) if (cast_back is not None and not add_inplace) else out
 
 
 class TriangleMultiplicationOutgoing(TriangleMultiplicativeUpdate):
@@ -169,7 +190,12 @@ class TriangleAttention(nn.Module):
     def _run(self, x: torch.Tensor, mask: Optional[torch.Tensor], transposed: bool,
              residual_inplace: bool) -> torch.Tensor:
         _forward_only(x, module=self)
-        w = self._weights(x.dtype, x.device)
+        x_in = x
+        x, cd, cast_back = _stream_and_compute_dtype(x, self.c_in)
+        if residual_inplace and x is not x_in:
+            # rows rounded for the kernels: the update is added to the caller's own rows
+            return x_in.add_(self._run(x_in, mask, transposed, residual_inplace=False))
+        w = self._weights(cd, x.device)
         src = x if x.is_contiguous() else x.contiguous()
         xb, mb = _per_batch(src, mask)
         out = src if residual_inplace else torch.empty_like(src)
@@ -181,7 +207,7 @@ class TriangleAttention(nn.Module):
         if residual_inplace and out is not x:
             x.copy_(out)
             return x
-        return out
+        return out.to(cast_back) if (cast_back is not None and not residual_inplace) else out
 
     def forward(self, x: torch.Tensor, mask: Optional[torch.Tensor] = None,
                 chunk_size: Optional[int] = None, triangle_attention: str = "torch",
