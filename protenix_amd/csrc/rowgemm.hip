@@ -183,6 +183,21 @@ rowgemm_in_kernel(RowGemmInParams p) {
   T* const sink = reinterpret_cast<T*>(g_store_sink) + lane * C::VE;
   constexpr int nch = IC::NCH;
 
+  // kRegRes: both LayerNorms' parameters as fp32 in LDS.  Read from global memory, all 32
+  // parameter loads of a tile are issued (and converted) ahead of the rows, 128 registers
+  // that this instantiation does not have.
+  __shared__ __attribute__((aligned(16))) float lds_affine2[4][kRegRes ? 16 * SL : 1];
+  if constexpr (kRegRes) {
+    for (int c = threadIdx.x; c < 16 * SL; c += NW * kWave) {
+      if (c < kCz) {
+        lds_affine2[0][c] = p.gamma ? to_f32(((const T*)p.gamma)[c]) : 1.0f;
+        lds_affine2[1][c] = p.beta ? to_f32(((const T*)p.beta)[c]) : 0.0f;
+      }
+      lds_affine2[2][c] = p.gamma2 ? to_f32(((const T*)p.gamma2)[c]) : 1.0f;
+      lds_affine2[3][c] = p.beta2 ? to_f32(((const T*)p.beta2)[c]) : 0.0f;
+    }
+    __syncthreads();
+  }
   if constexpr (kLdsAffine) {
     for (int c = threadIdx.x; c < kCz; c += NW * kWave) {
       lds_affine[0][c] = p.gamma ? to_f32(((const T*)p.gamma)[c]) : 1.0f;
@@ -286,18 +301,9 @@ rowgemm_in_kernel(RowGemmInParams p) {
     }
     load_rows_at<T, RB, true>(xf, (const TZ*)p.x, off, gamma, beta, p.eps, lane);
   } else if constexpr (kRegRes) {
-    // raw fp32 rows stay in registers for the residual add: lane (row n, half g) holds
-    // channels 16*kk + 8*g .. +7, which the permuted weight columns make the very channels
-    // its accumulator registers stand for
-#pragma unroll
-    for (int rb = 0; rb < RB; ++rb) {
-      int64_t pr = row0 + rb * 32 + n;
-      pr = pr < p.n_rows ? pr : p.n_rows - 1;
-      const TZ* rp = (const TZ*)p.x + p.xmap(pr) + 8 * g;
-#pragma unroll
-      for (int kk = 0; kk < KS; ++kk) zres[rb][kk] = load8<TZ>(rp + 16 * kk);
-      normalize_row<T, KS>(zres[rb], gamma, beta, p.eps, g, xf.f[rb]);
-    }
+    // (the fp32 rows are requested further down, once the triangle product's rows are on
+    // their way through the staging tile: both sets of raw rows at once do not fit the
+    // registers)
   } else if constexpr (MODE == kTriMulOut) {
     RowFrags<T, RB, KS> zraw;
     load_rows<T, RB, false>(zraw, (const T*)p.x, p.xmap, row0, p.n_rows, (const T*)nullptr,
@@ -334,6 +340,9 @@ rowgemm_in_kernel(RowGemmInParams p) {
         for (int ps = 0; ps < C::NPASS; ++ps) {
           int chn, r0;
           stage_coord<T>(ps, lane, chn, r0);
+          // (fp32 residual rows in registers: opaque per tile, or the eight plane offsets are
+          // kept in registers across the tile loop, which has none to spare)
+          if constexpr (kRegRes) asm volatile("" : "+v"(chn));
           const int64_t pr = row0 + rb * 32 + r0;
           const T* src = x2 + (int64_t)(32 * cg + chn) * p.n_rows;
           if constexpr (vec_ok) {
@@ -364,7 +373,26 @@ rowgemm_in_kernel(RowGemmInParams p) {
           for (int t = 0; t < 8; ++t)
             v[2 * cg + k2][t] = to_f32(st[(16 * k2 + 8 * g + t) * C::PITCH + n]);
       }
-      normalize_row<T>(v, gamma2, beta2, p.eps, g, xf2.f[rb]);
+      if constexpr (kRegRes)
+        normalize_row<T, SL, float, false>(v, lds_affine2[2], lds_affine2[3], p.eps, g, xf2.f[rb]);
+      else
+        normalize_row<T>(v, gamma2, beta2, p.eps, g, xf2.f[rb]);
+      if constexpr (kRegRes) {
+        // The raw fp32 rows stay in registers for the residual add: lane (row n, half g)
+        // holds channels 16*kk + 8*g .. +7, which the permuted weight columns make the very
+        // channels its accumulator registers stand for.  Requested only now (the row index
+        // is made to depend on the last normalised fragment, which keeps the loads from
+        // moving up): together with the fp32 copy of the triangle product's rows they do
+        // not fit the registers.
+        static_assert(RB == 1, "one row block per wave");
+        int64_t pr = row0 + n;
+        asm volatile("" : "+v"(pr) : "v"(xf2.f[rb][SL - 1]));
+        pr = pr < p.n_rows ? pr : p.n_rows - 1;
+        const TZ* rp = (const TZ*)p.x + p.xmap(pr) + 8 * g;
+#pragma unroll
+        for (int kk = 0; kk < KS; ++kk) zres[rb][kk] = load8<TZ>(rp + 16 * kk);
+        normalize_row<T, KS, float, false>(zres[rb], lds_affine2[0], lds_affine2[1], p.eps, g, xf.f[rb]);
+      }
     }
   }
 
@@ -479,8 +507,7 @@ rowgemm_in_kernel(RowGemmInParams p) {
       *reinterpret_cast<VE_t*>(rrow[rb][ps] >= 0 ? outp + off : sink) = v;
     }
   };
-  // (not unrolled: unrolled, the compiler hoists every chunk's loads to the top and spills them.
-  // kRegRes indexes the register copy of the rows by chunk and has to be unrolled.)
+  // (not unrolled: unrolled, the compiler hoists every chunk's loads to the top and spills them)
   auto chunk_body = [&](int ch) {
     const int buf = (!RES && C::NBUF == 2) ? (ch & 1) : 0;
     if constexpr (kDma) {
@@ -730,6 +757,15 @@ rowgemm_in_kernel(RowGemmInParams p) {
         TZ* stz = lds_stage_z[wave];
 #pragma unroll
         for (int rb = 0; rb < RB; ++rb) {
+          // this chunk's two fragments of the raw row (a uniform select: the chunk loop is
+          // not unrolled, and registers cannot be indexed by a loop counter)
+          f32x8 zr[2];
+#pragma unroll
+          for (int c = 0; c < KS / 2; ++c)
+            if (ch == c) {
+              zr[0] = zres[rb][2 * c];
+              zr[1] = zres[rb][2 * c + 1];
+            }
           wave_lds_sync();
 #pragma unroll
           for (int k2 = 0; k2 < 2; ++k2) {
@@ -740,7 +776,7 @@ rowgemm_in_kernel(RowGemmInParams p) {
               // linear_z output rounded to T, times the gate, rounded to T: the update
               const float u = to_f32(from_f32<T>(to_f32(from_f32<T>(acc[rb][0][r])) *
                                                  sigmoidf_fast(acc[rb][1][r])));
-              o[t] = p.add_residual ? zres[rb][2 * ch + k2][t] + u : u;
+              o[t] = p.add_residual ? zr[k2][t] + u : u;
             }
             // row n of the tile, columns 16*k2 + 8*g .. +7 (8-byte LDS stores)
             f32x2* dst = reinterpret_cast<f32x2*>(stz + n * CZ::PITCH + 16 * k2 + 8 * g);
@@ -793,13 +829,8 @@ rowgemm_in_kernel(RowGemmInParams p) {
       __syncthreads();
     }
   };
-  if constexpr (kRegRes) {
-#pragma unroll
-    for (int ch = 0; ch < nch; ++ch) chunk_body(ch);
-  } else {
 #pragma clang loop unroll(disable)
-    for (int ch = 0; ch < nch; ++ch) chunk_body(ch);
-  }
+  for (int ch = 0; ch < nch; ++ch) chunk_body(ch);
     if (!RES) break;
     tile += tile_step;
   }
