@@ -97,3 +97,56 @@ def test_state_dict_layout_matches_oracle_and_default_init_is_identity_shaped():
     assert P.TriangleAttentionEndingNode(128, 32, 4).starting is False
     with pytest.raises(NotImplementedError):
         P.AttentionPairBias(has_s=True)
+
+
+# state-dict keys of one Pairformer block, as the reference's modules declare them
+# (triangular.py:113-119, 190-197, 622-628; layers.py:340-357; primitives.py:175-188, 695-716;
+# transformer.py:79-98) - written out literally, not derived from any of this repository's code
+_BLOCK_KEYS = {
+    **{f"{m}.{k}": shape for m in ("tri_mul_out", "tri_mul_in") for k, shape in {
+        "linear_g.weight": (128, 128), "linear_z.weight": (128, 128),
+        "layer_norm_in.weight": (128,), "layer_norm_in.bias": (128,),
+        "layer_norm_out.weight": (128,), "layer_norm_out.bias": (128,),
+        "linear_a_p.weight": (128, 128), "linear_a_g.weight": (128, 128),
+        "linear_b_p.weight": (128, 128), "linear_b_g.weight": (128, 128)}.items()},
+    **{f"{m}.{k}": shape for m in ("tri_att_start", "tri_att_end") for k, shape in {
+        "layer_norm.weight": (128,), "layer_norm.bias": (128,), "linear.weight": (4, 128),
+        "mha.linear_q.weight": (128, 128), "mha.linear_k.weight": (128, 128),
+        "mha.linear_v.weight": (128, 128), "mha.linear_o.weight": (128, 128),
+        "mha.linear_g.weight": (128, 128)}.items()},
+    "pair_transition.layernorm1.weight": (128,), "pair_transition.layernorm1.bias": (128,),
+    "pair_transition.linear_no_bias_a.weight": (512, 128),
+    "pair_transition.linear_no_bias_b.weight": (512, 128),
+    "pair_transition.linear_no_bias.weight": (128, 512),
+    "attention_pair_bias.layernorm_a.weight": (384,), "attention_pair_bias.layernorm_a.bias": (384,),
+    "attention_pair_bias.attention.linear_q.weight": (384, 384),
+    "attention_pair_bias.attention.linear_q.bias": (384,),
+    "attention_pair_bias.attention.linear_k.weight": (384, 384),
+    "attention_pair_bias.attention.linear_v.weight": (384, 384),
+    "attention_pair_bias.attention.linear_o.weight": (384, 384),
+    "attention_pair_bias.attention.linear_g.weight": (384, 384),
+    "attention_pair_bias.layernorm_z.weight": (128,), "attention_pair_bias.layernorm_z.bias": (128,),
+    "attention_pair_bias.linear_nobias_z.weight": (16, 128),
+    "single_transition.layernorm1.weight": (384,), "single_transition.layernorm1.bias": (384,),
+    "single_transition.linear_no_bias_a.weight": (1536, 384),
+    "single_transition.linear_no_bias_b.weight": (1536, 384),
+    "single_transition.linear_no_bias.weight": (384, 1536),
+}
+
+
+def test_product_state_dict_is_the_reference_checkpoint_layout():
+    """A reference checkpoint loads unchanged: the product's PairformerStack has exactly the
+    reference's keys and shapes under blocks.{i}. (and so has the oracle)."""
+    import protenix_amd as P
+    from oracle import pairformer_oracle as O
+
+    for mod in (P, O):
+        sd = mod.PairformerStack(n_blocks=2).state_dict()
+        want = {f"blocks.{i}.{k}": v for i in range(2) for k, v in _BLOCK_KEYS.items()}
+        assert set(sd.keys()) == set(want.keys()), set(sd.keys()) ^ set(want.keys())
+        for k, shape in want.items():
+            assert tuple(sd[k].shape) == shape, (k, tuple(sd[k].shape))
+    # the MSA module's pair stack has no single track (pairformer.py:622-624)
+    sd = P.PairformerBlock(c_s=0).state_dict()
+    assert not any(k.startswith(("attention_pair_bias", "single_transition")) for k in sd)
+    assert len(sd) == len(_BLOCK_KEYS) - 16

@@ -251,13 +251,33 @@ def test_triattn_mask_semantics_chunking_and_ending_node():
     mk = (torch.rand(1, I, I) > 0.2).float()
     mk[..., 0, :] = 1
     assert torch.allclose(e(x, mk), m(x.transpose(1, 2), mk.transpose(1, 2)).transpose(1, 2), atol=1e-6)
-    # bias add order and sign: all keys get +c on the triangle bias -> no change
-    with torch.no_grad():
-        m2 = _mod(O.TriangleAttention, cz, D, H).float()
-        m2.linear.weight.zero_()
-        m2.layer_norm.bias.zero_()
-    base = m2(x, mask)
-    assert torch.isfinite(base).all()
+
+
+def test_attention_biases_are_added_to_the_logits():
+    """softmax_attention: the biases enter the logits additively, with a plus sign.  With v = I
+    the output IS the probability matrix: a per-query constant on every key changes nothing,
+    and raising one key's bias by d multiplies its odds by exp(d) exactly."""
+    g = torch.Generator().manual_seed(8)
+    S, d = 7, 4
+    q, k = torch.randn(2, 3, S, d, generator=g, dtype=D64), torch.randn(2, 3, S, d, generator=g, dtype=D64)
+    v = torch.eye(S, dtype=D64).expand(2, 3, S, S)
+    mb = torch.zeros(2, 1, 1, S, dtype=D64)
+    mb[..., 5] = -1e9                                        # a masked key
+    tb = torch.randn(1, 3, S, S, generator=g, dtype=D64)
+    p0 = O.softmax_attention(q, k, v, [mb, tb])
+    assert torch.allclose(p0.sum(-1), torch.ones(2, 3, S, dtype=D64), atol=1e-12)
+    assert (p0[..., 5] == 0).all()
+    shift = torch.randn(1, 3, S, 1, generator=g, dtype=D64)
+    assert torch.allclose(O.softmax_attention(q, k, v, [mb, tb + shift]), p0, atol=1e-12)
+    bump = torch.zeros(S, dtype=D64)
+    bump[2] = 0.75
+    p1 = O.softmax_attention(q, k, v, [mb, tb + bump])
+    want = p0 * torch.exp(bump)
+    want = want / want.sum(-1, keepdim=True)
+    assert torch.allclose(p1, want, atol=1e-12)
+    # the logits themselves: q.k with no hidden scale
+    a = torch.einsum("bhqd,bhkd->bhqk", q, k) + mb + tb
+    assert torch.allclose(p0, torch.softmax(a, -1), atol=1e-12)
 
 
 # ------------------------------------------------------------- Transition / APB
@@ -345,6 +365,18 @@ def test_stack_is_sequential_blocks_and_state_dict_keys():
         assert k in keys, k
     n = sum(p.numel() for p in O.PairformerBlock().parameters())
     assert n == 2 * 98816 + 2 * 82688 + 196864 + 740736 + 1770240
+    # the stack is its blocks applied in order, each to the previous one's (s, z)
+    O.seed_parameters_(st)
+    g = torch.Generator().manual_seed(3)
+    s = torch.randn(1, 9, 12, generator=g, dtype=D64)
+    z = torch.randn(1, 9, 9, 8, generator=g, dtype=D64)
+    pm = (torch.rand(1, 9, 9, generator=g) > 0.2).to(D64)
+    s1, z1 = st(s, z, pm)
+    s2, z2 = s, z
+    for blk in st.blocks:
+        s2, z2 = blk(s2, z2, pm)
+    assert torch.equal(s1, s2) and torch.equal(z1, z2)
+    assert not torch.equal(z1, z)
 
 
 def test_seeded_inputs_are_deterministic():
