@@ -210,6 +210,29 @@ PTX_API int ptx_triattn_fwd(const void* q, const void* k, const void* vt, const 
                     int key_pitch, int mask_transposed, float inf, int dtype, void* stream);
 
 /*
+ * The fused attention operator on standard-layout tensors: the contract of
+ * TriAttentionFunction.forward (tri_attention/op.py:37-77, kernel tri_attention/forward.py:22-188)
+ * as called from layers.py:539-583.  For every batch b, row i, head h, query position j:
+ *   O[b][i][j][h] = sum_k softmax_k( Q[b][i][j][h] . K[b][i][k][h] + Bias1[b][i][k]
+ *                                    + Bias2[b][h][j][k] ) V[b][i][k][h]
+ *   Q, K, V, O  [batch][n_rows][s][heads][d] contiguous (Q already scaled by 1/sqrt(d), as the
+ *               reference's caller does);  d = 32
+ *   Bias1       [batch][n_rows][s] (the reference's [B, N, 1, 1, S] mask bias) or NULL
+ *   Bias2       [batch][heads][s][s]
+ *   lse         fp32 [batch][n_rows][s][heads] or NULL: log2 of the sum over keys of
+ *               2^(logit * log2 e), the reference's M (forward.py:185-188)
+ *   workspace   ptx_triattn_core_workspace_elems(n_rows, s, heads) elements of `dtype`,
+ *               uninitialised (the operands repacked into the core's tile order)
+ * The logits are formed as (q.k + Bias1) + Bias2 in fp32 wherever Bias1 is non-zero, the
+ * order of layers.py:286-289; they are never materialised.  n_rows may differ from s (a chunk
+ * of rows).  dtype PTX_F32 or PTX_BF16.
+ */
+PTX_API int64_t ptx_triattn_core_workspace_elems(int n_rows, int s, int heads);
+PTX_API int ptx_triattn_core_fwd(const void* q, const void* k, const void* v, const void* bias1,
+                         const void* bias2, void* o, float* lse, void* workspace, int batch,
+                         int n_rows, int s, int heads, int d, int dtype, void* stream);
+
+/*
  * Triangle attention, stage 3 (layers.py:392-396 + the caller's residual add,
  * pairformer.py:189-213):  out(p) = [z(p) +] W_o o[p], where logical row p maps
  * to z[i][j] or, transposed = 1, z[j][i].  o [heads][n][n][d] as written by

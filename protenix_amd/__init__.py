@@ -8,6 +8,7 @@ from .layer_norm import FusedLayerNorm, LayerNorm
 from .pairformer import PairformerBlock, PairformerStack
 from .primitives import Linear, LinearNoBias, Transition
 from .transformer import AttentionPairBias
+from .tri_attention import TriAttentionFunction, tri_attention, tri_attention_forward
 from .triangular import (
     TriangleAttention,
     TriangleAttentionEndingNode,
@@ -23,5 +24,5 @@ __all__ = [
     "PairformerBlock", "PairformerStack", "Transition", "TriangleAttention",
     "TriangleAttentionEndingNode", "TriangleAttentionStartingNode",
     "TriangleMultiplicationIncoming", "TriangleMultiplicationOutgoing",
-    "TriangleMultiplicativeUpdate",
+    "TriangleMultiplicativeUpdate", "TriAttentionFunction", "tri_attention", "tri_attention_forward",
 ]

@@ -302,6 +302,60 @@ PTX_API int ptx_triattn_fwd(const void* q, const void* k, const void* vt, const 
   return after_launch("triattn_fwd");
 }
 
+PTX_API int64_t ptx_triattn_core_workspace_elems(int n_rows, int s, int heads) {
+  if (n_rows <= 0 || s <= 0 || heads <= 0) return 0;
+  const int64_t pitch = ptx_key_pitch(s);
+  return (int64_t)n_rows * s * heads * 32             // q in log2 units
+         + 2 * (int64_t)heads * n_rows * pitch * 32   // K, V^T key tiles
+         + ptx_triattn_bias_elems(s, heads);          // bias tiles
+}
+
+PTX_API int ptx_triattn_core_fwd(const void* q, const void* k, const void* v, const void* bias1,
+                                 const void* bias2, void* o, float* lse, void* workspace, int batch,
+                                 int n_rows, int s, int heads, int d, int dtype, void* stream) {
+  PTX_REQUIRE(dtype_ok(dtype), PTX_ERR_BAD_ARG, "triattn_core_fwd: unknown dtype %d", dtype);
+  PTX_REQUIRE(batch >= 0 && n_rows >= 0 && s >= 0 && heads >= 0, PTX_ERR_BAD_ARG,
+              "triattn_core_fwd: batch=%d n_rows=%d s=%d heads=%d", batch, n_rows, s, heads);
+  PTX_REQUIRE(d == 32, PTX_ERR_UNSUPPORTED, "triattn_core_fwd: only head dim 32 is built (got %d)", d);
+  PTX_REQUIRE(s <= 8192 && n_rows < 32768 && heads <= 64, PTX_ERR_UNSUPPORTED,
+              "triattn_core_fwd: n_rows=%d s=%d heads=%d too large", n_rows, s, heads);
+  if (batch == 0 || n_rows == 0 || s == 0 || heads == 0) return PTX_OK;
+  PTX_REQUIRE(q && k && v && bias2 && o && workspace, PTX_ERR_BAD_ARG,
+              "triattn_core_fwd: null pointer");
+  PTX_REQUIRE(aligned16(q) && aligned16(k) && aligned16(v) && aligned16(bias2) && aligned16(o) &&
+                  aligned16(workspace),
+              PTX_ERR_BAD_ARG, "triattn_core_fwd: pointers must be 16-byte aligned");
+  const int pitch = ptx_key_pitch(s);
+  const int64_t n_q = (int64_t)n_rows * s * heads * 32;
+  const int64_t n_kv = (int64_t)heads * n_rows * pitch * 32;
+  const int64_t n_b2 = (int64_t)heads * s * s, n_b1 = (int64_t)n_rows * s;
+  const size_t es = esize(dtype);
+  char* ws = (char*)workspace;
+  void* qs = ws;
+  void* kf = ws + n_q * es;
+  void* vtf = ws + (n_q + n_kv) * es;
+  void* bf = ws + (n_q + 2 * n_kv) * es;
+  for (int b = 0; b < batch; ++b) {
+    const char* qb = (const char*)q + b * n_q * es;
+    const char* kb = (const char*)k + b * n_q * es;
+    const char* vb = (const char*)v + b * n_q * es;
+    const char* b2 = (const char*)bias2 + b * n_b2 * es;
+    const char* b1 = bias1 ? (const char*)bias1 + b * n_b1 * es : nullptr;
+    char* ob = (char*)o + b * n_q * es;
+    float* lb = lse ? lse + (int64_t)b * n_rows * s * heads : nullptr;
+    PTX_DISPATCH(dtype, {
+      ptx::triattn_pack<T>((const T*)qb, (const T*)kb, (const T*)vb, (const T*)b2, (T*)qs, (T*)kf,
+                           (T*)vtf, (T*)bf, n_rows, s, heads, pitch, (hipStream_t)stream);
+      // standard layout [row][position][head][32]; no gate; bias1 is an additive bias per key
+      ptx::triattn_fwd_ex<T>((const T*)qs, (const T*)kf, (const T*)vtf, (const T*)nullptr,
+                             (const T*)bf, (const T*)b1, (T*)ob, n_rows, s, heads, pitch, 0, 0.0f, 1,
+                             32, (int64_t)s * heads * 32, (int64_t)heads * 32, lb, 1,
+                             (int64_t)s * heads, heads, (hipStream_t)stream);
+    });
+  }
+  return after_launch("triattn_core_fwd");
+}
+
 PTX_API int ptx_triattn_output(const void* o, const void* w_o, const void* z, void* out, int n, int c_in,
                        int transposed, int add_residual, int dtype, void* stream) {
   PTX_REQUIRE(dtype_ok_z(dtype), PTX_ERR_BAD_ARG, "triattn_output: unknown dtype %d", dtype);

@@ -46,18 +46,32 @@ constexpr float kLn2 = 0.6931471805599453f;
 // replaced by the reference 0, which makes exp2() of the raw logit the probability
 constexpr float kZeroReferenceLimit = 14.0f;
 
+// Addressing of q / gate / o and the optional outputs (see the kernel's header comment).
+struct AttnAux {
+  int64_t sh, si, sj;     // element strides of q, gate, o: head, row, query
+  int n_rows;
+  int mask_is_bias;
+  float* lse;             // or null
+  int64_t lh, li, lj;     // element strides of lse: head, row, query
+};
+
 // Rows of the pair tensor handled by one wave: one (more would share the bias tile, but do not
 // fit the register budget).
 #define PTX_ATTN_ROWS 1
 
 // NWQ waves per workgroup (4 or 8), each with 32 queries: the workgroup's waves share the staged
 // K / V^T tiles, so with 8 every wave moves one fragment per tile instead of two.
+// n: queries = keys per row; ax.n_rows: rows (= n for a whole pair tensor, fewer for a chunk of
+// rows).  q, gate and o are addressed through the element strides in `ax` (head, row, query; 32
+// contiguous channels at each position); gate may be null (no gating).  mask: per (row, key),
+// 0/1 values turned into inf*(mask-1), or with ax.mask_is_bias an additive bias used as it is.
+// ax.lse: optional log2-sum-exp2 of the logits per (head, row, query).
 template <typename T, int R, int NWQ>
 __global__ __launch_bounds__((NWQ * 64), (sizeof(T) == 2 ? 16 / NWQ : 2)) void triattn_fwd_kernel(
     const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ vt,
     const T* gate, const T* __restrict__ bias, const T* __restrict__ mask,
     T* o, int n, int heads, int key_pitch, int mask_transposed, float inf,
-    int n_qtiles, int n_rowgroups, int64_t total_items) {
+    int n_qtiles, int n_rowgroups, int64_t total_items, AttnAux ax) {
   typedef typename Vec8<T>::type V8;
   typedef typename Vec4<T>::type V4;
   // ring of 3 key tiles x R rows: iteration t reads tile t while tile t+2 is written
@@ -87,6 +101,7 @@ __global__ __launch_bounds__((NWQ * 64), (sizeof(T) == 2 ? 16 / NWQ : 2)) void t
   // queries all lie beyond n re-reads the last query block; nothing of either is stored.
   const T* b_tiles = bias + ((int64_t)h * q_blocks + min(q0 >> 5, q_blocks - 1)) * key_tiles * kAttnTileElems + lane * 8;
   const int qi = min(q0 + ln, n - 1);
+  const int n_rows = ax.n_rows;
   // Lanes whose query lies beyond n compute on whatever the bias workspace holds there; they
   // store nothing, and they are kept out of the wave-wide decisions below so that the path a
   // wave takes (and with it the rounding of its valid queries) never depends on that content.
@@ -97,7 +112,7 @@ __global__ __launch_bounds__((NWQ * 64), (sizeof(T) == 2 ? 16 / NWQ : 2)) void t
   int64_t qrow[R];                       // head-major q / gate / o row of this lane's query
 #pragma unroll
   for (int r = 0; r < R; ++r) {
-    qrow[r] = (((int64_t)h * n + min(i0 + r, n - 1)) * n + qi) * kD;
+    qrow[r] = h * ax.sh + min(i0 + r, n_rows - 1) * ax.si + qi * ax.sj;
 #pragma unroll
     for (int kk = 0; kk < 2; ++kk) qf[r][kk] = load8<T>(q + qrow[r] + 16 * kk + 8 * g);
   }
@@ -116,7 +131,7 @@ __global__ __launch_bounds__((NWQ * 64), (sizeof(T) == 2 ? 16 / NWQ : 2)) void t
   T pre_mv;
   // mask value of key kc for this wave's row: m_base[kc * m_stride] (stride 0: no mask, any
   // valid address - the value is discarded)
-  const int m_row = min(i0 + min(wave, R - 1), n - 1);
+  const int m_row = min(i0 + min(wave, R - 1), n_rows - 1);
   const unsigned m_stride = has_mask ? (mask_transposed ? n : 1) : 0;
   const T* m_base = mask_or_dummy + (has_mask ? (mask_transposed ? (int64_t)m_row : (int64_t)m_row * n) : 0);
   auto fetch = [&](int tile) {
@@ -125,7 +140,7 @@ __global__ __launch_bounds__((NWQ * 64), (sizeof(T) == 2 ? 16 / NWQ : 2)) void t
     for (int j = 0; j < FPW; ++j) {
       const int fid = wave * FPW + j;              // row = fid / 8, fragment = fid % 8
       const int r = fid >> 3, f = fid & 7;
-      const int64_t rowtiles = ((int64_t)h * n + min(i0 + r, n - 1)) * key_tiles + atile;
+      const int64_t rowtiles = ((int64_t)h * n_rows + min(i0 + r, n_rows - 1)) * key_tiles + atile;
       pre[j] = load8<T>((f < 4 ? k : vt) + rowtiles * kAttnTileElems + (f & 3) * 512 + lane * 8);
     }
     // wave w < R publishes the mask bias of row i0 + w; all waves load (uniform load count)
@@ -150,7 +165,7 @@ __global__ __launch_bounds__((NWQ * 64), (sizeof(T) == 2 ? 16 / NWQ : 2)) void t
       lds_kv[buf][fid >> 3][f][lane] = v;
     }
     if (wave < R) {
-      const float mb = has_mask ? inf * (to_f32(pre_mv) - 1.0f) : 0.0f;
+      const float mb = !has_mask ? 0.0f : ax.mask_is_bias ? to_f32(pre_mv) : inf * (to_f32(pre_mv) - 1.0f);
       lds_mb[buf][wave][lane] = key0 + lane < n ? mb : -INFINITY;
     }
   };
@@ -350,17 +365,23 @@ __global__ __launch_bounds__((NWQ * 64), (sizeof(T) == 2 ? 16 / NWQ : 2)) void t
   int qi_again = qi;
   asm volatile("" : "+v"(qi_again));
 #pragma unroll
-  for (int r = 0; r < R; ++r) qrow[r] = (((int64_t)h * n + min(i0 + r, n - 1)) * n + qi_again) * kD;
+  for (int r = 0; r < R; ++r) qrow[r] = h * ax.sh + min(i0 + r, n_rows - 1) * ax.si + qi_again * ax.sj;
   f32x4 gv[R][4];
 #pragma unroll
   for (int r = 0; r < R; ++r)
 #pragma unroll
-    for (int c = 0; c < 4; ++c)
-      gv[r][c] = to_f32(*reinterpret_cast<const V4*>(gate + qrow[r] + 4 * g + 8 * c));
+    for (int c = 0; c < 4; ++c) {
+      gv[r][c] = f32x4{1.0f, 1.0f, 1.0f, 1.0f};
+      if (gate) gv[r][c] = to_f32(*reinterpret_cast<const V4*>(gate + qrow[r] + 4 * g + 8 * c));
+    }
 #pragma unroll
   for (int r = 0; r < R; ++r) {
-    const float inv = fast_rcp(l_run[r] + swap32(l_run[r]));
-    if (q0 + ln < n && i0 + r < n) {
+    const float l_tot = l_run[r] + swap32(l_run[r]);
+    const float inv = fast_rcp(l_tot);
+    if (ax.lse && g == 0 && q0 + ln < n && i0 + r < n_rows)
+      ax.lse[h * ax.lh + (int64_t)(i0 + r) * ax.li + (int64_t)qi_again * ax.lj] =
+          m_run[r] * kLog2e + __builtin_amdgcn_logf(l_tot);   // v_log_f32 is log2
+    if (q0 + ln < n && i0 + r < n_rows) {
 #pragma unroll
       for (int c = 0; c < 4; ++c) {
         f32x4 ov;
@@ -379,27 +400,50 @@ template <typename T>
 int triattn_fwd(const T* q, const T* k, const T* vt, const T* g, const T* tri_bias, const T* mask,
                 T* o, int n, int heads, int key_pitch, int mask_transposed, float inf,
                 hipStream_t stream) {
-  if (n == 0) return 0;
+  // head-major q, gate, o of a whole pair tensor: [heads][n][n][32]
+  AttnAux ax = {};
+  ax.sh = (int64_t)n * n * kD;
+  ax.si = (int64_t)n * kD;
+  ax.sj = kD;
+  ax.n_rows = n;
+  return triattn_fwd_ex<T>(q, k, vt, g, tri_bias, mask, o, n, n, heads, key_pitch, mask_transposed, inf,
+                           0, ax.sh, ax.si, ax.sj, nullptr, 0, 0, 0, stream);
+}
+
+template <typename T>
+int triattn_fwd_ex(const T* q, const T* k, const T* vt, const T* g, const T* tri_bias,
+                   const T* mask, T* o, int n_rows, int n, int heads, int key_pitch,
+                   int mask_transposed, float inf, int mask_is_bias, int64_t sh, int64_t si,
+                   int64_t sj, float* lse, int64_t lh, int64_t li, int64_t lj, hipStream_t stream) {
+  if (n == 0 || n_rows == 0) return 0;
+  AttnAux ax = {sh, si, sj, n_rows, mask_is_bias, lse, lh, li, lj};
   constexpr int R = PTX_ATTN_ROWS;
   // 8-wave workgroups for long rows (measured: +2 % at n = 768, even at 1024, -2.6 % at 1536,
   // -2.2 % at 2048), where their 256 queries divide n or n is large enough for the idle waves
   // of the last one not to matter
   const bool wide = sizeof(T) == 2 && ((n % 256 == 0 && n >= 1536) || n >= 2048);
   const int n_qtiles = wide ? (n + 255) / 256 : (n + 127) / 128;
-  const int n_rowgroups = (n + R - 1) / R;
+  const int n_rowgroups = (n_rows + R - 1) / R;
   const int64_t total = (int64_t)heads * n_rowgroups * n_qtiles;
   const int64_t per_xcd = (total + 7) / 8;
   if (wide)
     triattn_fwd_kernel<T, R, 8><<<dim3((unsigned)(per_xcd * 8)), dim3(512), 0, stream>>>(
         q, k, vt, g, tri_bias, mask, o, n, heads, key_pitch, mask_transposed, inf, n_qtiles,
-        n_rowgroups, total);
+        n_rowgroups, total, ax);
   else
     triattn_fwd_kernel<T, R, 4><<<dim3((unsigned)(per_xcd * 8)), dim3(256), 0, stream>>>(
         q, k, vt, g, tri_bias, mask, o, n, heads, key_pitch, mask_transposed, inf, n_qtiles,
-        n_rowgroups, total);
+        n_rowgroups, total, ax);
   return 0;
 }
 
+#define PTX_INSTANTIATE_EX(T)                                                                     \
+  template int triattn_fwd_ex<T>(const T*, const T*, const T*, const T*, const T*, const T*, T*,  \
+                                 int, int, int, int, int, float, int, int64_t, int64_t, int64_t,  \
+                                 float*, int64_t, int64_t, int64_t, hipStream_t);
+PTX_INSTANTIATE_EX(float)
+PTX_INSTANTIATE_EX(bf16_t)
+#undef PTX_INSTANTIATE_EX
 template int triattn_fwd<float>(const float*, const float*, const float*, const float*,
                                 const float*, const float*, float*, int, int, int, int, float,
                                 hipStream_t);
