@@ -272,6 +272,35 @@ PTX_API int ptx_pair_bias_fwd(const void* z, const void* ln_w, const void* ln_b,
                       void* bias, int n, int c_z, int heads, int out_f32, float eps, int dtype,
                       void* stream);
 
+/*
+ * The single-representation track of a Pairformer block (c_s = 384): small operands that stay
+ * in the L2, so these entry points aim at few launches, not at a roofline.
+ *
+ * ptx_linear_fwd: Linear / LinearNoBias (primitives.py:83-98, F.linear):
+ *   out = [res +] x w^T [+ bias]      x [rows][k], w [n_out][k], bias [bias_cols] or NULL (added
+ *   to output columns < bias_cols), res [rows][n_out] or NULL, out [rows][split_col].
+ *   Output columns >= split_col are stored transposed in out_t [n_out - split_col][ldt] (entries
+ *   of rows in [rows, ldt) are written as zeros) - how the attention below wants V; pass
+ *   split_col = n_out (and out_t = NULL) for a plain linear layer.  k % 16 == 0, n_out % 8 == 0.
+ * ptx_swiglu_fwd: first half of Transition (primitives.py:206-230) for widths the fused
+ *   ptx_transition_fwd has no kernel for:  out [rows][hidden] = silu(x w_a^T) * (x w_b^T).
+ * ptx_single_attention_fwd: attention with pair bias and gating (transformer.py:196-254,
+ *   primitives.py:233-291, 636-879), per head h:
+ *   out[i][h] = sigmoid(g[i][h]) * sum_j softmax_j( q[i][h].k[j][h] * scale + bias[h][i][j] ) v[j][h]
+ *   q, k, g: rows of pitch ld holding heads * d channels, head-major (g NULL: no gate);
+ *   vt [heads * d][ldt], keys in [n, ldt) zero (as ptx_linear_fwd's out_t); bias [heads][n][n],
+ *   fp32 (bias_f32 = 1) or `dtype`, or NULL; out rows of pitch ldo.  d = 8, 16, 24 or 32.
+ *   Logits and softmax in fp32; the n x n logits are never materialised.
+ */
+PTX_API int ptx_linear_fwd(const void* x, const void* w, const void* bias, int bias_cols,
+                   const void* res, void* out, void* out_t, int split_col, int64_t ldt, int rows,
+                   int k, int n_out, int dtype, void* stream);
+PTX_API int ptx_swiglu_fwd(const void* x, const void* w_a, const void* w_b, void* out, int rows, int k,
+                   int hidden, int dtype, void* stream);
+PTX_API int ptx_single_attention_fwd(const void* q, const void* k, const void* vt, const void* g,
+                   const void* bias, int bias_f32, void* out, int n, int heads, int d, int64_t ld,
+                   int64_t ldt, int64_t ldo, float scale, int dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

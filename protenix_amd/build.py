@@ -14,7 +14,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libprotenix_amd.so")
-SOURCES = ["api.hip", "layernorm.hip", "rowgemm.hip", "triattn.hip", "attnpack.hip", "ntgemm.hip", "transition.hip"]
+SOURCES = ["api.hip", "layernorm.hip", "rowgemm.hip", "triattn.hip", "attnpack.hip", "ntgemm.hip", "transition.hip", "single.hip"]
 # per-source extra flags: the attention kernel's max reductions need no NaN
 # canonicalisation (lets the compiler form v_max3_f32)
 EXTRA_FLAGS = {"triattn.hip": ["-fno-honor-nans"]}

@@ -420,6 +420,71 @@ PTX_API int ptx_transition_fwd(const void* x, const void* ln_w, const void* ln_b
   return after_launch("transition");
 }
 
+PTX_API int ptx_linear_fwd(const void* x, const void* w, const void* bias, int bias_cols,
+                           const void* res, void* out, void* out_t, int split_col, int64_t ldt,
+                           int rows, int k, int n_out, int dtype, void* stream) {
+  PTX_REQUIRE(dtype_ok(dtype), PTX_ERR_BAD_ARG, "linear: unknown dtype %d", dtype);
+  PTX_REQUIRE(rows >= 0 && k > 0 && n_out >= 0, PTX_ERR_BAD_ARG, "linear: rows=%d k=%d n_out=%d",
+              rows, k, n_out);
+  PTX_REQUIRE(k % 16 == 0 && n_out % 8 == 0, PTX_ERR_UNSUPPORTED,
+              "linear: k must be a multiple of 16 and n_out of 8 (got k=%d n_out=%d)", k, n_out);
+  if (split_col < 0 || split_col > n_out) split_col = n_out;
+  if (rows == 0 || n_out == 0) return PTX_OK;
+  PTX_REQUIRE(x && w && (out || split_col == 0), PTX_ERR_BAD_ARG, "linear: null pointer");
+  if (split_col < n_out) {
+    PTX_REQUIRE(out_t, PTX_ERR_BAD_ARG, "linear: out_t is null");
+    PTX_REQUIRE(split_col % 32 == 0 && ldt % 8 == 0 && ldt >= rows && !res, PTX_ERR_BAD_ARG,
+                "linear: transposed tail needs split_col %% 32 == 0, ldt %% 8 == 0, ldt >= rows and "
+                "no residual (split_col=%d ldt=%lld)", split_col, (long long)ldt);
+    PTX_REQUIRE(aligned16(out_t), PTX_ERR_BAD_ARG, "linear: out_t must be 16-byte aligned");
+  }
+  PTX_REQUIRE(aligned16(x) && aligned16(w) && (!out || aligned16(out)) && (!res || aligned16(res)),
+              PTX_ERR_BAD_ARG, "linear: pointers must be 16-byte aligned");
+  PTX_DISPATCH(dtype, ptx::linear_fwd<T>(x, w, bias, bias ? bias_cols : 0, res, out, out_t,
+                                         split_col, ldt, rows, k, n_out, (hipStream_t)stream));
+  return after_launch("linear");
+}
+
+PTX_API int ptx_swiglu_fwd(const void* x, const void* w_a, const void* w_b, void* out, int rows,
+                           int k, int hidden, int dtype, void* stream) {
+  PTX_REQUIRE(dtype_ok(dtype), PTX_ERR_BAD_ARG, "swiglu: unknown dtype %d", dtype);
+  PTX_REQUIRE(rows >= 0 && k > 0 && hidden >= 0, PTX_ERR_BAD_ARG, "swiglu: rows=%d k=%d hidden=%d",
+              rows, k, hidden);
+  PTX_REQUIRE(k % 16 == 0 && hidden % 8 == 0, PTX_ERR_UNSUPPORTED,
+              "swiglu: k must be a multiple of 16 and hidden of 8 (got k=%d hidden=%d)", k, hidden);
+  if (rows == 0 || hidden == 0) return PTX_OK;
+  PTX_REQUIRE(x && w_a && w_b && out, PTX_ERR_BAD_ARG, "swiglu: null pointer");
+  PTX_REQUIRE(aligned16(x) && aligned16(w_a) && aligned16(w_b) && aligned16(out), PTX_ERR_BAD_ARG,
+              "swiglu: pointers must be 16-byte aligned");
+  PTX_DISPATCH(dtype, ptx::swiglu_fwd<T>(x, w_a, w_b, out, rows, k, hidden, (hipStream_t)stream));
+  return after_launch("swiglu");
+}
+
+PTX_API int ptx_single_attention_fwd(const void* q, const void* k, const void* vt, const void* g,
+                                     const void* bias, int bias_f32, void* out, int n, int heads,
+                                     int d, int64_t ld, int64_t ldt, int64_t ldo, float scale,
+                                     int dtype, void* stream) {
+  PTX_REQUIRE(dtype_ok(dtype), PTX_ERR_BAD_ARG, "single_attention: unknown dtype %d", dtype);
+  PTX_REQUIRE(n >= 0 && heads >= 0, PTX_ERR_BAD_ARG, "single_attention: n=%d heads=%d", n, heads);
+  PTX_REQUIRE(d > 0 && d <= 32 && d % 8 == 0, PTX_ERR_UNSUPPORTED,
+              "single_attention: head dim must be 8, 16, 24 or 32 (got %d)", d);
+  PTX_REQUIRE(n <= 32768 && heads <= 65535, PTX_ERR_UNSUPPORTED, "single_attention: n=%d heads=%d too large",
+              n, heads);
+  if (n == 0 || heads == 0) return PTX_OK;
+  PTX_REQUIRE(q && k && vt && out, PTX_ERR_BAD_ARG, "single_attention: null pointer");
+  PTX_REQUIRE(ld % 8 == 0 && ldo % 8 == 0 && ldt % 8 == 0 && ldt >= ((n + 31) / 32) * 32 &&
+                  ld >= (int64_t)heads * d && ldo >= (int64_t)heads * d,
+              PTX_ERR_BAD_ARG,
+              "single_attention: pitches must be multiples of 8, ld / ldo >= heads * d and "
+              "ldt >= n rounded up to 32 (ld=%lld ldt=%lld ldo=%lld)",
+              (long long)ld, (long long)ldt, (long long)ldo);
+  PTX_REQUIRE(aligned16(q) && aligned16(k) && aligned16(vt) && aligned16(out) && (!g || aligned16(g)),
+              PTX_ERR_BAD_ARG, "single_attention: pointers must be 16-byte aligned");
+  PTX_DISPATCH(dtype, ptx::single_attention_fwd<T>(q, k, vt, g, bias, bias_f32, out, n, heads, d, ld,
+                                                   ldt, ldo, scale, (hipStream_t)stream));
+  return after_launch("single_attention");
+}
+
 PTX_API int ptx_pair_bias_fwd(const void* z, const void* ln_w, const void* ln_b, const void* w, void* bias,
                       int n, int c_z, int heads, int out_f32, float eps, int dtype,
                       void* stream) {

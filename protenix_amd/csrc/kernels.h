@@ -50,6 +50,25 @@ template <typename T, typename TZ = T>
 int pair_bias_fwd(const void* z, const void* ln_w, const void* ln_b, const void* w, void* bias,
                   int n, int c_z, int heads, int out_f32, float eps, hipStream_t stream);
 
+// Small linear layers of the single-representation track (single.hip):
+//   out[rows][n_out] = [res +] x[rows][k] w[n_out][k]^T [+ bias on columns < bias_cols];
+//   output columns >= split_col go, transposed, to out_t[n_out - split_col][ldt] instead
+//   (rows in [rows, ldt) written as zeros); out then has split_col columns.
+template <typename T>
+int linear_fwd(const void* x, const void* w, const void* bias, int bias_cols, const void* res,
+               void* out, void* out_t, int split_col, int64_t ldt, int rows, int k, int n_out,
+               hipStream_t stream);
+//   out[rows][hidden] = silu(x w_a^T) * (x w_b^T)
+template <typename T>
+int swiglu_fwd(const void* x, const void* w_a, const void* w_b, void* out, int rows, int k,
+               int hidden, hipStream_t stream);
+// out[n][heads*d] = sigmoid(g) * softmax_k(q k^T * scale + bias[h]) v per head; q, k, g rows of
+// pitch ld, vt [heads*d][ldt] (keys beyond n hold zeros), bias [heads][n][n] fp32 or T.
+template <typename T>
+int single_attention_fwd(const void* q, const void* k, const void* vt, const void* g,
+                         const void* bias, int bias_f32, void* out, int n, int heads, int d,
+                         int64_t ld, int64_t ldt, int64_t ldo, float scale, hipStream_t stream);
+
 // x[c][i][j] = sum_k a[c][i][k] * b[c][j][k] for `batch` independent products;
 // a, b rows have pitch k_pitch (a multiple of 64, >= n), x is dense [batch][n][n].
 template <typename T>

@@ -292,3 +292,81 @@ def pair_bias(z: torch.Tensor, ln_w: Optional[torch.Tensor], ln_b: Optional[torc
         _call("pair_bias", lib.ptx_pair_bias_fwd, _ptr(z), _ptr(ln_w), _ptr(ln_b), _ptr(w), _ptr(out), n, c,
                                          heads, int(out_f32), eps, _dt_stream(z, w.dtype), _stream())
     return out
+
+
+# ---------------------------------------------------------------- single-representation track
+def linear(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None,
+           res: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """[res +] x w^T [+ bias] for x [..., k], w [n_out, k] in x's dtype (k % 16 == 0,
+    n_out % 8 == 0), on the HIP kernel of the single track."""
+    _dev(x, "x")
+    lib = _lib.load()
+    k, n_out = x.shape[-1], w.shape[0]
+    x2 = x.reshape(-1, k)
+    if not x2.is_contiguous():
+        x2 = x2.contiguous()
+    rows = x2.shape[0]
+    out = torch.empty((rows, n_out), dtype=x.dtype, device=x.device)
+    r2 = None
+    if res is not None:
+        r2 = res.reshape(-1, n_out)
+        if not r2.is_contiguous():
+            r2 = r2.contiguous()
+    with torch.cuda.device(x.device):
+        _call("linear", lib.ptx_linear_fwd, _ptr(x2), _ptr(w), _ptr(bias), n_out if bias is not None else 0,
+              _ptr(r2), _ptr(out), None, n_out, 0, rows, k, n_out, _dt(x), _stream())
+    return out.view(*x.shape[:-1], n_out)
+
+
+def linear_split(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], bias_cols: int,
+                 split_col: int) -> Tuple[torch.Tensor, torch.Tensor]:
+    """x [rows, k] -> (y[:, :split_col] row-major, y[:, split_col:] transposed with the row axis
+    padded with zeros to a multiple of 32), y = x w^T (+ bias on the first bias_cols columns)."""
+    _dev(x, "x")
+    lib = _lib.load()
+    rows, k = x.shape
+    n_out = w.shape[0]
+    ldt = ((rows + 31) // 32) * 32
+    out = torch.empty((rows, split_col), dtype=x.dtype, device=x.device)
+    out_t = torch.empty((n_out - split_col, ldt), dtype=x.dtype, device=x.device)
+    with torch.cuda.device(x.device):
+        _call("linear", lib.ptx_linear_fwd, _ptr(x), _ptr(w), _ptr(bias), bias_cols, None, _ptr(out),
+              _ptr(out_t), split_col, ldt, rows, k, n_out, _dt(x), _stream())
+    return out, out_t
+
+
+def swiglu(x: torch.Tensor, w_a: torch.Tensor, w_b: torch.Tensor) -> torch.Tensor:
+    """silu(x w_a^T) * (x w_b^T) for x [..., k]."""
+    _dev(x, "x")
+    lib = _lib.load()
+    k, hidden = x.shape[-1], w_a.shape[0]
+    x2 = x.reshape(-1, k)
+    if not x2.is_contiguous():
+        x2 = x2.contiguous()
+    out = torch.empty((x2.shape[0], hidden), dtype=x.dtype, device=x.device)
+    with torch.cuda.device(x.device):
+        _call("swiglu", lib.ptx_swiglu_fwd, _ptr(x2), _ptr(w_a), _ptr(w_b), _ptr(out), x2.shape[0], k,
+              hidden, _dt(x), _stream())
+    return out.view(*x.shape[:-1], hidden)
+
+
+def single_attention(qkg: torch.Tensor, vt: torch.Tensor, bias: Optional[torch.Tensor], heads: int,
+                     d: int, scale: float, gated: bool = True) -> torch.Tensor:
+    """qkg [n, 3 * heads * d] (q | k | gate logits, head-major), vt [heads * d, ldt], bias
+    [heads, n, n] fp32 or qkg's dtype -> gated attention output [n, heads * d]."""
+    _dev(qkg, "qkg")
+    lib = _lib.load()
+    n, hd = qkg.shape[0], heads * d
+    es = qkg.element_size()
+    out = torch.empty((n, hd), dtype=qkg.dtype, device=qkg.device)
+    base = qkg.data_ptr()
+    if bias is not None:
+        if bias.dtype not in (torch.float32, qkg.dtype):
+            bias = bias.to(qkg.dtype)
+        bias = bias.contiguous()
+    with torch.cuda.device(qkg.device):
+        _call("single_attention", lib.ptx_single_attention_fwd, base, base + hd * es, _ptr(vt),
+              base + 2 * hd * es if gated else None, _ptr(bias),
+              int(bias is not None and bias.dtype == torch.float32),
+              _ptr(out), n, heads, d, qkg.shape[1], vt.shape[1], hd, float(scale), _dt(qkg), _stream())
+    return out

@@ -3,8 +3,8 @@
 Mirrors protenix/model/modules/primitives.py:33-101 (Linear / LinearNoBias),
 :166-230 (Transition) and protenix/model/triangular/layers.py:104-197
 (OpenfoldLinear, by its initialiser names).  The pair Transition (c_in = 64, 128, or 256 in bf16)
-runs on the fused HIP kernels; other widths (the single track, c_in = 384) use
-the HIP LayerNorm and library GEMMs.
+runs on the fused HIP kernel; other widths (the single track, c_in = 384) use
+the HIP LayerNorm and the small-GEMM kernels of the single track.
 """
 from __future__ import annotations
 
@@ -98,6 +98,7 @@ class Transition(nn.Module):
         self.linear_no_bias = LinearNoBias(n * c_in, c_in, initializer="zeros")
         self._cache = _WeightCache()
         self._cache_ab = _WeightCache()
+        self._cache_lib = _WeightCache()
 
     def _weights(self, dtype, device) -> dict:
         ps = (self.layernorm1.weight, self.layernorm1.bias, self.linear_no_bias_a.weight,
@@ -107,11 +108,16 @@ class Transition(nn.Module):
             return {"ln_w": ln_w, "ln_b": ln_b, "packed": ops.transition_pack(w_a, w_b, w_o)}
         return self._cache.get(ps, dtype, device, make)
 
-    def forward(self, x: torch.Tensor, _residual_out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    def forward(self, x: torch.Tensor, _residual_out: Optional[torch.Tensor] = None,
+                _residual_new: bool = False) -> torch.Tensor:
         """Returns the update; with `_residual_out` (may be x itself) writes
-        x + update there instead and returns it."""
+        x + update there instead and returns it; with `_residual_new` returns x + update in a
+        new tensor."""
         _forward_only(x, module=self)
-        add = _residual_out is not None
+        if _residual_new and _residual_out is None and (
+                self.c_in in (64, 128) or (self.c_in == 256 and x.dtype == torch.bfloat16)):
+            _residual_out = torch.empty_like(x)
+        add = _residual_out is not None or _residual_new
         cd = ops.compute_dtype(x)     # bf16 for fp32 rows of <= 128 channels under bf16 autocast
         fused = self.c_in in (64, 128) or (self.c_in == 256 and x.dtype == torch.bfloat16)
         if fused and (self.n * self.c_in) % 64 == 0:
@@ -120,18 +126,29 @@ class Transition(nn.Module):
             # (an update computed on fp32 rows under autocast holds bf16 values: returned in
             # the autocast dtype, like the reference's last linear)
             return out if (add or cd == x.dtype) else out.to(cd)
-        # other widths: HIP LayerNorm + library GEMMs (a and b as one GEMM on the stacked weights)
+        # other widths (the single track, c_in = 384): HIP LayerNorm, SwiGLU and output kernels
         y = self.layernorm1(x)
+        plain = all(l.precision is None for l in (self.linear_no_bias_a, self.linear_no_bias_b,
+                                                  self.linear_no_bias))
+        if (plain and not torch.is_grad_enabled() and x.is_cuda and self.c_in % 16 == 0
+                and (self.n * self.c_in) % 16 == 0 and x.dtype in (torch.float32, torch.bfloat16)):
+            ps = (self.linear_no_bias_a.weight, self.linear_no_bias_b.weight, self.linear_no_bias.weight)
+            w_a, w_b, w_o = self._cache_ab.get(ps, y.dtype, y.device, lambda: tuple(
+                _cv(p, y.dtype, y.device) for p in ps))
+            h = ops.swiglu(y, w_a, w_b)
+            u = ops.linear(h, w_o, res=x if add else None)
+            return u if _residual_out is None else _residual_out.copy_(u)
+        # library GEMMs (a and b as one GEMM on the stacked weights)
         if (not torch.is_grad_enabled() and self.linear_no_bias_a.precision is None
                 and self.linear_no_bias_b.precision is None):
             ps = (self.linear_no_bias_a.weight, self.linear_no_bias_b.weight)
-            w_ab = self._cache_ab.get(ps, y.dtype, y.device, lambda: torch.cat(
+            w_ab = self._cache_lib.get(ps, y.dtype, y.device, lambda: torch.cat(
                 [_cv(p, y.dtype, y.device) for p in ps], 0).contiguous())
             a, b = F.linear(y, w_ab).chunk(2, dim=-1)
             h = F.silu(a) * b
         else:
             h = F.silu(self.linear_no_bias_a(y)) * self.linear_no_bias_b(y)
         u = self.linear_no_bias(h)
-        if add:
+        if _residual_out is not None:
             return _residual_out.copy_(x + u) if _residual_out is not x else x.add_(u)
-        return u
+        return x + u if add else u

@@ -4,8 +4,9 @@ pairformer.py:98-100; attention arithmetic of primitives.py:233-291, 636-879).
 
 The only pass over the pair tensor - LayerNorm(z) followed by the c_z -> heads
 projection - runs on the fused HIP kernel and never materialises LN(z).  The
-rest lives on the [N, c_s] single track: HIP LayerNorm, library GEMMs, and an
-fp32 softmax over [heads, N, N].
+rest lives on the [N, c_s] single track, on HIP kernels as well: LayerNorm, one
+stacked projection, a flash-style attention that streams the pair bias and never
+materialises the [heads, N, N] logits, and the output projection.
 """
 from __future__ import annotations
 
@@ -45,40 +46,61 @@ class Attention(nn.Module):
         if zero_init:
             nn.init.zeros_(self.linear_o.weight)
         self._cache_in = _WeightCache()
+        self._cache_out = _WeightCache()
 
     def _fused_in(self, dtype, device):
-        """q, k, v and gate projections of one input as a single GEMM: the four weights
-        stacked (and the q bias padded with zeros), built once per weight set."""
-        ps = (self.linear_q.weight, self.linear_q.bias, self.linear_k.weight, self.linear_v.weight,
-              self.linear_g.weight)
+        """q, k, gate and v projections of one input as a single GEMM: the four weights
+        stacked in that order (v last: its columns leave the kernel transposed, which is how
+        the attention kernel reads them) and the q bias, built once per weight set."""
+        ps = (self.linear_q.weight, self.linear_q.bias, self.linear_k.weight, self.linear_g.weight,
+              self.linear_v.weight)
 
         def make():
-            wq, bq, wk, wv, wg = (_cv(p, dtype, device) for p in ps)
-            w = torch.cat([wq, wk, wv, wg], 0).contiguous()
-            b = torch.zeros(w.shape[0], dtype=dtype, device=device)
-            if bq is not None:
-                b[: wq.shape[0]] = bq
-            return w, b
+            wq, bq, wk, wg, wv = (_cv(p, dtype, device) for p in ps)
+            return torch.cat([wq, wk, wg, wv], 0).contiguous(), bq
         return self._cache_in.get(ps, dtype, device, make)
 
+    def _hip_eligible(self, q_x: torch.Tensor, kv_x: torch.Tensor) -> bool:
+        plain = all(l is not None and l.precision is None for l in
+                    (self.linear_q, self.linear_k, self.linear_v, self.linear_g, self.linear_o))
+        return (q_x is kv_x and plain and q_x.is_cuda and self.c_q == self.c_k == self.c_v
+                and self.c_q % 16 == 0 and self.c_hidden % 8 == 0 and self.c_hidden <= 32
+                and q_x.dtype in (torch.float32, torch.bfloat16) and not torch.is_grad_enabled())
+
     def forward(self, q_x: torch.Tensor, kv_x: torch.Tensor,
-                attn_bias: Optional[torch.Tensor] = None, **_unused) -> torch.Tensor:
-        H = self.num_heads
-        g_lin = None
-        plain = all(l.precision is None for l in (self.linear_q, self.linear_k, self.linear_v))
-        if (q_x is kv_x and self.linear_g is not None and plain and self.linear_g.precision is None
-                and self.c_q == self.c_k == self.c_v and not torch.is_grad_enabled()):
-            w, b = self._fused_in(q_x.dtype, q_x.device)
-            q, k, v, g_lin = torch.nn.functional.linear(q_x, w, b).chunk(4, dim=-1)
-            q, k, v = (t.unflatten(-1, (H, -1)).transpose(-2, -3) for t in (q, k, v))
-        else:
-            q = self.linear_q(q_x).unflatten(-1, (H, -1)).transpose(-2, -3)
-            k = self.linear_k(kv_x).unflatten(-1, (H, -1)).transpose(-2, -3)
-            v = self.linear_v(kv_x).unflatten(-1, (H, -1)).transpose(-2, -3)
+                attn_bias: Optional[torch.Tensor] = None, residual: Optional[torch.Tensor] = None,
+                **_unused) -> torch.Tensor:
+        """Attention update of q_x; with `residual`, residual + update (added in the output
+        projection's epilogue)."""
+        H, d = self.num_heads, self.c_hidden
+        if self._hip_eligible(q_x, kv_x):
+            # Three HIP kernels per batch element: stacked projection (q | k | gate row-major,
+            # v transposed), flash-style attention with the pair bias and the gate, output
+            # projection (+ residual).  Logits and softmax are fp32 and never materialised.
+            w, bq = self._fused_in(q_x.dtype, q_x.device)
+            w_o = self._cache_out.get((self.linear_o.weight,), q_x.dtype, q_x.device,
+                                      lambda: _cv(self.linear_o.weight, q_x.dtype, q_x.device))
+            n, c = q_x.shape[-2], q_x.shape[-1]
+            xb = q_x.reshape(-1, n, c)
+            if not xb.is_contiguous():
+                xb = xb.contiguous()
+            bb = None
+            if attn_bias is not None:
+                bb = attn_bias.expand(*q_x.shape[:-2], H, n, n).reshape(-1, H, n, n)
+            outs = []
+            for i in range(xb.shape[0]):
+                qkg, vt = ops.linear_split(xb[i], w, bq, H * d, 3 * H * d)
+                outs.append(ops.single_attention(qkg, vt, None if bb is None else bb[i], H, d,
+                                                 1.0 / math.sqrt(d)))
+            o = outs[0] if len(outs) == 1 else torch.stack(outs)
+            return ops.linear(o.view(*q_x.shape[:-1], H * d), w_o, res=residual)
+        q = self.linear_q(q_x).unflatten(-1, (H, -1)).transpose(-2, -3)
+        k = self.linear_k(kv_x).unflatten(-1, (H, -1)).transpose(-2, -3)
+        v = self.linear_v(kv_x).unflatten(-1, (H, -1)).transpose(-2, -3)
         q = q / math.sqrt(self.c_hidden)
         # logits, softmax and the weighted sum in fp32 (the reference upcasts q, k
         # and the bias and relies on autocast for v; here v is upcast as well)
-        d = q.dtype
+        dt = q.dtype
         # (shielded from autocast, which would run both products in its own dtype again - as
         # the reference shields its non-SDPA branch, primitives.py:269)
         with torch.autocast("cuda", enabled=False):
@@ -88,12 +110,11 @@ class Attention(nn.Module):
                     attn_bias = attn_bias.unsqueeze(-3)
                 w = w + attn_bias.float()
             w = torch.softmax(w, dim=-1)
-            o = torch.matmul(w, v.float()).to(d).transpose(-2, -3)
+            o = torch.matmul(w, v.float()).to(dt).transpose(-2, -3)
         if self.linear_g is not None:
-            if g_lin is None:
-                g_lin = self.linear_g(q_x)
-            o = o * torch.sigmoid(g_lin).unflatten(-1, (H, -1))
-        return self.linear_o(o.flatten(-2))
+            o = o * torch.sigmoid(self.linear_g(q_x)).unflatten(-1, (H, -1))
+        out = self.linear_o(o.flatten(-2))
+        return out if residual is None else residual + out
 
 
 class AttentionPairBias(nn.Module):
@@ -142,9 +163,10 @@ class AttentionPairBias(nn.Module):
             raise NotImplementedError("local attention belongs to the diffusion module")
         return self.forward_with_bias(a, self.pair_bias(z))
 
-    def forward_with_bias(self, a: torch.Tensor, bias: torch.Tensor) -> torch.Tensor:
-        """The single-track part, given bias = pair_bias(z).  Split off so that a
-        caller can run it on another stream once the pass over z is done."""
+    def forward_with_bias(self, a: torch.Tensor, bias: torch.Tensor,
+                          residual: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """The single-track part, given bias = pair_bias(z) (with `residual`: residual + update).
+        Split off so that a caller can run it on another stream once the pass over z is done."""
         _forward_only(a, bias, module=self)
         a = self.layernorm_a(a)
-        return self.attention(q_x=a, kv_x=a, attn_bias=bias)
+        return self.attention(q_x=a, kv_x=a, attn_bias=bias, residual=residual)
