@@ -199,12 +199,20 @@ __device__ __forceinline__ int key_of_mfma_row(int m) {
   return 16 * (m >> 4) + 8 * ((m >> 2) & 1) + 4 * ((m >> 3) & 1) + (m & 3);
 }
 
+// One workgroup per (32 queries, head); its kAttnWaves waves take every kAttnWaves-th block of
+// 32 keys each and merge their partial results through LDS in a fixed order: the chain of
+// dependent loads a wave walks through is a quarter as long.
+constexpr int kAttnWaves = 4;
+
 template <typename T>
-__global__ __launch_bounds__(64) void single_attention_kernel(SingleAttnParams p) {
+__global__ __launch_bounds__(kAttnWaves * 64) void single_attention_kernel(SingleAttnParams p) {
   typedef typename Vec8<T>::type V8;
   typedef typename Vec4<T>::type V4;
   constexpr float kL2e = 1.4426950408889634f;
+  __shared__ float part_o[kAttnWaves][16][kWave];
+  __shared__ float part_ml[kAttnWaves][2][kWave];
   const int lane = threadIdx.x & 63, ln = lane & 31, g = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int h = blockIdx.y, q0 = blockIdx.x * 32;
   const int n = p.n, d = p.d;
   const int qi = min(q0 + ln, n - 1);
@@ -233,7 +241,7 @@ __global__ __launch_bounds__(64) void single_attention_kernel(SingleAttnParams p
   for (int r = 0; r < 16; ++r) acc_o[r] = 0.0f;
   float m_run = -INFINITY, l_run = 0.0f;
 
-  for (int key0 = 0; key0 < n; key0 += 32) {
+  for (int key0 = 32 * wave; key0 < n; key0 += 32 * kAttnWaves) {
     const bool tail = key0 + 32 > n;   // the same for the whole wave
     // K fragments (A operand: lane <-> key, slots <-> channels)
     const T* kp = kbase + (int64_t)min(key0 + krow, n - 1) * p.ld;
@@ -316,7 +324,28 @@ __global__ __launch_bounds__(64) void single_attention_kernel(SingleAttnParams p
     for (int ks = 0; ks < 2; ++ks) mma32(acc_o, vf[ks], pf[ks]);   // lane <-> query, register <-> channel
   }
 
-  const float inv = fast_rcp(l_run + swap32(l_run));
+  // merge the waves' partial results (a wave without key blocks contributes m = -inf, l = 0)
+  l_run += swap32(l_run);
+#pragma unroll
+  for (int r = 0; r < 16; ++r) part_o[wave][r][lane] = acc_o[r];
+  part_ml[wave][0][lane] = m_run;
+  part_ml[wave][1][lane] = l_run;
+  __syncthreads();
+  if (wave != 0) return;
+  float m_all = part_ml[0][0][lane];
+#pragma unroll
+  for (int w = 1; w < kAttnWaves; ++w) m_all = fmaxf(m_all, part_ml[w][0][lane]);
+  l_run = 0.0f;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) acc_o[r] = 0.0f;
+#pragma unroll
+  for (int w = 0; w < kAttnWaves; ++w) {
+    const float f = fast_exp2(part_ml[w][0][lane] - m_all);   // wave 0 always has a block: m_all is finite
+    l_run += part_ml[w][1][lane] * f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc_o[r] += part_o[w][r][lane] * f;
+  }
+  const float inv = fast_rcp(l_run);
   if (q0 + ln < n) {
     const T* gp = p.g ? (const T*)p.g + (int64_t)qi * p.ld + h * d : nullptr;
     T* op = (T*)p.out + (int64_t)qi * p.ldo + h * d;
@@ -359,7 +388,7 @@ int single_attention_fwd(const void* q, const void* k, const void* vt, const voi
   p.heads = heads;
   p.d = d;
   p.scale = scale;
-  single_attention_kernel<T><<<dim3((n + 31) / 32, heads), dim3(64), 0, stream>>>(p);
+  single_attention_kernel<T><<<dim3((n + 31) / 32, heads), dim3(kAttnWaves * 64), 0, stream>>>(p);
   return 0;
 }
 
