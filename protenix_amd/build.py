@@ -15,9 +15,9 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libprotenix_amd.so")
 SOURCES = ["api.hip", "layernorm.hip", "rowgemm.hip", "triattn.hip", "attnpack.hip", "ntgemm.hip", "transition.hip", "single.hip"]
-# per-source extra flags: the attention kernel's max reductions need no NaN
-# canonicalisation (lets the compiler form v_max3_f32)
-EXTRA_FLAGS = {"triattn.hip": ["-fno-honor-nans"]}
+# per-source extra flags (none: the attention core's redo checks of the form !(x < limit) are
+# what catches a NaN logit, so it is built with NaNs honoured like everything else)
+EXTRA_FLAGS = {}
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",
     # keep the compiler from forming packed-fp32 VALU ops

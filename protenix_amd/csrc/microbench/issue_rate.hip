@@ -71,15 +71,15 @@ template <int KIND, int NV>
 static double run(const char* name, float* d, int waves, int cus, double per_iter) {
   const int iters = 20000;
   hipEvent_t e0, e1;
-  hipEventCreate(&e0);
-  hipEventCreate(&e1);
+  (void)hipEventCreate(&e0);
+  (void)hipEventCreate(&e1);
   loop_kernel<KIND, NV><<<cus, 256 * waves>>>(d, 200);
-  hipEventRecord(e0);
+  (void)hipEventRecord(e0);
   loop_kernel<KIND, NV><<<cus, 256 * waves>>>(d, iters);
-  hipEventRecord(e1);
-  hipEventSynchronize(e1);
+  (void)hipEventRecord(e1);
+  (void)hipEventSynchronize(e1);
   float ms = 0;
-  hipEventElapsedTime(&ms, e0, e1);
+  (void)hipEventElapsedTime(&ms, e0, e1);
   const double ns_iter = ms * 1e6 / ((double)iters * waves);   // per SIMD and loop iteration of one wave
   const double ns = ns_iter / per_iter;
   if (g_unit == 0.0f && KIND == kMul && waves == 4) g_unit = (float)ns;
@@ -122,6 +122,6 @@ int main() {
     printf("      sum %.1f  max %.1f\n", mf + 16 * ex, mf > 16 * ex ? mf : 16 * ex);
     (void)a8; (void)a32; (void)e16;
   }
-  hipFree(d);
+  (void)hipFree(d);
   return 0;
 }

@@ -190,6 +190,30 @@ def test_triattn_random_mask_large_logits():
     assert rel_err(got, want) <= 1e-4
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_triattn_nan_stays_where_the_reference_puts_it(dtype):
+    """A NaN at z[i0, j0] reaches, in the reference, row i0 (a poisoned key of that row) and the
+    queries at position i0 of every row (their triangle bias).  The fast softmax paths of the
+    attention core must not spread it any further, and everything else must still be right."""
+    ref, prod = oracle_and_product(O.TriangleAttention, P.TriangleAttention, 128, 32, 4, dtype=dtype)
+    n, i0, j0 = 160, 37, 101
+    z = _z(n, dtype)
+    z[0, i0, j0, 5] = float("nan")
+    with torch.no_grad():
+        want = ref(z.float(), None)
+        got = prod(z.cuda(), None).float().cpu()
+    bad = torch.isnan(want).any(-1)[0]
+    expect = torch.zeros(n, n, dtype=torch.bool)
+    expect[i0, :] = True
+    expect[:, i0] = True
+    assert torch.equal(bad, expect)                       # the oracle's own spread, as derived
+    assert torch.isnan(got[0][expect]).any(-1).all()      # poisoned where the reference is
+    clean = ~expect
+    assert torch.isfinite(got[0][clean]).all()
+    err = (got[0][clean] - want[0][clean]).abs().max() / want[0][clean].abs().max()
+    assert err <= tol(dtype)
+
+
 # ------------------------------------------------------------------ Transition / pair bias
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("shape", [(1, 50, 50, 128), (3001, 128), (1, 64, 384)])
