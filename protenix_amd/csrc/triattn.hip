@@ -106,6 +106,9 @@ __global__ __launch_bounds__((NWQ * 64), (sizeof(T) == 2 ? 16 / NWQ : 2)) void t
   // store nothing, and they are kept out of the wave-wide decisions below so that the path a
   // wave takes (and with it the rounding of its valid queries) never depends on that content.
   const bool q_ok = q0 + ln < n;
+  // (as a lane mask: wave-wide decisions are ballots of the condition alone, combined with this
+  // mask on the scalar unit)
+  const uint64_t q_ok_mask = __builtin_amdgcn_ballot_w64(q_ok);
 
   // Q fragments (B operand): lane <-> query, slots <-> d = 16*kk + 8*g + t
   V8 qf[R][2];
@@ -260,7 +263,7 @@ __global__ __launch_bounds__((NWQ * 64), (sizeof(T) == 2 ? 16 / NWQ : 2)) void t
       if (!MASKED) mt *= kLn2;
       // (a half whose keys all lie beyond n has mt = -inf: the reference stays where it is)
       float m_new = fmaxf(m_run[0], mt);
-      if (!MASKED && __ballot(q_ok && !(fabsf(m_new) < kZeroReferenceLimit)) == 0ull) m_new = 0.0f;
+      if (!MASKED && (__builtin_amdgcn_ballot_w64(!(fabsf(m_new) < kZeroReferenceLimit)) & q_ok_mask) == 0ull) m_new = 0.0f;
       alpha = m_new == -INFINITY ? 1.0f : fast_exp2((m_run[0] - m_new) * kLog2e);
       m_run[0] = m_new;
     }
@@ -301,7 +304,7 @@ __global__ __launch_bounds__((NWQ * 64), (sizeof(T) == 2 ? 16 / NWQ : 2)) void t
       }
     }
     if constexpr (MODE == kOptimistic || MODE == kOptimisticZero) {
-      if (__ballot(q_ok && !(psum < kOptimisticLimit)) != 0ull) return false;
+      if ((__builtin_amdgcn_ballot_w64(!(psum < kOptimisticLimit)) & q_ok_mask) != 0ull) return false;
     }
     out.psum = psum;
     out.alpha = alpha;
@@ -310,18 +313,20 @@ __global__ __launch_bounds__((NWQ * 64), (sizeof(T) == 2 ? 16 / NWQ : 2)) void t
   auto process_tile = [&](int tile, V8 (&tb)[2][2]) {
     static_assert(R == 1, "the register budget of four waves per SIMD holds one row per wave");
     const int buf = tile % 3;
-    const float mb_lane = lds_mb[buf][0][lane];
+    // keys of the tile with a non-zero mask bias, as a lane mask (key <-> lane); half u's keys
+    // are the lanes with bit 4 == u
+    const uint64_t mb_mask = __builtin_amdgcn_ballot_w64(lds_mb[buf][0][lane] != 0.0f);
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
       HalfOut out;
       bool rescale = true;
       // this half's keys are those of lanes with bit 4 == u
-      if (__ballot(mb_lane != 0.0f && ((lane >> 4) & 1) == u) != 0ull) {
+      if ((mb_mask & (u ? 0xffff0000ffff0000ull : 0x0000ffff0000ffffull)) != 0ull) {
         half_row(std::integral_constant<int, kMasked>{}, buf, u, tb[u], out);
       } else {
         bool done = false;
         if (tile != 0 || u != 0) {
-          if (__ballot(q_ok && m_run[0] != 0.0f) == 0ull)
+          if ((__builtin_amdgcn_ballot_w64(m_run[0] != 0.0f) & q_ok_mask) == 0ull)
             done = half_row(std::integral_constant<int, kOptimisticZero>{}, buf, u, tb[u], out);
           else
             done = half_row(std::integral_constant<int, kOptimistic>{}, buf, u, tb[u], out);
