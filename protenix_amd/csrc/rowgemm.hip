@@ -149,8 +149,9 @@ rowgemm_in_kernel(RowGemmInParams p) {
   constexpr bool MIXED = !std::is_same<T, TZ>::value;
   static_assert(!MIXED || (sizeof(T) == 2 && sizeof(TZ) == 4 && KS <= 8),
                 "mixed storage: bf16 arithmetic on fp32 rows of at most 128 channels");
-  // kTriMulOut on an fp32 residual stream keeps the raw rows in registers (see below)
-  constexpr bool kRegRes = MIXED && MODE == kTriMulOut;
+  // kTriMulOut with bf16 arithmetic on rows of at most 128 channels keeps the raw rows (as
+  // fp32) in registers for the residual add instead of a copy in LDS (see below)
+  constexpr bool kRegRes = MODE == kTriMulOut && sizeof(T) == 2 && KS <= 8;
   constexpr bool RES = IC::RES;
   constexpr int NW = IC::NW, SL = IC::SL, FPW = IC::FPW;
   __shared__ V8 lds_w[IC::NFRAG][kWave];
@@ -291,7 +292,8 @@ rowgemm_in_kernel(RowGemmInParams p) {
     if constexpr (RES) asm volatile("" : "+s"(gamma), "+s"(beta), "+s"(gamma2), "+s"(beta2));
 
   RowFrags<T, RB, KS> xf;
-  f32x8 zres[kRegRes ? RB : 1][kRegRes ? KS : 1];
+  // (the raw rows in their storage type: fp32 rows as fp32, bf16 rows as bf16 - half the registers)
+  typename Vec8<TZ>::type zres[kRegRes ? RB : 1][kRegRes ? KS : 1];
   if constexpr (MODE == kTriMulIn) {
     int64_t off[RB];
 #pragma unroll
@@ -391,7 +393,10 @@ rowgemm_in_kernel(RowGemmInParams p) {
         const TZ* rp = (const TZ*)p.x + p.xmap(pr) + 8 * g;
 #pragma unroll
         for (int kk = 0; kk < KS; ++kk) zres[rb][kk] = load8<TZ>(rp + 16 * kk);
-        normalize_row<T, KS, float, false>(zres[rb], lds_affine2[0], lds_affine2[1], p.eps, g, xf.f[rb]);
+        if constexpr (MIXED)
+          normalize_row<T, KS, float, false>(zres[rb], lds_affine2[0], lds_affine2[1], p.eps, g, xf.f[rb]);
+        else
+          normalize_raw<T, KS, float, false>(zres[rb], lds_affine2[0], lds_affine2[1], p.eps, g, xf.f[rb]);
       }
     }
   }
@@ -763,8 +768,8 @@ rowgemm_in_kernel(RowGemmInParams p) {
 #pragma unroll
           for (int c = 0; c < KS / 2; ++c)
             if (ch == c) {
-              zr[0] = zres[rb][2 * c];
-              zr[1] = zres[rb][2 * c + 1];
+              zr[0] = to_f32(zres[rb][2 * c]);
+              zr[1] = to_f32(zres[rb][2 * c + 1]);
             }
           wave_lds_sync();
 #pragma unroll
@@ -776,12 +781,15 @@ rowgemm_in_kernel(RowGemmInParams p) {
               // linear_z output rounded to T, times the gate, rounded to T: the update
               const float u = to_f32(from_f32<T>(to_f32(from_f32<T>(acc[rb][0][r])) *
                                                  sigmoidf_fast(acc[rb][1][r])));
+              // (bf16 rows: the sum is rounded once more on its way to the tile, like z + update)
               o[t] = p.add_residual ? zr[k2][t] + u : u;
             }
             // row n of the tile, columns 16*k2 + 8*g .. +7 (8-byte LDS stores)
-            f32x2* dst = reinterpret_cast<f32x2*>(stz + n * CZ::PITCH + 16 * k2 + 8 * g);
+            const typename Vec8<TZ>::type ov = from_f32<TZ>(o);
+            u32x2* dst = reinterpret_cast<u32x2*>(stz + n * CZ::PITCH + 16 * k2 + 8 * g);
+            const u32x2* src = reinterpret_cast<const u32x2*>(&ov);
 #pragma unroll
-            for (int h2 = 0; h2 < 4; ++h2) dst[h2] = f32x2{o[2 * h2], o[2 * h2 + 1]};
+            for (int h2 = 0; h2 < (int)sizeof(ov) / 8; ++h2) dst[h2] = src[h2];
           }
           wave_lds_sync();
 #pragma unroll
