@@ -233,6 +233,27 @@ PTX_API int ptx_triattn_core_fwd(const void* q, const void* k, const void* v, co
                          int n_rows, int s, int heads, int d, int dtype, void* stream);
 
 /*
+ * Backward of the operator above: the contract of TriAttentionFunction.backward
+ * (tri_attention/op.py:79-163; kernels tri_attention/backward.py:27-609: preprocess, dK/dV,
+ * dQ, dBias2).  With P = 2^(S log2 e - lse), S the logits of the forward, and
+ * Delta = sum_d O * dO:
+ *   dS = P * (dO V^T - Delta),  dV = P^T dO,  dK = dS^T Q,  dQ = dS K   per (batch, row, head)
+ *   dBias2[b][h][j][k] = sum over rows of dS[b][i][j][h][k]
+ *   q, k, v, o, dout, dq, dk, dv  [batch][n_rows][s][heads][d] contiguous, q as given to the forward
+ *   bias1, bias2, lse             as in the forward (lse is required here)
+ *   dbias2   [batch][heads][s][s] in `dtype`, or NULL to skip it
+ *   delta    fp32 scratch, n_rows * s * heads elements, uninitialised
+ * The gradient of Bias1 is not formed: the reference returns an uninitialised tensor for it
+ * (op.py:120, 157-163), its Bias1 being a mask that never requires a gradient.  P is
+ * recomputed from the logits; sums run in fp32 and every output is rounded once.
+ * dtype PTX_F32 or PTX_BF16.
+ */
+PTX_API int ptx_triattn_core_bwd(const void* q, const void* k, const void* v, const void* bias1,
+                         const void* bias2, const void* o, const float* lse, const void* dout,
+                         void* dq, void* dk, void* dv, void* dbias2, float* delta, int batch,
+                         int n_rows, int s, int heads, int d, int dtype, void* stream);
+
+/*
  * Triangle attention, stage 3 (layers.py:392-396 + the caller's residual add,
  * pairformer.py:189-213):  out(p) = [z(p) +] W_o o[p], where logical row p maps
  * to z[i][j] or, transposed = 1, z[j][i].  o [heads][n][n][d] as written by

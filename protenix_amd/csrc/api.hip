@@ -356,6 +356,39 @@ PTX_API int ptx_triattn_core_fwd(const void* q, const void* k, const void* v, co
   return after_launch("triattn_core_fwd");
 }
 
+PTX_API int ptx_triattn_core_bwd(const void* q, const void* k, const void* v, const void* bias1,
+                                 const void* bias2, const void* o, const float* lse,
+                                 const void* dout, void* dq, void* dk, void* dv, void* dbias2,
+                                 float* delta, int batch, int n_rows, int s, int heads, int d,
+                                 int dtype, void* stream) {
+  PTX_REQUIRE(dtype_ok(dtype), PTX_ERR_BAD_ARG, "triattn_core_bwd: unknown dtype %d", dtype);
+  PTX_REQUIRE(batch >= 0 && n_rows >= 0 && s >= 0 && heads >= 0, PTX_ERR_BAD_ARG,
+              "triattn_core_bwd: batch=%d n_rows=%d s=%d heads=%d", batch, n_rows, s, heads);
+  PTX_REQUIRE(d == 32, PTX_ERR_UNSUPPORTED, "triattn_core_bwd: only head dim 32 is built (got %d)", d);
+  PTX_REQUIRE(s <= 8192 && n_rows < 32768 && heads <= 64, PTX_ERR_UNSUPPORTED,
+              "triattn_core_bwd: n_rows=%d s=%d heads=%d too large", n_rows, s, heads);
+  if (batch == 0 || n_rows == 0 || s == 0 || heads == 0) return PTX_OK;
+  PTX_REQUIRE(q && k && v && bias2 && o && lse && dout && dq && dk && dv && delta, PTX_ERR_BAD_ARG,
+              "triattn_core_bwd: null pointer");
+  PTX_REQUIRE(aligned16(q) && aligned16(k) && aligned16(v) && aligned16(o) && aligned16(dout) &&
+                  aligned16(dq) && aligned16(dk) && aligned16(dv),
+              PTX_ERR_BAD_ARG, "triattn_core_bwd: pointers must be 16-byte aligned");
+  const int64_t n_q = (int64_t)n_rows * s * heads * 32, n_l = (int64_t)n_rows * s * heads;
+  const int64_t n_b2 = (int64_t)heads * s * s, n_b1 = (int64_t)n_rows * s;
+  const size_t es = esize(dtype);
+  for (int b = 0; b < batch; ++b) {
+    const int64_t oq = b * n_q * (int64_t)es;
+    const char* b1 = bias1 ? (const char*)bias1 + b * n_b1 * es : nullptr;
+    char* db2 = dbias2 ? (char*)dbias2 + b * n_b2 * es : nullptr;
+    PTX_DISPATCH(dtype, ptx::triattn_bwd<T>(
+                            (const char*)q + oq, (const char*)k + oq, (const char*)v + oq, b1,
+                            (const char*)bias2 + b * n_b2 * es, (const char*)o + oq, lse + b * n_l,
+                            (const char*)dout + oq, (char*)dq + oq, (char*)dk + oq, (char*)dv + oq,
+                            db2, delta, n_rows, s, heads, (hipStream_t)stream));
+  }
+  return after_launch("triattn_core_bwd");
+}
+
 PTX_API int ptx_triattn_output(const void* o, const void* w_o, const void* z, void* out, int n, int c_in,
                        int transposed, int add_residual, int dtype, void* stream) {
   PTX_REQUIRE(dtype_ok_z(dtype), PTX_ERR_BAD_ARG, "triattn_output: unknown dtype %d", dtype);

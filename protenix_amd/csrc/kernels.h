@@ -94,5 +94,12 @@ int triattn_fwd_ex(const T* q, const T* k, const T* vt, const T* g, const T* tri
 template <typename T>
 int triattn_pack(const T* q, const T* k, const T* v, const T* bias2, T* qs, T* kf, T* vtf, T* bf,
                  int n_rows, int n, int heads, int key_pitch, hipStream_t stream);
+// Backward of the standard-layout attention operator: dQ, dK, dV [n_rows][s][heads][32] and,
+// when db2 is given, dBias2 [heads][s][s], from Q (scaled), K, V, O, dO, the biases and the
+// forward's log2-sum-exp2; delta [n_rows][s][heads] is fp32 scratch.
+template <typename T>
+int triattn_bwd(const void* q, const void* k, const void* v, const void* b1, const void* b2,
+                const void* o, const float* lse, const void* dout, void* dq, void* dk, void* dv,
+                void* db2, float* delta, int n_rows, int s, int heads, hipStream_t stream);
 
 }  // namespace ptx
