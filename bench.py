@@ -250,6 +250,38 @@ def main() -> int:
                 "trimul_contract_ms": round(con3, 4),
                 "trimul_contract_frac_mfma": round(256.0 * 768 ** 3 / (con3 * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4),
                 "workload": "TriangleMultiplicationOutgoing + Incoming, bf16, N_token=768, last 48 tokens padded"}
+            # the attention operator on standard-layout tensors, forward and backward, bf16,
+            # at the headline's attention shape (768 rows x 768 positions x 4 heads x 32)
+            with torch.enable_grad():
+                gq = torch.Generator(device=dev).manual_seed(0)
+                qkv = [torch.randn(1, 768, 768, 4, 32, device=dev, generator=gq).to(BF16) for _ in range(4)]
+                qo, ko, vo = (t.requires_grad_(True) for t in qkv[:3])
+                do = qkv[3]
+                b1o = torch.zeros(1, 768, 1, 1, 768, device=dev, dtype=BF16)
+                b2o = torch.randn(1, 1, 4, 768, 768, device=dev, generator=gq).to(BF16).requires_grad_(True)
+                f_ms, b_ms = [], []
+                for it in range(8):
+                    e0, e1, e2 = ev(), ev(), ev()
+                    e0.record()
+                    oo = P.TriAttentionFunction.apply(qo * 0.1768, ko, vo, b1o, b2o)
+                    e1.record()
+                    oo.backward(do)
+                    e2.record()
+                    torch.cuda.synchronize()
+                    if it >= 2:
+                        f_ms.append(e0.elapsed_time(e1))
+                        b_ms.append(e1.elapsed_time(e2))
+                    qo.grad = ko.grad = vo.grad = b2o.grad = None
+                fm, bm = statistics.median(f_ms), statistics.median(b_ms)
+                shapes["triattn_operator_fwd_bwd_768x768x4x32_bf16"] = {
+                    "fwd_ms": round(fm, 3), "bwd_ms": round(bm, 3),
+                    "bwd_frac_mfma": round(1280.0 * 768 ** 3 / (bm * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4),
+                    "algorithmic": "backward: 5 products of 2 * 768^3 * 4 * 32 flop (dV, dP, dS^T Q, dS K, "
+                                   "and the logits once); the kernels recompute the logits and dP in each of "
+                                   "three passes, 10 products executed",
+                    "workload": "TriAttentionFunction.apply + backward (dQ, dK, dV, dBias2); fwd_ms includes "
+                                "the scaling of Q and the repack of the operands into the core's tile order"}
+                del qkv, qo, ko, vo, do, b1o, b2o, oo
             # stand-alone LayerNorm over c_z = 128 on the pair tensor's rows
             for dt, name in ((BF16, "bf16"), (torch.float32, "fp32")):
                 x = torch.randn(768 * 768, 128, device=dev, dtype=dt)
