@@ -275,13 +275,19 @@ rowgemm_in_kernel(RowGemmInParams p) {
 
   while (true) {
     if (RES && tile >= n_tiles) break;
-    const int64_t row0 = tile * (RB * 32);
+    // The projections at the head of an update walk the pair tensor back to front.  The kernel
+    // before them has just written it front to back, so its tail is what the 256 MB memory-side
+    // cache still holds; read front to back, a tensor larger than that cache evicts its own
+    // tail before reaching it.
+    constexpr bool kBackward = MODE == kTriMulIn || MODE == kTriAttnIn;
+    const int64_t wtile = (kBackward && tile < n_tiles) ? n_tiles - 1 - tile : tile;
+    const int64_t row0 = wtile * (RB * 32);
     int pi0 = 0, pk0 = 0;
     if constexpr (MODE == kTriMulIn) {
-      const uint32_t vb = (uint32_t)(tile >> 2);
+      const uint32_t vb = (uint32_t)(wtile >> 2);
       const uint32_t ip = vb / n_kb;
       pk0 = (int)(vb - ip * n_kb) * 8;
-      pi0 = (int)ip * (16 * RB) + (int)(tile & 3) * (4 * RB);
+      pi0 = (int)ip * (16 * RB) + (int)(wtile & 3) * (4 * RB);
     }
     // (resident: made opaque per tile, or the affine parameters' loads and conversions are
     // hoisted out of the tile loop and held in registers)

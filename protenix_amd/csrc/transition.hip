@@ -100,7 +100,9 @@ __global__ __launch_bounds__((TrCfg<T, KS>::NW * 64)) void transition_fused_kern
                 "the staging tiles reuse the chunk buffers");
 
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int64_t row0 = ((int64_t)blockIdx.x * NW + wave) * (RB * 32);
+  // Workgroups take the rows back to front: the kernel before this one wrote the pair tensor
+  // front to back, and its tail is what the memory-side cache still holds.
+  const int64_t row0 = ((int64_t)(gridDim.x - 1 - blockIdx.x) * NW + wave) * (RB * 32);
 
   // chunk j (clamped for the address) -> buffer j % NBUF; every wave moves FPW fragments
   // (address = wave-uniform base in scalar registers + this lane's offset inside a fragment:
