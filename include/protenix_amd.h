@@ -284,6 +284,21 @@ PTX_API int ptx_transition_fwd(const void* x, const void* ln_w, const void* ln_b
                        int dtype, void* stream);
 
 /*
+ * The pair transition and the pair bias that follows it in a Pairformer block
+ * (pairformer.py:215-222: z = z + pair_transition(z); then attention_pair_bias reads z through
+ * transformer.py:191-194), in one launch: ptx_transition_fwd, and from the finished rows, while
+ * they pass through the kernel's epilogue,
+ *   bias[h][row] = (pb_w LN_pb(out[row]))[h]      pb_w [heads][c], heads <= 32
+ * as ptx_pair_bias_fwd computes it from the stored tensor (which would read it once more).
+ * bias is fp32 when bias_f32 = 1, else bf16.  c = 128; dtype PTX_BF16 or PTX_MIXED.
+ */
+PTX_API int ptx_transition_pair_bias_fwd(const void* x, const void* ln_w, const void* ln_b,
+                                 const void* packed, void* out, int64_t rows, int c, int n_factor,
+                                 int add_residual, float eps, const void* pb_ln_w,
+                                 const void* pb_ln_b, const void* pb_w, void* bias, int heads,
+                                 int bias_f32, float pb_eps, int dtype, void* stream);
+
+/*
  * Pair bias of the single-representation attention (transformer.py:191-194):
  *   bias[h][i][j] = (W LN(z[i][j]))[h],  W [heads][c_z], heads <= 32, c_z = 128 or
  * (bf16 only) 256.

@@ -453,6 +453,43 @@ PTX_API int ptx_transition_fwd(const void* x, const void* ln_w, const void* ln_b
   return after_launch("transition");
 }
 
+PTX_API int ptx_transition_pair_bias_fwd(const void* x, const void* ln_w, const void* ln_b,
+                                         const void* packed, void* out, int64_t rows, int c,
+                                         int n_factor, int add_residual, float eps,
+                                         const void* pb_ln_w, const void* pb_ln_b, const void* pb_w,
+                                         void* bias, int heads, int bias_f32, float pb_eps,
+                                         int dtype, void* stream) {
+  PTX_REQUIRE(dtype == PTX_BF16 || dtype == PTX_MIXED, PTX_ERR_UNSUPPORTED,
+              "transition_pair_bias: built for PTX_BF16 and PTX_MIXED only (got dtype %d)", dtype);
+  PTX_REQUIRE(rows >= 0 && n_factor > 0, PTX_ERR_BAD_ARG, "transition_pair_bias: rows=%lld n_factor=%d",
+              (long long)rows, n_factor);
+  PTX_REQUIRE(c == 128, PTX_ERR_UNSUPPORTED, "transition_pair_bias: only c = 128 is built (got %d)", c);
+  PTX_REQUIRE((n_factor * c) % 64 == 0 && n_factor <= 64, PTX_ERR_UNSUPPORTED,
+              "transition_pair_bias: n_factor=%d", n_factor);
+  PTX_REQUIRE(heads >= 1 && heads <= 32, PTX_ERR_UNSUPPORTED, "transition_pair_bias: heads=%d (1..32)",
+              heads);
+  PTX_REQUIRE(rows < ((int64_t)1 << 30), PTX_ERR_UNSUPPORTED, "transition_pair_bias: rows=%lld too large",
+              (long long)rows);
+  if (rows == 0) return PTX_OK;
+  PTX_REQUIRE(x && packed && out && pb_w && bias, PTX_ERR_BAD_ARG, "transition_pair_bias: null pointer");
+  PTX_REQUIRE(aligned16(x) && aligned16(packed) && aligned16(out) && aligned16(pb_w) && aligned16(bias) &&
+                  (!ln_w || aligned16(ln_w)) && (!ln_b || aligned16(ln_b)) &&
+                  (!pb_ln_w || aligned16(pb_ln_w)) && (!pb_ln_b || aligned16(pb_ln_b)),
+              PTX_ERR_BAD_ARG, "transition_pair_bias: pointers must be 16-byte aligned");
+  int rc;
+  if (dtype == PTX_MIXED)
+    rc = ptx::transition_pair_bias_fwd<ptx::bf16_t, float>(x, ln_w, ln_b, packed, out, rows, n_factor,
+                                                         add_residual, eps, pb_ln_w, pb_ln_b, pb_w, bias,
+                                                         heads, bias_f32, pb_eps, (hipStream_t)stream);
+  else
+    rc = ptx::transition_pair_bias_fwd<ptx::bf16_t, ptx::bf16_t>(x, ln_w, ln_b, packed, out, rows, n_factor,
+                                                               add_residual, eps, pb_ln_w, pb_ln_b, pb_w,
+                                                               bias, heads, bias_f32, pb_eps,
+                                                               (hipStream_t)stream);
+  PTX_REQUIRE(rc == 0, PTX_ERR_UNSUPPORTED, "transition_pair_bias: not built for this type");
+  return after_launch("transition_pair_bias");
+}
+
 PTX_API int ptx_linear_fwd(const void* x, const void* w, const void* bias, int bias_cols,
                            const void* res, void* out, void* out_t, int split_col, int64_t ldt,
                            int rows, int k, int n_out, int dtype, void* stream) {

@@ -46,6 +46,14 @@ template <typename T, typename TZ = T>
 int transition_fwd(const void* x, const void* ln_w, const void* ln_b, const void* packed,
                    void* out, int64_t rows, int c, int n_factor, int add_residual, float eps,
                    hipStream_t stream);
+// The transition on rows of 128 channels (16-bit arithmetic) with the pair bias of the single
+// attention, bias[h][row] = (W LN_pb(out[row]))[h], formed from the finished rows in its epilogue.
+template <typename T, typename TZ = T>
+int transition_pair_bias_fwd(const void* x, const void* ln_w, const void* ln_b, const void* packed,
+                             void* out, int64_t rows, int n_factor, int add_residual, float eps,
+                             const void* pb_ln_w, const void* pb_ln_b, const void* pb_w,
+                             void* bias, int heads, int bias_f32, float pb_eps,
+                             hipStream_t stream);
 template <typename T, typename TZ = T>
 int pair_bias_fwd(const void* z, const void* ln_w, const void* ln_b, const void* w, void* bias,
                   int n, int c_z, int heads, int out_f32, float eps, hipStream_t stream);

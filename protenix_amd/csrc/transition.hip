@@ -83,11 +83,22 @@ __global__ void transition_pack_kernel(const T* __restrict__ w_a, const T* __res
 
 // TZ: storage type of x and out (float with T = bf16: rows of an fp32 residual stream are
 // normalised in fp32 and rounded to T; the T-rounded update is added to the fp32 row).
-template <typename T, int KS, typename TZ = T>
+// PB: the pair bias of the single-representation attention that follows the transition in
+// a Pairformer block, bias[h][row] = (W LN_pb(out[row]))[h], formed from the finished rows
+// while they pass through the epilogue (a kernel of its own would read the pair tensor once
+// more for it).
+struct PairBiasArgs {
+  const void *gamma, *beta, *w;   // LayerNorm of the bias (either may be null), W [heads][c]
+  void* out;                      // [heads][n_rows], fp32 or T
+  int heads, out_f32;
+  float eps;
+};
+
+template <typename T, int KS, typename TZ = T, bool PB = false>
 __global__ __launch_bounds__((TrCfg<T, KS>::NW * 64)) void transition_fused_kernel(
     const TZ* x, const T* __restrict__ gamma, const T* __restrict__ beta,
     const T* __restrict__ packed, TZ* out, int64_t n_rows, int n_chunks, int add_residual,
-    float eps) {
+    float eps, PairBiasArgs pb) {
   typedef typename Vec8<T>::type V8;
   typedef typename VecE<TZ>::type VE_t;
   typedef TrCfg<T, KS> G;
@@ -260,6 +271,7 @@ __global__ __launch_bounds__((TrCfg<T, KS>::NW * 64)) void transition_fused_kern
   // every wave is past its last fragment read and all loads have landed) ----
   ring_barrier<0>();
   TZ* st = reinterpret_cast<TZ*>(&lds_w[0][0][0][0]) + wave * (32 * C::PITCH);
+  VE_t done[PB ? RB : 1][PB ? NOB : 1][PB ? C::NPASS : 1];   // PB: the finished rows, as stored
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
 #pragma unroll
@@ -275,10 +287,111 @@ __global__ __launch_bounds__((TrCfg<T, KS>::NW * 64)) void transition_fused_kern
       for (int ps = 0; ps < C::NPASS; ++ps) {
         int mj, m0;
         stage_coord<TZ>(ps, lane, mj, m0);
+        VE_t v = stage_get_vec<TZ>(st, mj, m0);
         if (obase[rb][ps] >= 0) {
-          VE_t v = stage_get_vec<TZ>(st, mj, m0);
           if (add_residual) v = add_vec<TZ>(v, resv[rb][ob][ps]);
           *reinterpret_cast<VE_t*>(out + obase[rb][ps] + ob * 32) = v;
+        }
+        if constexpr (PB) done[rb][ob][ps] = v;
+      }
+    }
+  }
+
+  if constexpr (PB) {
+    static_assert(!PB || (RB == 1 && sizeof(T) == 2), "pair-bias epilogue: one row block, 16-bit arithmetic");
+    // The bias' weights and LayerNorm parameters, requested before anything that waits: W as A
+    // fragments (rows beyond `heads` re-read the last head: those accumulator rows are not
+    // stored), gamma / beta for the columns this lane normalises.
+    const int n = lane & 31, g = lane >> 5;
+    V8 wf[KS];
+#pragma unroll
+    for (int kk = 0; kk < KS; ++kk)
+      wf[kk] = load8<T>((const T*)pb.w + (int64_t)min(n, pb.heads - 1) * kCx + 16 * kk + 8 * g);
+    const T* pg = pb.gamma ? (const T*)pb.gamma : default_gamma<T>();
+    const T* pbeta = pb.beta ? (const T*)pb.beta : default_beta<T>();
+    bf16x4 gm[NOB][C::VE / 4], bt[NOB][C::VE / 4];
+    {
+      const int m0 = (lane % C::LPM) * C::VE;   // as stage_coord: the same columns in every pass
+#pragma unroll
+      for (int ob = 0; ob < NOB; ++ob)
+#pragma unroll
+        for (int q4 = 0; q4 < C::VE / 4; ++q4) {
+          gm[ob][q4] = *reinterpret_cast<const bf16x4*>(pg + ob * 32 + m0 + 4 * q4);
+          bt[ob][q4] = *reinterpret_cast<const bf16x4*>(pbeta + ob * 32 + m0 + 4 * q4);
+        }
+    }
+    // LayerNorm statistics of the finished rows (as stored: TZ), two passes in fp32.  In the
+    // read-back layout a row's 32 columns of one block sit in LPM neighbouring lanes.
+    float mean[C::NPASS], rstd[C::NPASS];
+#pragma unroll
+    for (int ps = 0; ps < C::NPASS; ++ps) {
+      float sum = 0.0f;
+#pragma unroll
+      for (int ob = 0; ob < NOB; ++ob)
+#pragma unroll
+        for (int e = 0; e < C::VE; ++e) sum += to_f32(done[0][ob][ps][e]);
+#pragma unroll
+      for (int o = 1; o < C::LPM; o <<= 1) sum += __shfl_xor(sum, o, 64);
+      mean[ps] = sum * (1.0f / kCx);
+      float q = 0.0f;
+#pragma unroll
+      for (int ob = 0; ob < NOB; ++ob)
+#pragma unroll
+        for (int e = 0; e < C::VE; ++e) {
+          const float d = to_f32(done[0][ob][ps][e]) - mean[ps];
+          q += d * d;
+        }
+#pragma unroll
+      for (int o = 1; o < C::LPM; o <<= 1) q += __shfl_xor(q, o, 64);
+      rstd[ps] = rsqrtf(q * (1.0f / kCx) + pb.eps);
+    }
+    // per wave: 32 rows x 64 normalised columns in T, behind all waves' staging tiles (other
+    // waves may still be storing their rows)
+    constexpr int kPitchN = 64 + 4;      // elements: 34 dwords, rows 8-byte aligned
+    static_assert(NW * 32 * (C::PITCH * sizeof(TZ) + kPitchN * sizeof(T)) <=
+                      sizeof(u32x4_t) * (NBUF - 1) * kTrFrags * PIECES * kWave,
+                  "staging tiles and normalised tiles fit the chunk buffers");
+    T* stn = reinterpret_cast<T*>(reinterpret_cast<TZ*>(&lds_w[0][0][0][0]) + NW * (32 * C::PITCH)) +
+             wave * (32 * kPitchN);
+    f32x16 accb;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) accb[r] = 0.0f;
+#pragma unroll
+    for (int hb = 0; hb < NOB / 2; ++hb) {   // 64 columns at a time
+      wave_lds_sync();
+#pragma unroll
+      for (int o2 = 0; o2 < 2; ++o2)
+#pragma unroll
+        for (int ps = 0; ps < C::NPASS; ++ps) {
+          int mj, m0;
+          stage_coord<TZ>(ps, lane, mj, m0);
+          const int ob = 2 * hb + o2;
+#pragma unroll
+          for (int e4 = 0; e4 < C::VE; e4 += 4) {
+            f32x4 o;
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              o[e] = (to_f32(done[0][ob][ps][e4 + e]) - mean[ps]) * rstd[ps] * (float)gm[ob][e4 / 4][e] +
+                     (float)bt[ob][e4 / 4][e];
+            *reinterpret_cast<bf16x4*>(stn + mj * kPitchN + 32 * o2 + m0 + e4) = from_f32<T>(o);   // 8 bytes
+          }
+        }
+      wave_lds_sync();
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const u32x2* src = reinterpret_cast<const u32x2*>(stn + n * kPitchN + 16 * u + 8 * g);
+        u32x2 h2[2] = {src[0], src[1]};
+        mma32(accb, wf[4 * hb + u], *reinterpret_cast<const V8*>(h2));   // lane <-> row, register <-> head
+      }
+    }
+    const int64_t pr = row0 + n;
+    if (pr < n_rows) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int head = acc_row(r, g);
+        if (head < pb.heads) {
+          if (pb.out_f32) ((float*)pb.out)[(int64_t)head * n_rows + pr] = accb[r];
+          else ((T*)pb.out)[(int64_t)head * n_rows + pr] = from_f32<T>(accb[r]);
         }
       }
     }
@@ -310,10 +423,32 @@ static int transition_fwd_ks(const void* x, const void* ln_w, const void* ln_b, 
                              hipStream_t stream) {
   const int64_t rows_per_block = TrCfg<T, KS>::NW * TrCfg<T, KS>::RB * 32;
   const int64_t blocks = (rows + rows_per_block - 1) / rows_per_block;
-  transition_fused_kernel<T, KS, TZ><<<dim3((unsigned)blocks), dim3(TrCfg<T, KS>::NW * 64), 0, stream>>>(
+  transition_fused_kernel<T, KS, TZ, false><<<dim3((unsigned)blocks), dim3(TrCfg<T, KS>::NW * 64), 0, stream>>>(
       (const TZ*)x, (const T*)ln_w, (const T*)ln_b, (const T*)packed, (TZ*)out, rows,
-      16 * KS * n_factor / 32, add_residual, eps);
+      16 * KS * n_factor / 32, add_residual, eps, PairBiasArgs{});
   return 0;
+}
+
+template <typename T, typename TZ>
+int transition_pair_bias_fwd(const void* x, const void* ln_w, const void* ln_b, const void* packed,
+                             void* out, int64_t rows, int n_factor, int add_residual, float eps,
+                             const void* pb_ln_w, const void* pb_ln_b, const void* pb_w,
+                             void* bias, int heads, int bias_f32, float pb_eps,
+                             hipStream_t stream) {
+  if (rows == 0) return 0;
+  if constexpr (sizeof(T) == 2) {
+    constexpr int KS = 8;
+    static_assert(TrCfg<T, KS>::RB == 1, "the pair-bias epilogue handles one row block per wave");
+    const int64_t rows_per_block = TrCfg<T, KS>::NW * 32;
+    const int64_t blocks = (rows + rows_per_block - 1) / rows_per_block;
+    const PairBiasArgs pb = {pb_ln_w, pb_ln_b, pb_w, bias, heads, bias_f32, pb_eps};
+    transition_fused_kernel<T, KS, TZ, true><<<dim3((unsigned)blocks), dim3(TrCfg<T, KS>::NW * 64), 0, stream>>>(
+        (const TZ*)x, (const T*)ln_w, (const T*)ln_b, (const T*)packed, (TZ*)out, rows,
+        16 * KS * n_factor / 32, add_residual, eps, pb);
+    return 0;
+  } else {
+    return 1;   // 16-bit arithmetic only (the caller checks)
+  }
 }
 
 template <typename T, typename TZ>
@@ -346,5 +481,13 @@ template int transition_fwd<bf16_t, bf16_t>(const void*, const void*, const void
                                             void*, int64_t, int, int, int, float, hipStream_t);
 template int transition_fwd<bf16_t, float>(const void*, const void*, const void*, const void*,
                                            void*, int64_t, int, int, int, float, hipStream_t);
+template int transition_pair_bias_fwd<bf16_t, bf16_t>(const void*, const void*, const void*,
+                                                      const void*, void*, int64_t, int, int, float,
+                                                      const void*, const void*, const void*, void*,
+                                                      int, int, float, hipStream_t);
+template int transition_pair_bias_fwd<bf16_t, float>(const void*, const void*, const void*,
+                                                     const void*, void*, int64_t, int, int, float,
+                                                     const void*, const void*, const void*, void*,
+                                                     int, int, float, hipStream_t);
 
 }  // namespace ptx

@@ -260,9 +260,12 @@ def transition_pack(w_a: torch.Tensor, w_b: torch.Tensor, w_o: torch.Tensor) -> 
 
 
 def transition(x: torch.Tensor, w: dict, n_factor: int, add_residual: bool,
-               out: Optional[torch.Tensor] = None, eps: float = 1e-5) -> torch.Tensor:
+               out: Optional[torch.Tensor] = None, eps: float = 1e-5,
+               pair_bias_w: Optional[tuple] = None):
     """x [..., c] -> [x +] W_o(silu(W_a LN x) * W_b LN x), c = 64 or 128; `w["packed"]` comes from
-    transition_pack."""
+    transition_pack.  With `pair_bias_w = (ln_w, ln_b, w [heads, c])` (c = 128, bf16 arithmetic)
+    the same launch also forms the pair bias of the finished rows and the result is
+    (out, bias fp32 [heads, rows]) - what pair_bias() would compute from `out`."""
     _dev(x, "x")
     lib = _lib.load()
     c = x.shape[-1]
@@ -275,9 +278,16 @@ def transition(x: torch.Tensor, w: dict, n_factor: int, add_residual: bool,
         out = torch.empty_like(x2)
     o2 = out.view(-1, c)
     with torch.cuda.device(x.device):
-        _call("transition", lib.ptx_transition_fwd, _ptr(x2), _ptr(w["ln_w"]), _ptr(w["ln_b"]),
-              _ptr(w["packed"]), _ptr(o2), rows, c, n_factor, int(add_residual), eps, dt, st)
-    return out.view(x.shape)
+        if pair_bias_w is None:
+            _call("transition", lib.ptx_transition_fwd, _ptr(x2), _ptr(w["ln_w"]), _ptr(w["ln_b"]),
+                  _ptr(w["packed"]), _ptr(o2), rows, c, n_factor, int(add_residual), eps, dt, st)
+            return out.view(x.shape)
+        pln_w, pln_b, pw = pair_bias_w
+        bias = torch.empty((pw.shape[0], rows), dtype=torch.float32, device=x.device)
+        _call("transition", lib.ptx_transition_pair_bias_fwd, _ptr(x2), _ptr(w["ln_w"]), _ptr(w["ln_b"]),
+              _ptr(w["packed"]), _ptr(o2), rows, c, n_factor, int(add_residual), eps, _ptr(pln_w),
+              _ptr(pln_b), _ptr(pw.contiguous()), _ptr(bias), pw.shape[0], 1, eps, dt, st)
+    return out.view(x.shape), bias
 
 
 def pair_bias(z: torch.Tensor, ln_w: Optional[torch.Tensor], ln_b: Optional[torch.Tensor],

@@ -67,20 +67,37 @@ class PairformerBlock(nn.Module):
             return self._forward_autocast_unfused(s, z, pair_mask, ac)
         # (fp32 z under bf16 autocast: the same fused kernels, reading and updating the fp32
         # rows in place with bf16 arithmetic)
-        self._pair_track(z, pair_mask)
+        bias = self._pair_track(z, pair_mask, want_bias=self.c_s > 0)
         if self.c_s > 0:
-            s = self._single_track(s, self.attention_pair_bias.pair_bias(z))
+            s = self._single_track(s, bias)
         return s, z
 
-    def _pair_track(self, z: torch.Tensor, pair_mask: Optional[torch.Tensor]) -> None:
-        """The five pair updates, each "z += f(z)" fused into a kernel epilogue."""
+    def _pair_track(self, z: torch.Tensor, pair_mask: Optional[torch.Tensor],
+                    want_bias: bool = False) -> Optional[torch.Tensor]:
+        """The five pair updates, each "z += f(z)" fused into a kernel epilogue.  With
+        `want_bias`, also the pair bias of the single attention, read off the finished z: in
+        the transition's own epilogue where that kernel has one, by a kernel of its own
+        otherwise."""
         self.tri_mul_out(z, mask=pair_mask, inplace_safe=True, _add_with_inplace=True)
         self.tri_mul_in(z, mask=pair_mask, inplace_safe=True, _add_with_inplace=True)
         self.tri_att_start._run(z, pair_mask, transposed=False, residual_inplace=True)
         # ending node: the starting-node module of the reference applied to z^T with
         # mask^T, expressed through transposed addressing of z and mask
         self.tri_att_end._run(z, pair_mask, transposed=True, residual_inplace=True)
+        if not want_bias:
+            self.pair_transition(z, _residual_out=z)
+            return None
+        apb = self.attention_pair_bias
+        n = z.shape[-2]
+        if z.is_contiguous() and self.pair_transition.fuses_pair_bias(z, apb.n_heads):
+            # (one launch per pair tensor of a batch: the epilogue writes [heads][rows])
+            pbw = apb.pair_bias_weights(z)
+            zb = z.view(-1, n, n, z.shape[-1])
+            bias = [self.pair_transition(zi, _residual_out=zi, _pair_bias_w=pbw)[1] for zi in zb]
+            bias = bias[0] if len(bias) == 1 else torch.stack(bias)
+            return bias.view(*z.shape[:-3], apb.n_heads, n, n)
         self.pair_transition(z, _residual_out=z)
+        return apb.pair_bias(z)
 
     def _forward_autocast_unfused(self, s: Optional[torch.Tensor], z: torch.Tensor,
                                   pair_mask: Optional[torch.Tensor], ac: torch.dtype
@@ -156,8 +173,7 @@ class PairformerStack(nn.Module):
         side = self._side_stream(z.device)
         side.wait_stream(main)
         for blk in self.blocks:
-            blk._pair_track(z, pair_mask)
-            bias = blk.attention_pair_bias.pair_bias(z)   # reads z before the next block writes it
+            bias = blk._pair_track(z, pair_mask, want_bias=True)   # (bias: from z before the next block writes it)
             ready = main.record_event()
             with torch.cuda.stream(side):
                 side.wait_event(ready)

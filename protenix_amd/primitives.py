@@ -108,12 +108,23 @@ class Transition(nn.Module):
             return {"ln_w": ln_w, "ln_b": ln_b, "packed": ops.transition_pack(w_a, w_b, w_o)}
         return self._cache.get(ps, dtype, device, make)
 
+    def fuses_pair_bias(self, x: torch.Tensor, heads: int) -> bool:
+        """Whether forward(x, _pair_bias_w=...) is available: rows of 128 channels in bf16
+        arithmetic (bf16 rows, or fp32 rows under bf16 autocast), at most 32 heads."""
+        return (self.c_in == 128 and (self.n * self.c_in) % 64 == 0 and heads <= 32 and x.is_cuda
+                and ops.compute_dtype(x) == torch.bfloat16)
+
     def forward(self, x: torch.Tensor, _residual_out: Optional[torch.Tensor] = None,
-                _residual_new: bool = False) -> torch.Tensor:
+                _residual_new: bool = False, _pair_bias_w: Optional[tuple] = None):
         """Returns the update; with `_residual_out` (may be x itself) writes
         x + update there instead and returns it; with `_residual_new` returns x + update in a
-        new tensor."""
+        new tensor.  With `_pair_bias_w = (ln_w, ln_b, w)` (bf16; see fuses_pair_bias) and a
+        residual output, returns (x + update, fp32 bias [heads, rows]) from one launch."""
         _forward_only(x, module=self)
+        if _pair_bias_w is not None:
+            assert _residual_out is not None and self.fuses_pair_bias(x, _pair_bias_w[2].shape[0])
+            return ops.transition(x, self._weights(torch.bfloat16, x.device), self.n, add_residual=True,
+                                  out=_residual_out, pair_bias_w=_pair_bias_w)
         if _residual_new and _residual_out is None and (
                 self.c_in in (64, 128) or (self.c_in == 256 and x.dtype == torch.bfloat16)):
             _residual_out = torch.empty_like(x)

@@ -142,13 +142,16 @@ class AttentionPairBias(nn.Module):
         self.linear_nobias_z = LinearNoBias(in_features=c_z, out_features=n_heads)
         self._cache = _WeightCache()
 
+    def pair_bias_weights(self, z: torch.Tensor) -> tuple:
+        """(LayerNorm weight, bias, projection [heads, c_z]) in the arithmetic type of z's kernels."""
+        ps = (self.layernorm_z.weight, self.layernorm_z.bias, self.linear_nobias_z.weight)
+        cd = ops.compute_dtype(z)     # bf16 for fp32 rows of 128 channels under bf16 autocast
+        return self._cache.get(ps, cd, z.device, lambda: tuple(_cv(p, cd, z.device) for p in ps))
+
     def pair_bias(self, z: torch.Tensor) -> torch.Tensor:
         """[*, N, N, c_z] -> fp32 [*, heads, N, N] = permute(linear(LN(z)))
         (transformer.py:191-194)."""
-        ps = (self.layernorm_z.weight, self.layernorm_z.bias, self.linear_nobias_z.weight)
-        cd = ops.compute_dtype(z)     # bf16 for fp32 rows of 128 channels under bf16 autocast
-        ln_w, ln_b, w = self._cache.get(ps, cd, z.device,
-                                        lambda: tuple(_cv(p, cd, z.device) for p in ps))
+        ln_w, ln_b, w = self.pair_bias_weights(z)
         n, c = z.shape[-2], z.shape[-1]
         zb = z.contiguous().reshape(-1, n, n, c)
         out = torch.stack([ops.pair_bias(zb[i], ln_w, ln_b, w, out_f32=True)
