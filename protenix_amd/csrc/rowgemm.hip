@@ -46,7 +46,7 @@ struct RowGemmInParams {
   RowMap mmap;
   int n;                // tokens (n_rows = n*n for pair tensors)
   int pitch;            // row pitch of a, b (TRIMUL_IN) / v^T, triangle bias (TRIATTN_IN)
-  int aux;              // TRIATTN_IN: heads; PAIRBIAS: heads | out_f32 << 8
+  int aux;              // TRIATTN_IN: heads; PAIRBIAS: heads | out_f32 << 8; TRIMUL_IN: walk back to front
   float q_scale;        // TRIATTN_IN: log2(e)/sqrt(d)
   // TRIMUL_OUT only
   const void* x2;       // channel-major triangle product [128][n_rows]
@@ -279,8 +279,10 @@ rowgemm_in_kernel(RowGemmInParams p) {
     // before them has just written it front to back, so its tail is what the 256 MB memory-side
     // cache still holds; read front to back, a tensor larger than that cache evicts its own
     // tail before reaching it.
-    constexpr bool kBackward = MODE == kTriMulIn || MODE == kTriAttnIn;
-    const int64_t wtile = (kBackward && tile < n_tiles) ? n_tiles - 1 - tile : tile;
+    // (The outgoing triangle multiplication opens a block, behind the transition of the block
+    // before, which itself walks back to front: that projection walks forward.)
+    const bool backward = MODE == kTriAttnIn || (MODE == kTriMulIn && p.aux != 0);
+    const int64_t wtile = (backward && tile < n_tiles) ? n_tiles - 1 - tile : tile;
     const int64_t row0 = wtile * (RB * 32);
     int pi0 = 0, pk0 = 0;
     if constexpr (MODE == kTriMulIn) {
@@ -1077,6 +1079,7 @@ int trimul_project(const void* z, const void* mask, const void* ln_w, const void
   p.mmap = pair_map(n, 1, incoming != 0);
   p.n = n;
   p.pitch = k_pitch;
+  p.aux = incoming != 0;   // walk direction (see the kernel)
   if (c_z == 64) return launch_rowgemm_in<T, kTriMulIn, 4, TZ>(p, stream);
   if (c_z == 256) {
     if constexpr (sizeof(T) == 2 && sizeof(TZ) == 2) return launch_rowgemm_in<T, kTriMulIn, 16>(p, stream);
