@@ -166,11 +166,33 @@ def _workspace(shape, dtype, device) -> torch.Tensor:
     return torch.empty(shape, dtype=dtype, device=device)
 
 
-def _mask_for(mask: Optional[torch.Tensor], z: torch.Tensor,
-              dtype: Optional[torch.dtype] = None) -> Optional[torch.Tensor]:
+# The same pair mask comes back for every update of every block: its copy in the kernels' dtype
+# (and, for the ending node, its transpose: the attention core then reads a row's key mask as
+# one run of memory instead of a strided gather per key tile) is made once and kept.  An entry
+# holds the caller's tensor, so its storage cannot be freed and handed out again while the entry
+# lives, and is valid for that storage, view geometry and version counter only.
+_mask_cache: list = []
+
+
+def _mask_for(mask: Optional[torch.Tensor], z: torch.Tensor, dtype: Optional[torch.dtype] = None,
+              transpose: bool = False) -> Optional[torch.Tensor]:
     if mask is None:
         return None
-    return mask.to(device=z.device, dtype=dtype or z.dtype).contiguous()
+    dtype = dtype or z.dtype
+    key = (mask.untyped_storage().data_ptr(), mask.storage_offset(), tuple(mask.shape), tuple(mask.stride()),
+           mask.dtype, mask.device, mask._version, dtype, z.device, transpose)
+    for i, (k, _, out) in enumerate(_mask_cache):
+        if k == key:
+            if i:
+                _mask_cache.insert(0, _mask_cache.pop(i))
+            return out
+    out = mask.to(device=z.device, dtype=dtype)
+    out = out.transpose(-1, -2).contiguous() if transpose else out.contiguous()
+    if out.untyped_storage().data_ptr() == mask.untyped_storage().data_ptr():
+        return out      # the caller's own tensor: nothing was made, nothing to keep
+    _mask_cache.insert(0, (key, mask, out))
+    del _mask_cache[8:]
+    return out
 
 
 def triangle_multiplication(z: torch.Tensor, mask: Optional[torch.Tensor], w: dict, incoming: bool,
@@ -218,7 +240,8 @@ def triangle_attention(z: torch.Tensor, mask: Optional[torch.Tensor], w: dict, h
     cd = w["w_q"].dtype
     dt, st = _dt_stream(z, cd), _stream()
     pitch = key_pitch(n)
-    mask = _mask_for(mask, z, cd)
+    # (ending node: the key mask of logical row i is mask[:, i]; a transposed copy makes it a row)
+    mask = _mask_for(mask, z, cd, transpose=transposed)
     dev = z.device
     # attention-core layouts (see include/protenix_amd.h): q, gate, output head-major; K, V^T
     # and the triangle bias in fragment-ordered key tiles
@@ -235,7 +258,7 @@ def triangle_attention(z: torch.Tensor, mask: Optional[torch.Tensor], w: dict, h
               int(transposed), eps, dt, st)
         # o overwrites g: each element of g is read once, by the thread that then writes o there
         _call("triattn_fwd", lib.ptx_triattn_fwd, _ptr(q), _ptr(k), _ptr(vt), _ptr(g), _ptr(tb),
-              _ptr(mask), _ptr(g), n, heads, d, pitch, int(transposed), float(inf), dt, st)
+              _ptr(mask), _ptr(g), n, heads, d, pitch, 0, float(inf), dt, st)
         del q, k, vt, tb
         if out is None:
             out = torch.empty_like(z)

@@ -190,6 +190,31 @@ def test_triattn_random_mask_large_logits():
     assert rel_err(got, want) <= 1e-4
 
 
+@pytest.mark.parametrize("starting", [True, False])
+def test_triattn_mask_changed_in_place_and_replaced(starting):
+    """The converted (and, for the ending node, transposed) copy of a mask is kept between
+    calls: a mask edited in place, and a new mask tensor of the same shape, must each be seen.
+    Non-symmetric masks, so that a missed transpose shows as well."""
+    ref, prod = oracle_and_product(O.TriangleAttention, P.TriangleAttention, 128, 32, 4, starting=starting)
+    n = 80
+    z = _z(n, torch.float32)
+    g = torch.Generator().manual_seed(11)
+    mask = (torch.rand(1, n, n, generator=g) > 0.3).float()
+    mask_dev = mask.cuda()
+    with torch.no_grad():
+        assert rel_err(prod(z.cuda(), mask_dev), ref(z, mask)) <= 1e-4
+        assert rel_err(prod(z.cuda(), mask_dev), ref(z, mask)) <= 1e-4      # served from the kept copy
+        mask[0, :, 5] = 0
+        mask[0, 7, :] = 1
+        mask_dev[0, :, 5] = 0                                               # in place: same tensor
+        mask_dev[0, 7, :] = 1
+        assert rel_err(prod(z.cuda(), mask_dev), ref(z, mask)) <= 1e-4
+        other = (torch.rand(1, n, n, generator=g) > 0.5).float()
+        del mask_dev
+        assert rel_err(prod(z.cuda(), other.cuda()), ref(z, other)) <= 1e-4  # a new tensor, maybe the old address
+        assert rel_err(prod(z.cuda(), other.bool().cuda()), ref(z, other)) <= 1e-4
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_triattn_nan_stays_where_the_reference_puts_it(dtype):
     """A NaN at z[i0, j0] reaches, in the reference, row i0 (a poisoned key of that row) and the
