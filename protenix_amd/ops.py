@@ -188,8 +188,14 @@ def _mask_for(mask: Optional[torch.Tensor], z: torch.Tensor, dtype: Optional[tor
             return out
     out = mask.to(device=z.device, dtype=dtype)
     out = out.transpose(-1, -2).contiguous() if transpose else out.contiguous()
-    if out.untyped_storage().data_ptr() == mask.untyped_storage().data_ptr():
-        return out      # the caller's own tensor: nothing was made, nothing to keep
+    # A mask of all ones changes no bit of any result (x * 1, logit + 0): it is handed on as
+    # "no mask", which spares the kernels its loads.  Looking costs one synchronisation per
+    # mask (not per call), and is skipped under stream capture, where none is allowed.
+    if out.is_cuda and not torch.cuda.is_current_stream_capturing():
+        if bool((out == 1).all()):
+            out = None
+    elif out.untyped_storage().data_ptr() == mask.untyped_storage().data_ptr():
+        return out      # the caller's own tensor, unexamined: nothing to keep
     _mask_cache.insert(0, (key, mask, out))
     del _mask_cache[8:]
     return out

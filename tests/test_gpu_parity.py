@@ -216,6 +216,27 @@ def test_triattn_mask_changed_in_place_and_replaced(starting):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+def test_block_all_ones_mask_is_no_mask(dtype):
+    """A mask of all ones is handed to the kernels as "no mask" (decided once per mask): the same
+    bits as with the mask loaded and applied, which is what a capturing stream still does."""
+    ref, prod = oracle_and_product(O.PairformerBlock, P.PairformerBlock, dtype=dtype)
+    s, z, pm = (t.cuda() for t in O.make_inputs(70, dtype=dtype))
+    with torch.no_grad():
+        s0, z0 = prod(s, z, None)
+        s1, z1 = prod(s, z, pm)
+        P.ops._mask_cache.clear()
+        keep = torch.cuda.is_current_stream_capturing
+        torch.cuda.is_current_stream_capturing = lambda: True      # the mask is then used unexamined
+        try:
+            s2, z2 = prod(s, z, pm.clone())
+        finally:
+            torch.cuda.is_current_stream_capturing = keep
+            P.ops._mask_cache.clear()
+    assert torch.equal(z0, z1) and torch.equal(s0, s1)
+    assert torch.equal(z0, z2) and torch.equal(s0, s2)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_triattn_nan_stays_where_the_reference_puts_it(dtype):
     """A NaN at z[i0, j0] reaches, in the reference, row i0 (a poisoned key of that row) and the
     queries at position i0 of every row (their triangle bias).  The fast softmax paths of the
