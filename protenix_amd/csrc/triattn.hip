@@ -66,7 +66,13 @@ struct AttnAux {
 // contiguous channels at each position); gate may be null (no gating).  mask: per (row, key),
 // 0/1 values turned into inf*(mask-1), or with ax.mask_is_bias an additive bias used as it is.
 // ax.lse: optional log2-sum-exp2 of the logits per (head, row, query).
-template <typename T, int R, int NWQ>
+// MK: kMaskGiven, or no mask (its own instantiations: a mask of all ones is passed as none by
+// the host side).  Without a mask only a last, partial key tile publishes a per-key bias
+// (-inf beyond n), and no other tile pays for the mask's load, its LDS round trip or the test of
+// its values (kMaskTail); where the keys fill whole tiles nothing of the masked path is left in
+// the kernel (kMaskNone).
+enum { kMaskNone = 0, kMaskTail = 1, kMaskGiven = 2 };
+template <typename T, int R, int NWQ, int MK>
 __global__ __launch_bounds__((NWQ * 64), (sizeof(T) == 2 ? 16 / NWQ : 2)) void triattn_fwd_kernel(
     const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ vt,
     const T* gate, const T* __restrict__ bias, const T* __restrict__ mask,
@@ -94,8 +100,7 @@ __global__ __launch_bounds__((NWQ * 64), (sizeof(T) == 2 ? 16 / NWQ : 2)) void t
   const int key_tiles = key_pitch >> 6;
   const int q_blocks = (n + 31) >> 5;
   const int n_tiles = (n + kKeyTile - 1) / kKeyTile;
-  const bool has_mask = mask != nullptr;
-  const T* mask_or_dummy = has_mask ? mask : q;   // any valid address: the value is discarded
+  constexpr bool has_mask = MK == kMaskGiven;
   // Operand tiles in fragment order (common.h): 2048 elements per key tile, this lane's
   // 8 elements of fragment f at f*512 + lane*8.  Rows beyond n re-read row n-1, a wave whose
   // queries all lie beyond n re-reads the last query block; nothing of either is stored.
@@ -132,11 +137,10 @@ __global__ __launch_bounds__((NWQ * 64), (sizeof(T) == 2 ? 16 / NWQ : 2)) void t
   constexpr int FPW = 8 * R / NWQ;   // fragments each wave moves per tile
   V8 pre[FPW];
   T pre_mv;
-  // mask value of key kc for this wave's row: m_base[kc * m_stride] (stride 0: no mask, any
-  // valid address - the value is discarded)
+  // mask value of key kc for this wave's row: m_base[kc * m_stride]
   const int m_row = min(i0 + min(wave, R - 1), n_rows - 1);
-  const unsigned m_stride = has_mask ? (mask_transposed ? n : 1) : 0;
-  const T* m_base = mask_or_dummy + (has_mask ? (mask_transposed ? (int64_t)m_row : (int64_t)m_row * n) : 0);
+  const unsigned m_stride = mask_transposed ? n : 1;
+  const T* m_base = has_mask ? mask + (mask_transposed ? (int64_t)m_row : (int64_t)m_row * n) : nullptr;
   auto fetch = [&](int tile) {
     const int64_t atile = min(tile, n_tiles - 1);
 #pragma unroll
@@ -147,8 +151,10 @@ __global__ __launch_bounds__((NWQ * 64), (sizeof(T) == 2 ? 16 / NWQ : 2)) void t
       pre[j] = load8<T>((f < 4 ? k : vt) + rowtiles * kAttnTileElems + (f & 3) * 512 + lane * 8);
     }
     // wave w < R publishes the mask bias of row i0 + w; all waves load (uniform load count)
-    const int kc = min(tile * kKeyTile + lane, n - 1);
-    pre_mv = m_base[__umul24(kc, m_stride)];   // both below 2^15
+    if constexpr (has_mask) {
+      const int kc = min(tile * kKeyTile + lane, n - 1);
+      pre_mv = m_base[__umul24(kc, m_stride)];   // both below 2^15
+    }
   };
   auto stash = [&](int tile) {
     const int buf = tile % 3;
@@ -167,7 +173,7 @@ __global__ __launch_bounds__((NWQ * 64), (sizeof(T) == 2 ? 16 / NWQ : 2)) void t
       }
       lds_kv[buf][fid >> 3][f][lane] = v;
     }
-    if (wave < R) {
+    if (wave < R && (has_mask || (MK == kMaskTail && tail))) {
       const float mb = !has_mask ? 0.0f : ax.mask_is_bias ? to_f32(pre_mv) : inf * (to_f32(pre_mv) - 1.0f);
       lds_mb[buf][wave][lane] = key0 + lane < n ? mb : -INFINITY;
     }
@@ -315,7 +321,9 @@ __global__ __launch_bounds__((NWQ * 64), (sizeof(T) == 2 ? 16 / NWQ : 2)) void t
     const int buf = tile % 3;
     // keys of the tile with a non-zero mask bias, as a lane mask (key <-> lane); half u's keys
     // are the lanes with bit 4 == u
-    const uint64_t mb_mask = __builtin_amdgcn_ballot_w64(lds_mb[buf][0][lane] != 0.0f);
+    const uint64_t mb_mask = (has_mask || (MK == kMaskTail && tile * kKeyTile + kKeyTile > n))
+                                 ? __builtin_amdgcn_ballot_w64(lds_mb[buf][0][lane] != 0.0f)
+                                 : 0ull;
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
       HalfOut out;
@@ -431,14 +439,21 @@ int triattn_fwd_ex(const T* q, const T* k, const T* vt, const T* g, const T* tri
   const int n_rowgroups = (n_rows + R - 1) / R;
   const int64_t total = (int64_t)heads * n_rowgroups * n_qtiles;
   const int64_t per_xcd = (total + 7) / 8;
-  if (wide)
-    triattn_fwd_kernel<T, R, 8><<<dim3((unsigned)(per_xcd * 8)), dim3(512), 0, stream>>>(
-        q, k, vt, g, tri_bias, mask, o, n, heads, key_pitch, mask_transposed, inf, n_qtiles,
-        n_rowgroups, total, ax);
-  else
-    triattn_fwd_kernel<T, R, 4><<<dim3((unsigned)(per_xcd * 8)), dim3(256), 0, stream>>>(
-        q, k, vt, g, tri_bias, mask, o, n, heads, key_pitch, mask_transposed, inf, n_qtiles,
-        n_rowgroups, total, ax);
+#define PTX_ATTN_LAUNCH(NWQ, MK)                                                                  \
+  triattn_fwd_kernel<T, R, NWQ, MK><<<dim3((unsigned)(per_xcd * 8)), dim3(NWQ * 64), 0, stream>>>( \
+      q, k, vt, g, tri_bias, mask, o, n, heads, key_pitch, mask_transposed, inf, n_qtiles,        \
+      n_rowgroups, total, ax)
+  const int mk = mask ? kMaskGiven : n % kKeyTile ? kMaskTail : kMaskNone;
+  if (wide) {
+    if (mk == kMaskGiven) PTX_ATTN_LAUNCH(8, kMaskGiven);
+    else if (mk == kMaskTail) PTX_ATTN_LAUNCH(8, kMaskTail);
+    else PTX_ATTN_LAUNCH(8, kMaskNone);
+  } else {
+    if (mk == kMaskGiven) PTX_ATTN_LAUNCH(4, kMaskGiven);
+    else if (mk == kMaskTail) PTX_ATTN_LAUNCH(4, kMaskTail);
+    else PTX_ATTN_LAUNCH(4, kMaskNone);
+  }
+#undef PTX_ATTN_LAUNCH
   return 0;
 }
 
