@@ -186,6 +186,8 @@ PTX_API int ptx_trimul_output(const void* x, const void* z, const void* ln_in_w,
  *   elements;  key_pitch = ptx_key_pitch(n).   d = 32;  c_in = 64 or 128 with 4 heads,
  *   or (bf16 only) c_in = 256 with 8 heads  (w_q, w_k, w_v, w_g [heads*d][c_in],
  *   w_b [heads][c_in]).
+ * g = NULL (c_in = 128, 4 heads, PTX_BF16 / PTX_MIXED): no gate is written; stage 2 is then
+ * called without one and ptx_triattn_gate_output forms it in stage 3.
  */
 PTX_API int ptx_triattn_project(const void* z, const void* ln_w, const void* ln_b, const void* w_q,
                         const void* w_k, const void* w_v, const void* w_g, const void* w_b,
@@ -203,7 +205,7 @@ PTX_API int ptx_triattn_project(const void* z, const void* ln_w, const void* ln_
  * layers.py:286-291 does.
  *   mask [n][n] in `dtype` or NULL; mask(i,k) = mask[i][k], or mask[k][i] when
  *   mask_transposed = 1.   q, k, vt, g, tri_bias as written by stage 1;
- *   o [heads][n][n][d] (may alias g, not q/k/vt).
+ *   o [heads][n][n][d] (may alias g, not q/k/vt).   g = NULL: no gate (g = 1).
  */
 PTX_API int ptx_triattn_fwd(const void* q, const void* k, const void* vt, const void* g,
                     const void* tri_bias, const void* mask, void* o, int n, int heads, int d,
@@ -262,6 +264,19 @@ PTX_API int ptx_triattn_core_bwd(const void* q, const void* k, const void* v, co
  */
 PTX_API int ptx_triattn_output(const void* o, const void* w_o, const void* z, void* out, int n,
                        int c_in, int transposed, int add_residual, int dtype, void* stream);
+
+/*
+ * Stage 3 with the gate of layers.py:386-390 formed here, from rows this stage loads anyway:
+ *   out(p) = [z(p) +] W_o ( sigmoid(W_g LN(z(p))) * o[p] )
+ * for o written ungated by stage 2 (g = NULL there and in stage 1): the gate tensor is then
+ * neither written nor read.  ln_w / ln_b: the LayerNorm of stage 1 (either may be NULL);
+ * w_g [heads*d][c_in], w_o [c_in][heads*d]; gate and gated product are rounded to bf16 as the
+ * reference's are.  c_in = 128, heads = 4 (d = 32); dtype PTX_BF16 or PTX_MIXED; out may alias z.
+ */
+PTX_API int ptx_triattn_gate_output(const void* o, const void* z, const void* ln_w, const void* ln_b,
+                            const void* w_g, const void* w_o, void* out, int n, int c_in,
+                            int heads, int transposed, int add_residual, float eps, int dtype,
+                            void* stream);
 
 /*
  * Transition (primitives.py:190-230), one fused kernel:

@@ -42,6 +42,7 @@ SIGNATURES = {
     "ptx_triattn_core_workspace_elems": (_l, [_i, _i, _i]),
     "ptx_triattn_core_fwd": (_i, [_p] * 8 + [_i, _i, _i, _i, _i, _i, _p]),
     "ptx_triattn_core_bwd": (_i, [_p] * 13 + [_i, _i, _i, _i, _i, _i, _p]),
+    "ptx_triattn_gate_output": (_i, [_p] * 7 + [_i, _i, _i, _i, _i, _f, _i, _p]),
     "ptx_transition_packed_elems": (_l, [_i, _i]),
     "ptx_transition_pack": (_i, [_p, _p, _p, _p, _i, _i, _i, _p]),
     "ptx_transition_fwd": (_i, [_p] * 5 + [_l, _i, _i, _i, _f, _i, _p]),

@@ -267,11 +267,14 @@ PTX_API int ptx_triattn_project(const void* z, const void* ln_w, const void* ln_
               "triattn_project: key_pitch=%d, expected %d", key_pitch, ptx_key_pitch(n));
   PTX_REQUIRE(n <= 8192, PTX_ERR_UNSUPPORTED, "triattn_project: n=%d too large (8192 at most)", n);
   if (n == 0) return PTX_OK;
-  PTX_REQUIRE(z && w_q && w_k && w_v && w_g && w_b && q && k && vt && g && tri_bias,
+  PTX_REQUIRE(z && w_q && w_k && w_v && w_g && w_b && q && k && vt && tri_bias,
               PTX_ERR_BAD_ARG, "triattn_project: null pointer");
+  // without a gate output: where ptx_triattn_gate_output exists to form the gate instead
+  PTX_REQUIRE(g || (c_in == 128 && heads == 4 && dtype != PTX_F32), PTX_ERR_UNSUPPORTED,
+              "triattn_project: g = NULL needs c_in = 128, 4 heads and 16-bit arithmetic");
   PTX_REQUIRE(aligned16(z) && aligned16(w_q) && aligned16(w_k) && aligned16(w_v) &&
                   aligned16(w_g) && aligned16(w_b) && aligned16(q) && aligned16(k) &&
-                  aligned16(vt) && aligned16(g) && aligned16(tri_bias) &&
+                  aligned16(vt) && (!g || aligned16(g)) && aligned16(tri_bias) &&
                   (!ln_w || aligned16(ln_w)) &&
                   (!ln_b || aligned16(ln_b)),
               PTX_ERR_BAD_ARG, "triattn_project: pointers must be 16-byte aligned");
@@ -292,8 +295,8 @@ PTX_API int ptx_triattn_fwd(const void* q, const void* k, const void* vt, const 
               "triattn_fwd: key_pitch=%d, expected %d", key_pitch, ptx_key_pitch(n));
   PTX_REQUIRE(n < 32768, PTX_ERR_UNSUPPORTED, "triattn_fwd: n=%d too large", n);
   if (n == 0 || heads == 0) return PTX_OK;
-  PTX_REQUIRE(q && k && vt && g && tri_bias && o, PTX_ERR_BAD_ARG, "triattn_fwd: null pointer");
-  PTX_REQUIRE(aligned16(q) && aligned16(k) && aligned16(vt) && aligned16(g) &&
+  PTX_REQUIRE(q && k && vt && tri_bias && o, PTX_ERR_BAD_ARG, "triattn_fwd: null pointer");
+  PTX_REQUIRE(aligned16(q) && aligned16(k) && aligned16(vt) && (!g || aligned16(g)) &&
                   aligned16(tri_bias) && aligned16(o),
               PTX_ERR_BAD_ARG, "triattn_fwd: pointers must be 16-byte aligned");
   PTX_DISPATCH(dtype, ptx::triattn_fwd<T>((const T*)q, (const T*)k, (const T*)vt, (const T*)g,
@@ -405,6 +408,31 @@ PTX_API int ptx_triattn_output(const void* o, const void* w_o, const void* z, vo
   PTX_DISPATCH_Z(dtype, (ptx::triattn_output<T, TZ>)(o, w_o, z, out, n, c_in, transposed, add_residual,
                                              (hipStream_t)stream));
   return after_launch("triattn_output");
+}
+
+PTX_API int ptx_triattn_gate_output(const void* o, const void* z, const void* ln_w, const void* ln_b,
+                                    const void* w_g, const void* w_o, void* out, int n, int c_in,
+                                    int heads, int transposed, int add_residual, float eps, int dtype,
+                                    void* stream) {
+  PTX_REQUIRE(dtype == PTX_BF16 || dtype == PTX_MIXED, PTX_ERR_UNSUPPORTED,
+              "triattn_gate_output: built for PTX_BF16 and PTX_MIXED only (got dtype %d)", dtype);
+  PTX_REQUIRE(n >= 0, PTX_ERR_BAD_ARG, "triattn_gate_output: n=%d", n);
+  PTX_REQUIRE(c_in == 128 && heads == 4, PTX_ERR_UNSUPPORTED,
+              "triattn_gate_output: only c_in = 128 with 4 heads of 32 is built (got c_in=%d heads=%d)",
+              c_in, heads);
+  PTX_REQUIRE(n < 32768, PTX_ERR_UNSUPPORTED, "triattn_gate_output: n=%d too large", n);
+  if (n == 0) return PTX_OK;
+  PTX_REQUIRE(o && z && w_g && w_o && out, PTX_ERR_BAD_ARG, "triattn_gate_output: null pointer");
+  PTX_REQUIRE(aligned16(o) && aligned16(z) && aligned16(w_g) && aligned16(w_o) && aligned16(out) &&
+                  (!ln_w || aligned16(ln_w)) && (!ln_b || aligned16(ln_b)),
+              PTX_ERR_BAD_ARG, "triattn_gate_output: pointers must be 16-byte aligned");
+  if (dtype == PTX_MIXED)
+    ptx::triattn_gate_output<float>(o, z, ln_w, ln_b, w_g, w_o, out, n, transposed, add_residual, eps,
+                                    (hipStream_t)stream);
+  else
+    ptx::triattn_gate_output<ptx::bf16_t>(o, z, ln_w, ln_b, w_g, w_o, out, n, transposed, add_residual,
+                                          eps, (hipStream_t)stream);
+  return after_launch("triattn_gate_output");
 }
 
 PTX_API int64_t ptx_transition_packed_elems(int c, int n_factor) {

@@ -38,6 +38,12 @@ int triattn_project(const void* z, const void* ln_w, const void* ln_b, const voi
 template <typename T, typename TZ = T>
 int triattn_output(const void* o, const void* w_o, const void* z, void* out, int n, int c_z,
                    int transposed, int add_residual, hipStream_t stream);
+// out = [z +] W_o (sigmoid(W_g LN(z)) * o) on rows of 128 channels, 4 heads, 16-bit arithmetic:
+// the last stage of the triangle attention with the gate formed here (o ungated, head-major).
+template <typename TZ>
+int triattn_gate_output(const void* o, const void* z, const void* ln_w, const void* ln_b,
+                        const void* w_g, const void* w_o, void* out, int n, int transposed,
+                        int add_residual, float eps, hipStream_t stream);
 // transition weights -> fragment-ordered chunks of 32 hidden (3 * n_factor*c * c elements)
 template <typename T>
 int transition_pack(const void* w_a, const void* w_b, const void* w_o, void* packed, int c,

@@ -522,6 +522,11 @@ rowgemm_in_kernel(RowGemmInParams p) {
   };
   // (not unrolled: unrolled, the compiler hoists every chunk's loads to the top and spills them)
   auto chunk_body = [&](int ch) {
+    // kTriAttnIn without a gate output (the gate is then formed by the output kernel): the
+    // gate's chunks are passed over (resident weights only: the rings count their loads)
+    if constexpr (MODE == kTriAttnIn && RES) {
+      if (!p.out[2] && ch / (Widths<KS>::HIDDEN / 64) == 2) return;
+    }
     const int buf = (!RES && C::NBUF == 2) ? (ch & 1) : 0;
     if constexpr (kDma) {
       // the other buffer was last read in the previous chunk, which every wave has left

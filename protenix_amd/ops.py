@@ -233,6 +233,12 @@ def triangle_multiplication(z: torch.Tensor, mask: Optional[torch.Tensor], w: di
     return out
 
 
+# Triangle attention on rows of 128 channels in bf16 arithmetic: the gate is formed by the output
+# kernel (ptx_triattn_gate_output) instead of travelling through memory.  False restores the
+# three stages with a stored gate (tests compare the two).
+late_gate_enabled = True
+
+
 def triangle_attention(z: torch.Tensor, mask: Optional[torch.Tensor], w: dict, heads: int, d: int,
                        inf: float, transposed: bool, add_residual: bool,
                        out: Optional[torch.Tensor] = None, eps: float = 1e-5) -> torch.Tensor:
@@ -252,24 +258,32 @@ def triangle_attention(z: torch.Tensor, mask: Optional[torch.Tensor], w: dict, h
     # attention-core layouts (see include/protenix_amd.h): q, gate, output head-major; K, V^T
     # and the triangle bias in fragment-ordered key tiles
     n_kv, n_tb = lib.ptx_triattn_kv_elems(n, heads), lib.ptx_triattn_bias_elems(n, heads)
+    # rows of 128 channels in bf16 arithmetic: no gate tensor, the output kernel forms the gate
+    late_gate = late_gate_enabled and c == 128 and heads == 4 and d == 32 and cd == torch.bfloat16
     q = _workspace((heads, n, n, d), cd, dev)
-    g = _workspace((heads, n, n, d), cd, dev)
+    g = _workspace((heads, n, n, d), cd, dev)     # the gate, then (or only) the attention output
     k = _workspace((n_kv,), cd, dev)
     vt = _workspace((n_kv,), cd, dev)
     tb = _workspace((n_tb,), cd, dev)
     with torch.cuda.device(dev):
         _call("triattn_project", lib.ptx_triattn_project, _ptr(z), _ptr(w["ln_w"]),
               _ptr(w["ln_b"]), _ptr(w["w_q"]), _ptr(w["w_k"]), _ptr(w["w_v"]), _ptr(w["w_g"]),
-              _ptr(w["w_b"]), _ptr(q), _ptr(k), _ptr(vt), _ptr(g), _ptr(tb), n, c, heads, d, pitch,
-              int(transposed), eps, dt, st)
+              _ptr(w["w_b"]), _ptr(q), _ptr(k), _ptr(vt), None if late_gate else _ptr(g), _ptr(tb),
+              n, c, heads, d, pitch, int(transposed), eps, dt, st)
         # o overwrites g: each element of g is read once, by the thread that then writes o there
-        _call("triattn_fwd", lib.ptx_triattn_fwd, _ptr(q), _ptr(k), _ptr(vt), _ptr(g), _ptr(tb),
-              _ptr(mask), _ptr(g), n, heads, d, pitch, 0, float(inf), dt, st)
+        _call("triattn_fwd", lib.ptx_triattn_fwd, _ptr(q), _ptr(k), _ptr(vt),
+              None if late_gate else _ptr(g), _ptr(tb), _ptr(mask), _ptr(g), n, heads, d, pitch, 0,
+              float(inf), dt, st)
         del q, k, vt, tb
         if out is None:
             out = torch.empty_like(z)
-        _call("triattn_output", lib.ptx_triattn_output, _ptr(g), _ptr(w["w_o"]), _ptr(z), _ptr(out), n, c,
-                                          int(transposed), int(add_residual), dt, st)
+        if late_gate:
+            _call("triattn_output", lib.ptx_triattn_gate_output, _ptr(g), _ptr(z), _ptr(w["ln_w"]),
+                  _ptr(w["ln_b"]), _ptr(w["w_g"]), _ptr(w["w_o"]), _ptr(out), n, c, heads,
+                  int(transposed), int(add_residual), eps, dt, st)
+        else:
+            _call("triattn_output", lib.ptx_triattn_output, _ptr(g), _ptr(w["w_o"]), _ptr(z), _ptr(out),
+                  n, c, int(transposed), int(add_residual), dt, st)
     return out
 
 
