@@ -38,7 +38,7 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 # from profiles/trunk_n768_fp32_residual_hbm_traffic.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # on this benchmark, calibrated against a plain elementwise kernel of known size), not measured
 # in this run.  Algorithmic: 594432 + 147456 KiB.
-TRIATTN_FWD_TRAFFIC_BYTES_N768 = (604564 + 147460) * 1024
+TRIATTN_FWD_TRAFFIC_BYTES_N768 = (451945 + 147460) * 1024
 TRAFFIC_SOURCE = "profiles/trunk_n768_fp32_residual_hbm_traffic.txt (rocprofv3 --pmc, not measured in this run)"
 
 
@@ -54,8 +54,8 @@ def _work(n: int, z_bytes: int) -> dict:
         "transition":      ("mfma", 393216.0 * n * n),            # 3 GEMMs 128<->512, fused
         "trimul_project":  ("hbm", ez + 2.0 * e),                 # read z, write a and b
         "trimul_output":   ("hbm", e + 2.0 * ez),                 # read x and z, write z
-        "triattn_project": ("hbm", ez + 4.0 * e),                 # read z, write q k v g (+ bias)
-        "triattn_output":  ("hbm", e + 2.0 * ez),                 # read o and z, write z
+        "triattn_project": ("hbm", ez + 3.0 * e),                 # read z, write q k v (+ bias); no gate tensor
+        "triattn_output":  ("hbm", e + 2.0 * ez),                 # read o and z, write z (forms the gate)
         "pair_bias":       ("hbm", ez + 16 * n * n * 4),          # read z, write fp32 [16,N,N]
         "layernorm":       ("hbm", None),                         # single track only, tiny
     }
