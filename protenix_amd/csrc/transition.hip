@@ -87,6 +87,17 @@ __global__ void transition_pack_kernel(const T* __restrict__ w_a, const T* __res
 // a Pairformer block, bias[h][row] = (W LN_pb(out[row]))[h], formed from the finished rows
 // while they pass through the epilogue (a kernel of its own would read the pair tensor once
 // more for it).
+// Sum over groups of LPM (4 or 8) neighbouring lanes on the vector ALU's lane-permute path
+// (quad swaps, then the mirror of each half row): every lane of a group ends up with the sum.
+template <int LPM> __device__ __forceinline__ float group_sum(float v) {
+  static_assert(LPM == 4 || LPM == 8, "groups of 4 or 8 lanes");
+  v += __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0xB1, 0xf, 0xf, true));   // quad_perm [1,0,3,2]
+  v += __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x4E, 0xf, 0xf, true));   // quad_perm [2,3,0,1]
+  if (LPM == 8)
+    v += __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x141, 0xf, 0xf, true));  // row_half_mirror
+  return v;
+}
+
 struct PairBiasArgs {
   const void *gamma, *beta, *w;   // LayerNorm of the bias (either may be null), W [heads][c]
   void* out;                      // [heads][n_rows], fp32 or T
@@ -114,6 +125,22 @@ __global__ __launch_bounds__((TrCfg<T, KS>::NW * 64)) void transition_fused_kern
   // Workgroups take the rows back to front: the kernel before this one wrote the pair tensor
   // front to back, and its tail is what the memory-side cache still holds.
   const int64_t row0 = ((int64_t)(gridDim.x - 1 - blockIdx.x) * NW + wave) * (RB * 32);
+
+  // PB: the bias' weight as A fragments (rows beyond `heads` repeat the last head: those
+  // accumulator rows are not stored) and its LayerNorm parameters as fp32, parked in LDS for
+  // the epilogue: fetched there from global memory they would cost every tile a round trip
+  // that nothing hides.  (Visible to all waves after the first ring barrier below.)
+  __shared__ V8 lds_pbw[PB ? KS : 1][kWave];
+  __shared__ __attribute__((aligned(16))) float lds_pba[2][PB ? 16 * KS : 4];
+  if constexpr (PB) {
+    static_assert(!PB || NW == KS, "one weight fragment per wave");
+    lds_pbw[wave][lane] = load8<T>((const T*)pb.w + (int64_t)min(lane & 31, pb.heads - 1) * kCx +
+                                   16 * wave + 8 * (lane >> 5));
+    for (int c = threadIdx.x; c < kCx; c += NW * kWave) {
+      lds_pba[0][c] = pb.gamma ? to_f32(((const T*)pb.gamma)[c]) : 1.0f;
+      lds_pba[1][c] = pb.beta ? to_f32(((const T*)pb.beta)[c]) : 0.0f;
+    }
+  }
 
   // chunk j (clamped for the address) -> buffer j % NBUF; every wave moves FPW fragments
   // (address = wave-uniform base in scalar registers + this lane's offset inside a fragment:
@@ -299,27 +326,8 @@ __global__ __launch_bounds__((TrCfg<T, KS>::NW * 64)) void transition_fused_kern
 
   if constexpr (PB) {
     static_assert(!PB || (RB == 1 && sizeof(T) == 2), "pair-bias epilogue: one row block, 16-bit arithmetic");
-    // The bias' weights and LayerNorm parameters, requested before anything that waits: W as A
-    // fragments (rows beyond `heads` re-read the last head: those accumulator rows are not
-    // stored), gamma / beta for the columns this lane normalises.
     const int n = lane & 31, g = lane >> 5;
-    V8 wf[KS];
-#pragma unroll
-    for (int kk = 0; kk < KS; ++kk)
-      wf[kk] = load8<T>((const T*)pb.w + (int64_t)min(n, pb.heads - 1) * kCx + 16 * kk + 8 * g);
-    const T* pg = pb.gamma ? (const T*)pb.gamma : default_gamma<T>();
-    const T* pbeta = pb.beta ? (const T*)pb.beta : default_beta<T>();
-    bf16x4 gm[NOB][C::VE / 4], bt[NOB][C::VE / 4];
-    {
-      const int m0 = (lane % C::LPM) * C::VE;   // as stage_coord: the same columns in every pass
-#pragma unroll
-      for (int ob = 0; ob < NOB; ++ob)
-#pragma unroll
-        for (int q4 = 0; q4 < C::VE / 4; ++q4) {
-          gm[ob][q4] = *reinterpret_cast<const bf16x4*>(pg + ob * 32 + m0 + 4 * q4);
-          bt[ob][q4] = *reinterpret_cast<const bf16x4*>(pbeta + ob * 32 + m0 + 4 * q4);
-        }
-    }
+    const int m0c = (lane % C::LPM) * C::VE;   // as stage_coord: the same columns in every pass
     // LayerNorm statistics of the finished rows (as stored: TZ), two passes in fp32.  In the
     // read-back layout a row's 32 columns of one block sit in LPM neighbouring lanes.
     float mean[C::NPASS], rstd[C::NPASS];
@@ -330,8 +338,7 @@ __global__ __launch_bounds__((TrCfg<T, KS>::NW * 64)) void transition_fused_kern
       for (int ob = 0; ob < NOB; ++ob)
 #pragma unroll
         for (int e = 0; e < C::VE; ++e) sum += to_f32(done[0][ob][ps][e]);
-#pragma unroll
-      for (int o = 1; o < C::LPM; o <<= 1) sum += __shfl_xor(sum, o, 64);
+      sum = group_sum<C::LPM>(sum);
       mean[ps] = sum * (1.0f / kCx);
       float q = 0.0f;
 #pragma unroll
@@ -341,8 +348,7 @@ __global__ __launch_bounds__((TrCfg<T, KS>::NW * 64)) void transition_fused_kern
           const float d = to_f32(done[0][ob][ps][e]) - mean[ps];
           q += d * d;
         }
-#pragma unroll
-      for (int o = 1; o < C::LPM; o <<= 1) q += __shfl_xor(q, o, 64);
+      q = group_sum<C::LPM>(q);
       rstd[ps] = rsqrtf(q * (1.0f / kCx) + pb.eps);
     }
     // per wave: 32 rows x 64 normalised columns in T, behind all waves' staging tiles (other
@@ -368,11 +374,12 @@ __global__ __launch_bounds__((TrCfg<T, KS>::NW * 64)) void transition_fused_kern
           const int ob = 2 * hb + o2;
 #pragma unroll
           for (int e4 = 0; e4 < C::VE; e4 += 4) {
+            const f32x4 gm = *reinterpret_cast<const f32x4*>(&lds_pba[0][ob * 32 + m0c + e4]);
+            const f32x4 bt = *reinterpret_cast<const f32x4*>(&lds_pba[1][ob * 32 + m0c + e4]);
             f32x4 o;
 #pragma unroll
             for (int e = 0; e < 4; ++e)
-              o[e] = (to_f32(done[0][ob][ps][e4 + e]) - mean[ps]) * rstd[ps] * (float)gm[ob][e4 / 4][e] +
-                     (float)bt[ob][e4 / 4][e];
+              o[e] = (to_f32(done[0][ob][ps][e4 + e]) - mean[ps]) * rstd[ps] * gm[e] + bt[e];
             *reinterpret_cast<bf16x4*>(stn + mj * kPitchN + 32 * o2 + m0 + e4) = from_f32<T>(o);   // 8 bytes
           }
         }
@@ -381,7 +388,7 @@ __global__ __launch_bounds__((TrCfg<T, KS>::NW * 64)) void transition_fused_kern
       for (int u = 0; u < 4; ++u) {
         const u32x2* src = reinterpret_cast<const u32x2*>(stn + n * kPitchN + 16 * u + 8 * g);
         u32x2 h2[2] = {src[0], src[1]};
-        mma32(accb, wf[4 * hb + u], *reinterpret_cast<const V8*>(h2));   // lane <-> row, register <-> head
+        mma32(accb, lds_pbw[4 * hb + u][lane], *reinterpret_cast<const V8*>(h2));   // lane <-> row, register <-> head
       }
     }
     const int64_t pr = row0 + n;
