@@ -179,6 +179,15 @@ def _mask_for(mask: Optional[torch.Tensor], z: torch.Tensor, dtype: Optional[tor
     if mask is None:
         return None
     dtype = dtype or z.dtype
+
+    def convert() -> torch.Tensor:
+        out = mask.to(device=z.device, dtype=dtype)
+        return out.transpose(-1, -2).contiguous() if transpose else out.contiguous()
+
+    # Under stream capture the conversion is part of what is recorded: a replay must convert the
+    # mask it is given then, so nothing is looked up, examined or kept.
+    if not z.is_cuda or torch.cuda.is_current_stream_capturing():
+        return convert()
     key = (mask.untyped_storage().data_ptr(), mask.storage_offset(), tuple(mask.shape), tuple(mask.stride()),
            mask.dtype, mask.device, mask._version, dtype, z.device, transpose)
     for i, (k, _, out) in enumerate(_mask_cache):
@@ -186,16 +195,12 @@ def _mask_for(mask: Optional[torch.Tensor], z: torch.Tensor, dtype: Optional[tor
             if i:
                 _mask_cache.insert(0, _mask_cache.pop(i))
             return out
-    out = mask.to(device=z.device, dtype=dtype)
-    out = out.transpose(-1, -2).contiguous() if transpose else out.contiguous()
+    out = convert()
     # A mask of all ones changes no bit of any result (x * 1, logit + 0): it is handed on as
     # "no mask", which spares the kernels its loads.  Looking costs one synchronisation per
-    # mask (not per call), and is skipped under stream capture, where none is allowed.
-    if out.is_cuda and not torch.cuda.is_current_stream_capturing():
-        if bool((out == 1).all()):
-            out = None
-    elif out.untyped_storage().data_ptr() == mask.untyped_storage().data_ptr():
-        return out      # the caller's own tensor, unexamined: nothing to keep
+    # mask (not per call).
+    if bool((out == 1).all()):
+        out = None
     _mask_cache.insert(0, (key, mask, out))
     del _mask_cache[8:]
     return out

@@ -51,3 +51,23 @@ def test_graphed_block_without_single_track():
             _, z_ref = blk(None, z, None)
             s_got, z_got = fast(None, z, None)
         assert s_got is None and torch.equal(z_got, z_ref)
+
+
+def test_graphed_replays_convert_the_mask_they_are_given():
+    """The pair mask's converted copy is kept between eager calls; a graph must not bake in the
+    copy (or the "all ones: no mask" verdict) of the mask it was captured with."""
+    st = _stack(BF16, n_blocks=2)
+    fast = P.Graphed(st)
+    n = 72
+    s, z, _ = O.make_inputs(n, seed=3, dtype=BF16)
+    s, z = s.cuda(), z.cuda()
+    masks = [torch.ones(1, n, n), O.make_inputs(n, n_pad=9)[2], torch.ones(1, n, n),
+             (torch.rand(1, n, n, generator=torch.Generator().manual_seed(1)) > 0.3).float()]
+    for m in masks:
+        m = m.cuda()
+        with torch.no_grad():
+            s_ref, z_ref = st(s, z, m)
+            s_got, z_got = fast(s, z, m)
+        assert torch.equal(z_got, z_ref) and torch.equal(s_got, s_ref)
+    assert len(fast.shapes()) == 1
+
