@@ -273,6 +273,21 @@ rowgemm_in_kernel(RowGemmInParams p) {
     for (int j = 0; j < FPW; ++j) lds_w[buf * 2 * SL + wave * FPW + j][lane] = pre[j];
   };
 
+  // kPrefetch: the raw rows of a tile are requested one tile ahead, so that their way from
+  // memory lies under the previous tile's chunk loop.
+  constexpr bool kPrefetch = RES && MODE == kTriAttnIn && RB == 1;
+  typename Vec8<TZ>::type raw[kPrefetch ? KS : 1];
+  auto issue_rows = [&](int64_t t) {
+    if constexpr (kPrefetch) {
+      const int64_t wt = n_tiles - 1 - t;          // back to front, as below
+      int64_t pr = wt * 32 + (lane & 31);
+      pr = pr < p.n_rows ? pr : p.n_rows - 1;
+      const TZ* rp = (const TZ*)p.x + p.xmap(pr) + 8 * (lane >> 5);
+#pragma unroll
+      for (int kk = 0; kk < KS; ++kk) raw[kk] = load8<TZ>(rp + 16 * kk);
+    }
+  };
+  if (kPrefetch && tile < n_tiles) issue_rows(tile);
   while (true) {
     if (RES && tile >= n_tiles) break;
     // The projections at the head of an update walk the pair tensor back to front.  The kernel
@@ -327,7 +342,14 @@ rowgemm_in_kernel(RowGemmInParams p) {
       normalize_raw<T>(zraw.f[rb], gamma, beta, p.eps, g, xf.f[rb]);
     }
   } else {
-    if constexpr (kLdsAffine)
+    if constexpr (kPrefetch) {
+      f32x8 v[KS];
+#pragma unroll
+      for (int kk = 0; kk < KS; ++kk) v[kk] = to_f32(raw[kk]);
+      normalize_row<T, KS, float, false>(v, lds_affine[0], lds_affine[1], p.eps, g, xf.f[0]);
+      const int64_t nt = tile + tile_step;
+      issue_rows(nt < n_tiles ? nt : tile);
+    } else if constexpr (kLdsAffine)
       load_rows<T, RB, true, KS, float, false>(xf, (const TZ*)p.x, p.xmap, row0, p.n_rows, lds_affine[0],
                                                lds_affine[1], p.eps, lane);
     else
@@ -874,7 +896,9 @@ static int device_cu_count() {
 template <typename T, int MODE, int KS, typename TZ = T>
 int launch_rowgemm_in(const RowGemmInParams& p, hipStream_t stream) {
   typedef InCfg<T, MODE, KS> IC;
-  constexpr int RB = (sizeof(T) == 2 && MODE != kTriMulOut && KS <= 8) ? 2 : 1;
+  // (the attention projection on rows of 128 channels: one row block, and the registers the
+  // second would take hold the next tile's raw rows instead - see kPrefetch in the kernel)
+  constexpr int RB = (sizeof(T) == 2 && MODE != kTriMulOut && KS <= 8 && !(KS == 8 && MODE == kTriAttnIn)) ? 2 : 1;
   int64_t tiles = (p.n_rows + RB * 32 - 1) / (RB * 32);   // wave tiles, as in the kernel
   if (MODE == kTriMulIn) tiles = (int64_t)((p.n + 16 * RB - 1) / (16 * RB)) * (p.pitch / 8) * 4;
   if (tiles == 0) return 0;
