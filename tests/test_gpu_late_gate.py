@@ -24,7 +24,7 @@ def _run(prod, z, mask, mixed, late):
 
 @pytest.mark.parametrize("mixed", [False, True])
 @pytest.mark.parametrize("starting", [True, False])
-@pytest.mark.parametrize("n,n_pad", [(37, 5), (64, 0), (100, 7), (256, 32)])
+@pytest.mark.parametrize("n,n_pad", [(1, 0), (2, 0), (33, 1), (37, 5), (64, 0), (100, 7), (256, 32)])
 def test_late_gate_equals_stored_gate_and_oracle(mixed, starting, n, n_pad):
     dt = torch.float32 if mixed else torch.bfloat16
     ref, prod = oracle_and_product(O.TriangleAttention, P.TriangleAttention, 128, 32, 4,
