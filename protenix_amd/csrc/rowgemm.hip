@@ -245,6 +245,25 @@ rowgemm_in_kernel(RowGemmInParams p) {
   // for a chunk counts the stores issued after its loads (see the end of the chunk loop): a
   // register-staged prefetch would make the compiler drain every store before each chunk.
   constexpr bool kDma = sizeof(T) == 2 && !RES;
+  // kPrefetch: the raw rows of a tile are requested one tile ahead, so that their way from
+  // memory lies under the previous tile's chunk loop.
+  constexpr bool kPrefetch = RES && MODE == kTriAttnIn && RB == 1;
+  typename Vec8<TZ>::type raw[kPrefetch ? KS : 1];
+  auto issue_rows = [&](int64_t t) {
+    if constexpr (kPrefetch) {
+      const int64_t wt = n_tiles - 1 - t;          // back to front, as below
+      int64_t pr = wt * 32 + (lane & 31);
+      pr = pr < p.n_rows ? pr : p.n_rows - 1;
+      const TZ* rp = (const TZ*)p.x + p.xmap(pr) + 8 * (lane >> 5);
+#pragma unroll
+      for (int kk = 0; kk < KS; ++kk) raw[kk] = load8<TZ>(rp + 16 * kk);
+    }
+  };
+  // (the first tile's rows go first: their LayerNorm then runs while the weights arrive)
+  if (kPrefetch && tile < n_tiles) issue_rows(tile);
+  // (A wait for the resident weights deferred to the first tile's first chunk, so that they
+  // would travel under that tile's row loads, was tried: the conditional barrier inside the
+  // tile loop cost the triangle-multiplication output 848 bytes of spills per lane.)
   if constexpr (RES) {
     for (int f = wave; f < IC::NFRAG; f += NW) dma_frag(f, f);
     ring_barrier<0>();
@@ -273,21 +292,6 @@ rowgemm_in_kernel(RowGemmInParams p) {
     for (int j = 0; j < FPW; ++j) lds_w[buf * 2 * SL + wave * FPW + j][lane] = pre[j];
   };
 
-  // kPrefetch: the raw rows of a tile are requested one tile ahead, so that their way from
-  // memory lies under the previous tile's chunk loop.
-  constexpr bool kPrefetch = RES && MODE == kTriAttnIn && RB == 1;
-  typename Vec8<TZ>::type raw[kPrefetch ? KS : 1];
-  auto issue_rows = [&](int64_t t) {
-    if constexpr (kPrefetch) {
-      const int64_t wt = n_tiles - 1 - t;          // back to front, as below
-      int64_t pr = wt * 32 + (lane & 31);
-      pr = pr < p.n_rows ? pr : p.n_rows - 1;
-      const TZ* rp = (const TZ*)p.x + p.xmap(pr) + 8 * (lane >> 5);
-#pragma unroll
-      for (int kk = 0; kk < KS; ++kk) raw[kk] = load8<TZ>(rp + 16 * kk);
-    }
-  };
-  if (kPrefetch && tile < n_tiles) issue_rows(tile);
   while (true) {
     if (RES && tile >= n_tiles) break;
     // The projections at the head of an update walk the pair tensor back to front.  The kernel
