@@ -351,8 +351,10 @@ rowgemm_in_kernel(RowGemmInParams p) {
 #pragma unroll
       for (int kk = 0; kk < KS; ++kk) v[kk] = to_f32(raw[kk]);
       normalize_row<T, KS, float, false>(v, lds_affine[0], lds_affine[1], p.eps, g, xf.f[0]);
+      // (no branch around the loads: with one, this instantiation spills.  A wave past its
+      // last tile reads the rows every such wave reads, out of the L2.)
       const int64_t nt = tile + tile_step;
-      issue_rows(nt < n_tiles ? nt : tile);
+      issue_rows(nt < n_tiles ? nt : n_tiles - 1);
     } else if constexpr (kLdsAffine)
       load_rows<T, RB, true, KS, float, false>(xf, (const TZ*)p.x, p.xmap, row0, p.n_rows, lds_affine[0],
                                                lds_affine[1], p.eps, lane);
