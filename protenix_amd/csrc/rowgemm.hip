@@ -305,9 +305,21 @@ rowgemm_in_kernel(RowGemmInParams p) {
     const int64_t row0 = wtile * (RB * 32);
     int pi0 = 0, pk0 = 0;
     if constexpr (MODE == kTriMulIn) {
+      // Patches in the order of the memory rows they read: the outer index is the slow one for
+      // the outgoing product (z[i][k]), the inner one for the incoming product (z[k][i]), whose
+      // walk then runs through the pair tensor's rows back to front like the other projections'
+      // instead of sweeping all rows once per strip of columns.
       const uint32_t vb = (uint32_t)(wtile >> 2);
-      const uint32_t ip = vb / n_kb;
-      pk0 = (int)(vb - ip * n_kb) * 8;
+      uint32_t ip, kb;
+      if (p.aux != 0) {
+        const uint32_t n_ip = (uint32_t)(p.n + 16 * RB - 1) / (16 * RB);
+        kb = vb / n_ip;
+        ip = vb - kb * n_ip;
+      } else {
+        ip = vb / n_kb;
+        kb = vb - ip * n_kb;
+      }
+      pk0 = (int)kb * 8;
       pi0 = (int)ip * (16 * RB) + (int)(wtile & 3) * (4 * RB);
     }
     // (resident: made opaque per tile, or the affine parameters' loads and conversions are
