@@ -2,7 +2,7 @@
 // activations and the 16-head attention with pair bias.  A thousandth of the block's work,
 // so these kernels aim at few launches and no intermediate round trips rather than at a
 // roofline: operands go from global memory (L2-resident at these sizes) straight into MFMA
-// fragments, one wave per 32 x 32 output tile, no LDS.
+// fragments; a 32 x 32 output tile belongs to one workgroup.
 //
 //   linear_kernel           out = [res +] x W^T [+ bias], optionally with a tail of the output
 //                           columns stored transposed (the attention's V^T); or, SwiGLU,
@@ -45,37 +45,52 @@ template <typename T> __device__ __forceinline__ typename Vec8<T>::type zero8() 
   return z;
 }
 
+// One workgroup per 32 x 32 output tile; its kLinWaves waves each take a quarter of K and the
+// partial tiles are summed through LDS in wave order.  The layers have 288 to 1152 tiles, a few
+// per compute unit: with four small workgroups resident per unit, all of a unit's tiles are in
+// flight together, their waves cover one another's load latency, and the fp32 MFMAs of a tile
+// are spread over the unit's four SIMDs.
+constexpr int kLinWaves = 4;
+
 template <typename T, int EPI>
-__global__ __launch_bounds__(64) void linear_kernel(LinearParams p) {
+__global__ __launch_bounds__(kLinWaves * 64, 4) void linear_kernel(LinearParams p) {
   typedef typename Vec8<T>::type V8;
   typedef typename Vec4<T>::type V4;
+  constexpr int NACC = EPI == kEpiSwiGLU ? 32 : 16;
+  __shared__ float part[kLinWaves][NACC][kWave];
   const int lane = threadIdx.x & 63, ln = lane & 31, g = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int col_blocks = (p.n_out + 31) >> 5;
   const int rb = blockIdx.x / col_blocks, cb = blockIdx.x - rb * col_blocks;
   const int row0 = rb * 32, col0 = cb * 32;
-  const bool transposed = col0 >= p.split_col;   // the same for the whole wave
+  const bool transposed = col0 >= p.split_col;   // the same for the whole workgroup
   const int xr = min(row0 + ln, p.rows - 1);
   const int wc = min(col0 + ln, p.n_out - 1);
   const T* xp = (const T*)p.x + (int64_t)xr * p.ldx + 8 * g;
   const T* wp = (const T*)p.w + (int64_t)wc * p.k + 8 * g;
   const T* wp2 = EPI == kEpiSwiGLU ? (const T*)p.w2 + (int64_t)wc * p.k + 8 * g : wp;
 
+  // K steps of 16 (k is a multiple of 16), an equal share per wave
+  const int steps = p.k >> 4;
+  const int per_wave = (steps + kLinWaves - 1) / kLinWaves;
+  const int s_begin = wave * per_wave, s_end = min(steps, s_begin + per_wave);
+
   f32x16 acc, acc2;
 #pragma unroll
   for (int r = 0; r < 16; ++r) acc[r] = acc2[r] = 0.0f;
-  constexpr int KC = 8;   // K steps of 16 requested together
-  for (int k0 = 0; k0 < p.k; k0 += 16 * KC) {
+  constexpr int KC = 3;   // K steps requested together
+  for (int s0 = s_begin; s0 < s_end; s0 += KC) {
     V8 xa[KC], wa[KC], wb[KC];
 #pragma unroll
     for (int s = 0; s < KC; ++s) {
-      const int kk = min(k0 + 16 * s, p.k - 16);   // steps beyond k re-read the last one
+      const int kk = 16 * min(s0 + s, steps - 1);   // steps beyond the slice re-read a valid one
       xa[s] = load8<T>(xp + kk);
       wa[s] = load8<T>(wp + kk);
       if (EPI == kEpiSwiGLU) wb[s] = load8<T>(wp2 + kk);
     }
 #pragma unroll
     for (int s = 0; s < KC; ++s) {
-      if (k0 + 16 * s < p.k) {
+      if (s0 + s < s_end) {
         if (transposed) {
           mma32(acc, xa[s], wa[s]);    // lane <-> column, register <-> row
         } else {
@@ -85,48 +100,51 @@ __global__ __launch_bounds__(64) void linear_kernel(LinearParams p) {
       }
     }
   }
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    part[wave][r][lane] = acc[r];
+    if (EPI == kEpiSwiGLU) part[wave][16 + r][lane] = acc2[r];
+  }
+  __syncthreads();
 
+  // wave w finishes accumulator registers 4w .. 4w + 3 of every lane: four neighbouring output
+  // columns (rows, for the transposed tail) 8*w + 4*g + {0 .. 3}
+  f32x4 y = {0.0f, 0.0f, 0.0f, 0.0f}, y2 = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+  for (int w = 0; w < kLinWaves; ++w) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      y[e] += part[w][4 * wave + e][lane];
+      if (EPI == kEpiSwiGLU) y2[e] += part[w][16 + 4 * wave + e][lane];
+    }
+  }
+  const int sub = 8 * wave + 4 * g;
   if (!transposed) {
-    const int row = row0 + ln;
+    const int row = row0 + ln, col = col0 + sub;
+    if (row < p.rows && col < p.n_out) {   // (n_out is a multiple of 4)
 #pragma unroll
-    for (int a = 0; a < 4; ++a) {
-      const int col = col0 + 8 * a + 4 * g;
-      if (row < p.rows && col < p.n_out) {   // (n_out is a multiple of 4)
-        f32x4 v;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          float y = acc[4 * a + e];
-          if (EPI == kEpiSwiGLU) {
-            // a and b rounded to T first, as the two linear layers of the reference do
-            const float av = to_f32(from_f32<T>(y)), bv = to_f32(from_f32<T>(acc2[4 * a + e]));
-            y = to_f32(from_f32<T>(av * sigmoidf_fast(av))) * bv;
-          } else if (p.bias && col + e < p.bias_cols) {
-            y += to_f32(((const T*)p.bias)[col + e]);
-          }
-          v[e] = y;
+      for (int e = 0; e < 4; ++e) {
+        if (EPI == kEpiSwiGLU) {
+          // a and b rounded to T first, as the two linear layers of the reference do
+          const float av = to_f32(from_f32<T>(y[e])), bv = to_f32(from_f32<T>(y2[e]));
+          y[e] = to_f32(from_f32<T>(av * sigmoidf_fast(av))) * bv;
+        } else if (p.bias && col + e < p.bias_cols) {
+          y[e] += to_f32(((const T*)p.bias)[col + e]);
         }
-        if (p.res) {
-          const f32x4 rv = to_f32(*reinterpret_cast<const V4*>((const T*)p.res + (int64_t)row * p.ldr + col));
-#pragma unroll
-          for (int e = 0; e < 4; ++e) v[e] = to_f32(from_f32<T>(v[e])) + rv[e];
-        }
-        *reinterpret_cast<V4*>((T*)p.out + (int64_t)row * p.ldo + col) = from_f32<T>(v);
       }
+      if (p.res) {
+        const f32x4 rv = to_f32(*reinterpret_cast<const V4*>((const T*)p.res + (int64_t)row * p.ldr + col));
+#pragma unroll
+        for (int e = 0; e < 4; ++e) y[e] = to_f32(from_f32<T>(y[e])) + rv[e];
+      }
+      *reinterpret_cast<V4*>((T*)p.out + (int64_t)row * p.ldo + col) = from_f32<T>(y);
     }
   } else {
-    const int col = col0 + ln;
-    if (col < p.n_out) {
-      T* dst = (T*)p.out_t + (int64_t)(col - p.split_col) * p.ldt;
+    const int col = col0 + ln, row = row0 + sub;
+    if (col < p.n_out && row < p.ldt) {   // (ldt is a multiple of 4)
 #pragma unroll
-      for (int a = 0; a < 4; ++a) {
-        const int row = row0 + 8 * a + 4 * g;
-        if (row < p.ldt) {   // (ldt is a multiple of 4)
-          f32x4 v;
-#pragma unroll
-          for (int e = 0; e < 4; ++e) v[e] = row + e < p.rows ? acc[4 * a + e] : 0.0f;
-          *reinterpret_cast<V4*>(dst + row) = from_f32<T>(v);
-        }
-      }
+      for (int e = 0; e < 4; ++e) y[e] = row + e < p.rows ? y[e] : 0.0f;
+      *reinterpret_cast<V4*>((T*)p.out_t + (int64_t)(col - p.split_col) * p.ldt + row) = from_f32<T>(y);
     }
   }
 }
@@ -154,7 +172,7 @@ int linear_fwd(const void* x, const void* w, const void* bias, int bias_cols, co
   p.n_out = n_out;
   const int64_t row_span = (p.split_col < n_out && ldt > rows) ? ldt : rows;
   const int64_t tiles = ((row_span + 31) / 32) * ((n_out + 31) / 32);
-  linear_kernel<T, kEpiStore><<<dim3((unsigned)tiles), dim3(64), 0, stream>>>(p);
+  linear_kernel<T, kEpiStore><<<dim3((unsigned)tiles), dim3(kLinWaves * 64), 0, stream>>>(p);
   return 0;
 }
 
@@ -174,7 +192,7 @@ int swiglu_fwd(const void* x, const void* w_a, const void* w_b, void* out, int r
   p.k = k;
   p.n_out = hidden;
   const int64_t tiles = (((int64_t)rows + 31) / 32) * ((hidden + 31) / 32);
-  linear_kernel<T, kEpiSwiGLU><<<dim3((unsigned)tiles), dim3(64), 0, stream>>>(p);
+  linear_kernel<T, kEpiSwiGLU><<<dim3((unsigned)tiles), dim3(kLinWaves * 64), 0, stream>>>(p);
   return 0;
 }
 
