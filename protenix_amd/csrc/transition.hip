@@ -31,13 +31,17 @@ namespace ptx {
 // NOB = c / 32 output blocks.
 template <typename T, int KS> struct TrCfg {
   // (rows of 256 channels, bf16 only: one row block, and three 48 KB chunk buffers)
-  // Waves per workgroup.  bf16 rows of 128 channels: 8 waves (two per SIMD) of one row block
-  // each.  A single wave issues a vector instruction only every ~9 cycles (two waves: one every
+  // Four waves per workgroup.  bf16 rows of 128 channels: one row block per wave and a ring of
+  // three chunk buffers (72 KB), so that two workgroups share a compute unit, two waves per
+  // SIMD.  A single wave issues a vector instruction only every ~9 cycles (two waves: one every
   // ~5 per SIMD), and the SwiGLU is vector work, so two thin waves beat one fat one by 6 %
-  // although every weight fragment read from LDS then feeds one MFMA instead of two.
-  static constexpr int NW = (sizeof(T) == 2 && KS == 8) ? 8 : 4;
-  static constexpr int RB = (sizeof(T) == 2 && KS <= 8 && NW == 4) ? 2 : 1;     // row blocks of 32 per wave
-  static constexpr int NBUF = (sizeof(T) == 2 && KS <= 8) ? 4 : 3;   // chunk buffers in LDS
+  // although every weight fragment read from LDS then feeds one MFMA instead of two; and two
+  // workgroups of four beat one of eight by another 7 % although the weights then stream into
+  // LDS twice per 256 rows: a workgroup's row loads, LayerNorm and stores leave the matrix pipe
+  // idle unless another workgroup, at another point of its life, has the unit's other waves.
+  static constexpr int NW = 4;
+  static constexpr int RB = (sizeof(T) == 2 && KS == 4) ? 2 : 1;     // row blocks of 32 per wave
+  static constexpr int NBUF = (sizeof(T) == 2 && KS == 4) ? 4 : 3;   // chunk buffers in LDS
   static constexpr int D = NBUF - 2;                    // chunks the loads run ahead (two are in use)
   static constexpr int PIECES = (int)sizeof(T) / 2;     // 16-byte pieces per lane and fragment
   static constexpr int NOB = KS / 2;
@@ -106,7 +110,7 @@ struct PairBiasArgs {
 };
 
 template <typename T, int KS, typename TZ = T, bool PB = false>
-__global__ __launch_bounds__((TrCfg<T, KS>::NW * 64)) void transition_fused_kernel(
+__global__ __launch_bounds__((TrCfg<T, KS>::NW * 64), 2) void transition_fused_kernel(
     const TZ* x, const T* __restrict__ gamma, const T* __restrict__ beta,
     const T* __restrict__ packed, TZ* out, int64_t n_rows, int n_chunks, int add_residual,
     float eps, PairBiasArgs pb) {
@@ -126,16 +130,12 @@ __global__ __launch_bounds__((TrCfg<T, KS>::NW * 64)) void transition_fused_kern
   // front to back, and its tail is what the memory-side cache still holds.
   const int64_t row0 = ((int64_t)(gridDim.x - 1 - blockIdx.x) * NW + wave) * (RB * 32);
 
-  // PB: the bias' weight as A fragments (rows beyond `heads` repeat the last head: those
-  // accumulator rows are not stored) and its LayerNorm parameters as fp32, parked in LDS for
-  // the epilogue: fetched there from global memory they would cost every tile a round trip
-  // that nothing hides.  (Visible to all waves after the first ring barrier below.)
-  __shared__ V8 lds_pbw[PB ? KS : 1][kWave];
+  // PB: the bias' LayerNorm parameters as fp32, parked in LDS for the epilogue: fetched there
+  // from global memory they would cost every tile a round trip that nothing hides.  (Visible
+  // to all waves after the first ring barrier below.)  The bias' weight follows into the
+  // freed chunk buffers when the epilogue starts.
   __shared__ __attribute__((aligned(16))) float lds_pba[2][PB ? 16 * KS : 4];
   if constexpr (PB) {
-    static_assert(!PB || NW == KS, "one weight fragment per wave");
-    lds_pbw[wave][lane] = load8<T>((const T*)pb.w + (int64_t)min(lane & 31, pb.heads - 1) * kCx +
-                                   16 * wave + 8 * (lane >> 5));
     for (int c = threadIdx.x; c < kCx; c += NW * kWave) {
       lds_pba[0][c] = pb.gamma ? to_f32(((const T*)pb.gamma)[c]) : 1.0f;
       lds_pba[1][c] = pb.beta ? to_f32(((const T*)pb.beta)[c]) : 0.0f;
@@ -298,6 +298,20 @@ __global__ __launch_bounds__((TrCfg<T, KS>::NW * 64)) void transition_fused_kern
   // every wave is past its last fragment read and all loads have landed) ----
   ring_barrier<0>();
   TZ* st = reinterpret_cast<TZ*>(&lds_w[0][0][0][0]) + wave * (32 * C::PITCH);
+  // PB: the bias' weight as A fragments (rows beyond `heads` repeat the last head: those
+  // accumulator rows are not stored), behind the staging and normalised tiles; it arrives
+  // by direct-to-LDS loads while the rows are stored (waited for before its first use).
+  constexpr int kPitchN = 64 + 4;      // normalised tile, elements: 34 dwords, rows 8-byte aligned
+  constexpr size_t kPbwOffset = PB ? (NW * 32 * (C::PITCH * sizeof(TZ) + kPitchN * sizeof(T)) + 1023) / 1024 * 1024 : 0;
+  static_assert(!PB || kPbwOffset + KS * kWave * sizeof(V8) <= sizeof(u32x4_t) * NBUF * kTrFrags * PIECES * kWave,
+                "staging tiles, normalised tiles and the bias weight fit the chunk buffers");
+  V8 (*lds_pbw)[kWave] = reinterpret_cast<V8 (*)[kWave]>(reinterpret_cast<char*>(&lds_w[0][0][0][0]) + kPbwOffset);
+  if constexpr (PB) {
+    static_assert(!PB || sizeof(V8) == 16, "one 16-byte piece per lane and fragment");
+    const uint32_t voff = (uint32_t)((min(lane & 31, pb.heads - 1) * kCx + 8 * (lane >> 5)) * sizeof(T));
+    for (int f = wave; f < KS; f += NW)
+      load_to_lds16_s<0>(uniform64((uint64_t)((const T*)pb.w + 16 * f)), voff, lds_address(&lds_pbw[f][0]));
+  }
   VE_t done[PB ? RB : 1][PB ? NOB : 1][PB ? C::NPASS : 1];   // PB: the finished rows, as stored
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
@@ -353,7 +367,6 @@ __global__ __launch_bounds__((TrCfg<T, KS>::NW * 64)) void transition_fused_kern
     }
     // per wave: 32 rows x 64 normalised columns in T, behind all waves' staging tiles (other
     // waves may still be storing their rows)
-    constexpr int kPitchN = 64 + 4;      // elements: 34 dwords, rows 8-byte aligned
     static_assert(NW * 32 * (C::PITCH * sizeof(TZ) + kPitchN * sizeof(T)) <=
                       sizeof(u32x4_t) * (NBUF - 1) * kTrFrags * PIECES * kWave,
                   "staging tiles and normalised tiles fit the chunk buffers");
@@ -362,6 +375,8 @@ __global__ __launch_bounds__((TrCfg<T, KS>::NW * 64)) void transition_fused_kern
     f32x16 accb;
 #pragma unroll
     for (int r = 0; r < 16; ++r) accb[r] = 0.0f;
+    // every wave's share of the bias weight has landed (and this wave's row stores are out)
+    ring_barrier<0>();
 #pragma unroll
     for (int hb = 0; hb < NOB / 2; ++hb) {   // 64 columns at a time
       wave_lds_sync();
