@@ -212,6 +212,22 @@ PTX_API int ptx_triattn_fwd(const void* q, const void* k, const void* vt, const 
                     int key_pitch, int mask_transposed, float inf, int dtype, void* stream);
 
 /*
+ * The same stage on rows row_begin .. row_begin + row_count - 1 only, with keys 0 .. n_keys - 1
+ * taking part and the keys from n_keys on treated as masked for every row of the range (weight
+ * exactly zero, which is what inf*(mask-1) gives a masked key of a row that has unmasked ones,
+ * layers.py:286-291).  For the pair masks of padded batches, mask = m (x) m with the padding at
+ * the end (the reference's pair_mask, pairformer.py:103-112 from loss.py:589): the n_valid valid
+ * rows go through one call with mask = NULL, n_keys = n_valid, which neither loads a mask nor
+ * visits the padded keys; the padded rows, whose keys are all masked, through a second call
+ * with the mask and n_keys = n.  All tensors are the whole-tensor ones of ptx_triattn_fwd;
+ * ptx_triattn_fwd is this call with row_begin = 0, row_count = n, n_keys = n.
+ */
+PTX_API int ptx_triattn_fwd_rows(const void* q, const void* k, const void* vt, const void* g,
+                                 const void* tri_bias, const void* mask, void* o, int n, int heads,
+                                 int d, int key_pitch, int mask_transposed, float inf, int row_begin,
+                                 int row_count, int n_keys, int dtype, void* stream);
+
+/*
  * The fused attention operator on standard-layout tensors: the contract of
  * TriAttentionFunction.forward (tri_attention/op.py:37-77, kernel tri_attention/forward.py:22-188)
  * as called from layers.py:539-583.  For every batch b, row i, head h, query position j:

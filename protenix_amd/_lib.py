@@ -38,6 +38,7 @@ SIGNATURES = {
     "ptx_trimul_output": (_i, [_p] * 9 + [_i, _i, _i, _i, _f, _i, _p]),
     "ptx_triattn_project": (_i, [_p] * 13 + [_i, _i, _i, _i, _i, _i, _f, _i, _p]),
     "ptx_triattn_fwd": (_i, [_p] * 7 + [_i, _i, _i, _i, _i, _f, _i, _p]),
+    "ptx_triattn_fwd_rows": (_i, [_p] * 7 + [_i, _i, _i, _i, _i, _f, _i, _i, _i, _i, _p]),
     "ptx_triattn_output": (_i, [_p, _p, _p, _p, _i, _i, _i, _i, _i, _p]),
     "ptx_triattn_core_workspace_elems": (_l, [_i, _i, _i]),
     "ptx_triattn_core_fwd": (_i, [_p] * 8 + [_i, _i, _i, _i, _i, _i, _p]),

@@ -284,25 +284,46 @@ PTX_API int ptx_triattn_project(const void* z, const void* ln_w, const void* ln_
   return after_launch("triattn_project");
 }
 
+static int triattn_fwd_checked(const char* what, const void* q, const void* k, const void* vt,
+                               const void* g, const void* tri_bias, const void* mask, void* o, int n,
+                               int heads, int d, int key_pitch, int mask_transposed, float inf,
+                               int row_begin, int row_count, int n_keys, int dtype, void* stream) {
+  if (dtype == PTX_MIXED) dtype = PTX_BF16;   // no residual-stream tensor here
+  PTX_REQUIRE(dtype_ok(dtype), PTX_ERR_BAD_ARG, "%s: unknown dtype %d", what, dtype);
+  PTX_REQUIRE(n >= 0 && heads >= 0, PTX_ERR_BAD_ARG, "%s: n=%d heads=%d", what, n, heads);
+  PTX_REQUIRE(d == 32, PTX_ERR_UNSUPPORTED, "%s: only head dim 32 is built (got %d)", what, d);
+  PTX_REQUIRE(key_pitch == ptx_key_pitch(n), PTX_ERR_BAD_ARG, "%s: key_pitch=%d, expected %d", what,
+              key_pitch, ptx_key_pitch(n));
+  PTX_REQUIRE(n < 32768, PTX_ERR_UNSUPPORTED, "%s: n=%d too large", what, n);
+  PTX_REQUIRE(row_begin >= 0 && row_count >= 0 && row_begin <= n - row_count, PTX_ERR_BAD_ARG,
+              "%s: rows %d .. +%d of %d", what, row_begin, row_count, n);
+  PTX_REQUIRE(n_keys >= (n > 0) && n_keys <= n, PTX_ERR_BAD_ARG, "%s: n_keys=%d of %d", what, n_keys, n);
+  if (n == 0 || heads == 0 || row_count == 0) return PTX_OK;
+  PTX_REQUIRE(q && k && vt && tri_bias && o, PTX_ERR_BAD_ARG, "%s: null pointer", what);
+  PTX_REQUIRE(aligned16(q) && aligned16(k) && aligned16(vt) && (!g || aligned16(g)) &&
+                  aligned16(tri_bias) && aligned16(o),
+              PTX_ERR_BAD_ARG, "%s: pointers must be 16-byte aligned", what);
+  PTX_DISPATCH(dtype, ptx::triattn_fwd<T>((const T*)q, (const T*)k, (const T*)vt, (const T*)g,
+                                          (const T*)tri_bias, (const T*)mask, (T*)o, n, heads,
+                                          key_pitch, mask_transposed, inf, row_begin, row_count,
+                                          n_keys, (hipStream_t)stream));
+  return after_launch(what);
+}
+
 PTX_API int ptx_triattn_fwd(const void* q, const void* k, const void* vt, const void* g,
                     const void* tri_bias, const void* mask, void* o, int n, int heads, int d,
                     int key_pitch, int mask_transposed, float inf, int dtype, void* stream) {
-  if (dtype == PTX_MIXED) dtype = PTX_BF16;   // no residual-stream tensor here
-  PTX_REQUIRE(dtype_ok(dtype), PTX_ERR_BAD_ARG, "triattn_fwd: unknown dtype %d", dtype);
-  PTX_REQUIRE(n >= 0 && heads >= 0, PTX_ERR_BAD_ARG, "triattn_fwd: n=%d heads=%d", n, heads);
-  PTX_REQUIRE(d == 32, PTX_ERR_UNSUPPORTED, "triattn_fwd: only head dim 32 is built (got %d)", d);
-  PTX_REQUIRE(key_pitch == ptx_key_pitch(n), PTX_ERR_BAD_ARG,
-              "triattn_fwd: key_pitch=%d, expected %d", key_pitch, ptx_key_pitch(n));
-  PTX_REQUIRE(n < 32768, PTX_ERR_UNSUPPORTED, "triattn_fwd: n=%d too large", n);
-  if (n == 0 || heads == 0) return PTX_OK;
-  PTX_REQUIRE(q && k && vt && tri_bias && o, PTX_ERR_BAD_ARG, "triattn_fwd: null pointer");
-  PTX_REQUIRE(aligned16(q) && aligned16(k) && aligned16(vt) && (!g || aligned16(g)) &&
-                  aligned16(tri_bias) && aligned16(o),
-              PTX_ERR_BAD_ARG, "triattn_fwd: pointers must be 16-byte aligned");
-  PTX_DISPATCH(dtype, ptx::triattn_fwd<T>((const T*)q, (const T*)k, (const T*)vt, (const T*)g,
-                                          (const T*)tri_bias, (const T*)mask, (T*)o, n, heads,
-                                          key_pitch, mask_transposed, inf, (hipStream_t)stream));
-  return after_launch("triattn_fwd");
+  return triattn_fwd_checked("triattn_fwd", q, k, vt, g, tri_bias, mask, o, n, heads, d, key_pitch,
+                             mask_transposed, inf, 0, n, n, dtype, stream);
+}
+
+PTX_API int ptx_triattn_fwd_rows(const void* q, const void* k, const void* vt, const void* g,
+                                 const void* tri_bias, const void* mask, void* o, int n, int heads,
+                                 int d, int key_pitch, int mask_transposed, float inf, int row_begin,
+                                 int row_count, int n_keys, int dtype, void* stream) {
+  return triattn_fwd_checked("triattn_fwd_rows", q, k, vt, g, tri_bias, mask, o, n, heads, d,
+                             key_pitch, mask_transposed, inf, row_begin, row_count, n_keys, dtype,
+                             stream);
 }
 
 PTX_API int64_t ptx_triattn_core_workspace_elems(int n_rows, int s, int heads) {
@@ -353,7 +374,7 @@ PTX_API int ptx_triattn_core_fwd(const void* q, const void* k, const void* v, co
       ptx::triattn_fwd_ex<T>((const T*)qs, (const T*)kf, (const T*)vtf, (const T*)nullptr,
                              (const T*)bf, (const T*)b1, (T*)ob, n_rows, s, heads, pitch, 0, 0.0f, 1,
                              32, (int64_t)s * heads * 32, (int64_t)heads * 32, lb, 1,
-                             (int64_t)s * heads, heads, (hipStream_t)stream);
+                             (int64_t)s * heads, heads, 0, n_rows, s, (hipStream_t)stream);
     });
   }
   return after_launch("triattn_core_fwd");

@@ -93,15 +93,18 @@ int nt_gemm_batched(const T* a, const T* b, T* x, int n, int k_pitch, int batch,
 template <typename T>
 int triattn_fwd(const T* q, const T* k, const T* vt, const T* g, const T* tri_bias, const T* mask,
                 T* o, int n, int heads, int key_pitch, int mask_transposed, float inf,
-                hipStream_t stream);
+                int row_begin, int row_count, int n_keys, hipStream_t stream);
 // The same core on n_rows rows of n queries / keys, with q / g / o addressed through element
 // strides (head, row, query), an optional gate (g may be null), the mask either 0/1 values or
 // (mask_is_bias) an additive bias per (row, key), and an optional log2-sum-exp2 output.
+// The launch covers rows row_begin .. row_begin + row_count - 1 and lets keys 0 .. n_keys - 1
+// take part (keys beyond count as masked: weight exactly zero).
 template <typename T>
 int triattn_fwd_ex(const T* q, const T* k, const T* vt, const T* g, const T* tri_bias,
                    const T* mask, T* o, int n_rows, int n, int heads, int key_pitch,
                    int mask_transposed, float inf, int mask_is_bias, int64_t sh, int64_t si,
-                   int64_t sj, float* lse, int64_t lh, int64_t li, int64_t lj, hipStream_t stream);
+                   int64_t sj, float* lse, int64_t lh, int64_t li, int64_t lj, int row_begin,
+                   int row_count, int n_keys, hipStream_t stream);
 // Standard-layout K, V [n_rows][n][heads][32] and bias [heads][n][n] -> the core's fragment-
 // ordered K, V^T and bias (bias and nothing else multiplied by log2(e)); q [n_rows][n][heads][32]
 // -> qs, the same layout multiplied by log2(e).

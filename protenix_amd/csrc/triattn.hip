@@ -53,6 +53,8 @@ struct AttnAux {
   int mask_is_bias;
   float* lse;             // or null
   int64_t lh, li, lj;     // element strides of lse: head, row, query
+  int row0;               // first row of this launch (a launch may cover a range of the rows)
+  int n_keys;             // keys 0 .. n_keys-1 take part (n_keys <= n; the rest count as masked)
 };
 
 // Rows of the pair tensor handled by one wave: one (more would share the bias tile, but do not
@@ -67,10 +69,9 @@ struct AttnAux {
 // 0/1 values turned into inf*(mask-1), or with ax.mask_is_bias an additive bias used as it is.
 // ax.lse: optional log2-sum-exp2 of the logits per (head, row, query).
 // MK: kMaskGiven, or no mask (its own instantiations: a mask of all ones is passed as none by
-// the host side).  Without a mask only a last, partial key tile publishes a per-key bias
-// (-inf beyond n), and no other tile pays for the mask's load, its LDS round trip or the test of
-// its values (kMaskTail); where the keys fill whole tiles nothing of the masked path is left in
-// the kernel (kMaskNone).
+// the host side).  Without a mask nothing of the masked path is left in the kernel; a last,
+// partial key tile takes the same paths as the others with the logits of the keys beyond
+// n_keys set to -inf (kMaskTail; kMaskNone where the keys fill whole tiles).
 enum { kMaskNone = 0, kMaskTail = 1, kMaskGiven = 2 };
 template <typename T, int R, int NWQ, int MK>
 __global__ __launch_bounds__((NWQ * 64), (sizeof(T) == 2 ? 16 / NWQ : 2)) void triattn_fwd_kernel(
@@ -93,13 +94,14 @@ __global__ __launch_bounds__((NWQ * 64), (sizeof(T) == 2 ? 16 / NWQ : 2)) void t
   const int64_t item = (int64_t)(blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
   if (item >= total_items) return;
   const int qt = (int)(item % n_qtiles);
-  const int i0 = (int)((item / n_qtiles) % n_rowgroups) * R;   // first of this workgroup's R rows
+  const int i0 = ax.row0 + (int)((item / n_qtiles) % n_rowgroups) * R;   // first of this workgroup's R rows
   const int h = (int)(item / ((int64_t)n_qtiles * n_rowgroups));
 
   const int q0 = (qt * NWQ + wave) * 32;   // first query of this wave
   const int key_tiles = key_pitch >> 6;
   const int q_blocks = (n + 31) >> 5;
-  const int n_tiles = (n + kKeyTile - 1) / kKeyTile;
+  const int nk = ax.n_keys;
+  const int n_tiles = (nk + kKeyTile - 1) / kKeyTile;
   constexpr bool has_mask = MK == kMaskGiven;
   // Operand tiles in fragment order (common.h): 2048 elements per key tile, this lane's
   // 8 elements of fragment f at f*512 + lane*8.  Rows beyond n re-read row n-1, a wave whose
@@ -129,8 +131,9 @@ __global__ __launch_bounds__((NWQ * 64), (sizeof(T) == 2 ? 16 / NWQ : 2)) void t
   // `tile` may run past the last tile: the pipeline below never branches around a load, so
   // that the compiler can count the outstanding loads exactly.  Addresses use the clamped
   // tile; the mask bias and the V^T zeroing use the real key index, which makes a phantom
-  // tile contribute exactly nothing.  Keys beyond n hold garbage in K (removed by the -inf
-  // mask bias) and are zeroed in V^T (0 * garbage must stay 0).
+  // tile contribute exactly nothing.  Keys beyond n_keys hold garbage (or, below n, keys that
+  // are left out) in K, removed by the -inf mask bias, and are zeroed in V^T (0 * garbage must
+  // stay 0).
   // fetch() only issues loads; everything that consumes a loaded value (mask -> additive
   // bias, zeroing of V^T beyond n) happens in stash(), one tile of work later, so no wait
   // for memory sits in the issue path.
@@ -159,7 +162,7 @@ __global__ __launch_bounds__((NWQ * 64), (sizeof(T) == 2 ? 16 / NWQ : 2)) void t
   auto stash = [&](int tile) {
     const int buf = tile % 3;
     const int key0 = tile * kKeyTile;
-    const bool tail = key0 + kKeyTile > n;   // uniform
+    const bool tail = key0 + kKeyTile > nk;   // uniform
 #pragma unroll
     for (int j = 0; j < FPW; ++j) {
       const int fid = wave * FPW + j;
@@ -169,13 +172,15 @@ __global__ __launch_bounds__((NWQ * 64), (sizeof(T) == 2 ? 16 / NWQ : 2)) void t
         // V^T fragment (u, s): slots <-> keys 32g + 16u + 8s + t
         const int koff = key0 + 32 * g + 16 * ((f >> 1) & 1) + 8 * (f & 1);
 #pragma unroll
-        for (int t = 0; t < 8; ++t) v[t] = koff + t < n ? v[t] : (T)0.0f;
+        for (int t = 0; t < 8; ++t) v[t] = koff + t < nk ? v[t] : (T)0.0f;
       }
       lds_kv[buf][fid >> 3][f][lane] = v;
     }
-    if (wave < R && (has_mask || (MK == kMaskTail && tail))) {
-      const float mb = !has_mask ? 0.0f : ax.mask_is_bias ? to_f32(pre_mv) : inf * (to_f32(pre_mv) - 1.0f);
-      lds_mb[buf][wave][lane] = key0 + lane < n ? mb : -INFINITY;
+    if constexpr (has_mask) {
+      if (wave < R) {
+        const float mb = ax.mask_is_bias ? to_f32(pre_mv) : inf * (to_f32(pre_mv) - 1.0f);
+        lds_mb[buf][wave][lane] = key0 + lane < nk ? mb : 0.0f;   // (beyond n_keys: see TAIL)
+      }
     }
   };
 
@@ -225,9 +230,15 @@ __global__ __launch_bounds__((NWQ * 64), (sizeof(T) == 2 ? 16 / NWQ : 2)) void t
     V8 pf[2];
     float psum, alpha;
   };
-  auto half_row = [&](auto mode_tag, int buf, int u, V8 (&tbh)[2], HalfOut& out) -> bool {
+  // TAIL: the tile holds keys beyond n_keys; their logits, whatever was made of the K rows and
+  // mask values found there, are replaced by -inf before the softmax (weight zero).  The other
+  // keys of such a tile take the same path as in any other tile, so a mask of all ones gives
+  // the bits that no mask gives.
+  auto half_row = [&](auto mode_tag, auto tail_tag, int buf, int u, int key0, V8 (&tbh)[2],
+                      HalfOut& out) -> bool {
     constexpr int MODE = decltype(mode_tag)::value;
     constexpr bool MASKED = MODE == kMasked;
+    constexpr bool TAIL = decltype(tail_tag)::value;
     V8 kf[2];
 #pragma unroll
     for (int kk = 0; kk < 2; ++kk) kf[kk] = lds_kv[buf][0][u * 2 + kk][lane];
@@ -257,6 +268,11 @@ __global__ __launch_bounds__((NWQ * 64), (sizeof(T) == 2 ? 16 / NWQ : 2)) void t
           s[8 * c + t] = mbv == -INFINITY ? -INFINITY : v;
         }
       }
+    }
+    if constexpr (TAIL) {
+      const int kfirst = key0 + 32 * g + 16 * u;   // register e <-> key kfirst + e
+#pragma unroll
+      for (int e = 0; e < 16; ++e) s[e] = kfirst + e < nk ? s[e] : -INFINITY;
     }
     float alpha = 1.0f;
     if constexpr (MODE == kClassic || MODE == kMasked) {
@@ -319,28 +335,37 @@ __global__ __launch_bounds__((NWQ * 64), (sizeof(T) == 2 ? 16 / NWQ : 2)) void t
   auto process_tile = [&](int tile, V8 (&tb)[2][2]) {
     static_assert(R == 1, "the register budget of four waves per SIMD holds one row per wave");
     const int buf = tile % 3;
+    const int key0 = tile * kKeyTile;
     // keys of the tile with a non-zero mask bias, as a lane mask (key <-> lane); half u's keys
     // are the lanes with bit 4 == u
-    const uint64_t mb_mask = (has_mask || (MK == kMaskTail && tile * kKeyTile + kKeyTile > n))
-                                 ? __builtin_amdgcn_ballot_w64(lds_mb[buf][0][lane] != 0.0f)
-                                 : 0ull;
+    uint64_t mb_mask = 0ull;
+    if constexpr (has_mask) mb_mask = __builtin_amdgcn_ballot_w64(lds_mb[buf][0][lane] != 0.0f);
+    const bool tail_tile = MK != kMaskNone && key0 + kKeyTile > nk;   // uniform
+    // the unmasked paths of one half: optimistic against the reference the earlier tiles left,
+    // classic if there is none yet or the optimistic one had to give up
+    auto unmasked_half = [&](auto tail_tag, int u, HalfOut& out) -> bool {
+      bool done = false;
+      if (tile != 0 || u != 0) {
+        if ((__builtin_amdgcn_ballot_w64(m_run[0] != 0.0f) & q_ok_mask) == 0ull)
+          done = half_row(std::integral_constant<int, kOptimisticZero>{}, tail_tag, buf, u, key0, tb[u], out);
+        else
+          done = half_row(std::integral_constant<int, kOptimistic>{}, tail_tag, buf, u, key0, tb[u], out);
+      }
+      if (!done) half_row(std::integral_constant<int, kClassic>{}, tail_tag, buf, u, key0, tb[u], out);
+      return !done;   // classic: O and l are rescaled first
+    };
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
       HalfOut out;
       bool rescale = true;
       // this half's keys are those of lanes with bit 4 == u
-      if ((mb_mask & (u ? 0xffff0000ffff0000ull : 0x0000ffff0000ffffull)) != 0ull) {
-        half_row(std::integral_constant<int, kMasked>{}, buf, u, tb[u], out);
+      if (has_mask && (mb_mask & (u ? 0xffff0000ffff0000ull : 0x0000ffff0000ffffull)) != 0ull) {
+        if (tail_tile) half_row(std::integral_constant<int, kMasked>{}, std::true_type{}, buf, u, key0, tb[u], out);
+        else half_row(std::integral_constant<int, kMasked>{}, std::false_type{}, buf, u, key0, tb[u], out);
+      } else if (tail_tile) {
+        rescale = unmasked_half(std::true_type{}, u, out);
       } else {
-        bool done = false;
-        if (tile != 0 || u != 0) {
-          if ((__builtin_amdgcn_ballot_w64(m_run[0] != 0.0f) & q_ok_mask) == 0ull)
-            done = half_row(std::integral_constant<int, kOptimisticZero>{}, buf, u, tb[u], out);
-          else
-            done = half_row(std::integral_constant<int, kOptimistic>{}, buf, u, tb[u], out);
-        }
-        if (!done) half_row(std::integral_constant<int, kClassic>{}, buf, u, tb[u], out);
-        else rescale = false;
+        rescale = unmasked_half(std::false_type{}, u, out);
       }
       if (rescale) {
 #pragma unroll
@@ -412,7 +437,7 @@ __global__ __launch_bounds__((NWQ * 64), (sizeof(T) == 2 ? 16 / NWQ : 2)) void t
 template <typename T>
 int triattn_fwd(const T* q, const T* k, const T* vt, const T* g, const T* tri_bias, const T* mask,
                 T* o, int n, int heads, int key_pitch, int mask_transposed, float inf,
-                hipStream_t stream) {
+                int row_begin, int row_count, int n_keys, hipStream_t stream) {
   // head-major q, gate, o of a whole pair tensor: [heads][n][n][32]
   AttnAux ax = {};
   ax.sh = (int64_t)n * n * kD;
@@ -420,30 +445,31 @@ int triattn_fwd(const T* q, const T* k, const T* vt, const T* g, const T* tri_bi
   ax.sj = kD;
   ax.n_rows = n;
   return triattn_fwd_ex<T>(q, k, vt, g, tri_bias, mask, o, n, n, heads, key_pitch, mask_transposed, inf,
-                           0, ax.sh, ax.si, ax.sj, nullptr, 0, 0, 0, stream);
+                           0, ax.sh, ax.si, ax.sj, nullptr, 0, 0, 0, row_begin, row_count, n_keys, stream);
 }
 
 template <typename T>
 int triattn_fwd_ex(const T* q, const T* k, const T* vt, const T* g, const T* tri_bias,
                    const T* mask, T* o, int n_rows, int n, int heads, int key_pitch,
                    int mask_transposed, float inf, int mask_is_bias, int64_t sh, int64_t si,
-                   int64_t sj, float* lse, int64_t lh, int64_t li, int64_t lj, hipStream_t stream) {
-  if (n == 0 || n_rows == 0) return 0;
-  AttnAux ax = {sh, si, sj, n_rows, mask_is_bias, lse, lh, li, lj};
+                   int64_t sj, float* lse, int64_t lh, int64_t li, int64_t lj, int row_begin,
+                   int row_count, int n_keys, hipStream_t stream) {
+  if (n == 0 || n_rows == 0 || row_count == 0) return 0;
+  AttnAux ax = {sh, si, sj, n_rows, mask_is_bias, lse, lh, li, lj, row_begin, n_keys};
   constexpr int R = PTX_ATTN_ROWS;
   // 8-wave workgroups for long rows (measured: +2 % at n = 768, even at 1024, -2.6 % at 1536,
   // -2.2 % at 2048), where their 256 queries divide n or n is large enough for the idle waves
   // of the last one not to matter
   const bool wide = sizeof(T) == 2 && ((n % 256 == 0 && n >= 1536) || n >= 2048);
   const int n_qtiles = wide ? (n + 255) / 256 : (n + 127) / 128;
-  const int n_rowgroups = (n_rows + R - 1) / R;
+  const int n_rowgroups = (row_count + R - 1) / R;
   const int64_t total = (int64_t)heads * n_rowgroups * n_qtiles;
   const int64_t per_xcd = (total + 7) / 8;
 #define PTX_ATTN_LAUNCH(NWQ, MK)                                                                  \
   triattn_fwd_kernel<T, R, NWQ, MK><<<dim3((unsigned)(per_xcd * 8)), dim3(NWQ * 64), 0, stream>>>( \
       q, k, vt, g, tri_bias, mask, o, n, heads, key_pitch, mask_transposed, inf, n_qtiles,        \
       n_rowgroups, total, ax)
-  const int mk = mask ? kMaskGiven : n % kKeyTile ? kMaskTail : kMaskNone;
+  const int mk = mask ? kMaskGiven : n_keys % kKeyTile ? kMaskTail : kMaskNone;
   if (wide) {
     if (mk == kMaskGiven) PTX_ATTN_LAUNCH(8, kMaskGiven);
     else if (mk == kMaskTail) PTX_ATTN_LAUNCH(8, kMaskTail);
@@ -460,15 +486,15 @@ int triattn_fwd_ex(const T* q, const T* k, const T* vt, const T* g, const T* tri
 #define PTX_INSTANTIATE_EX(T)                                                                     \
   template int triattn_fwd_ex<T>(const T*, const T*, const T*, const T*, const T*, const T*, T*,  \
                                  int, int, int, int, int, float, int, int64_t, int64_t, int64_t,  \
-                                 float*, int64_t, int64_t, int64_t, hipStream_t);
+                                 float*, int64_t, int64_t, int64_t, int, int, int, hipStream_t);
 PTX_INSTANTIATE_EX(float)
 PTX_INSTANTIATE_EX(bf16_t)
 #undef PTX_INSTANTIATE_EX
 template int triattn_fwd<float>(const float*, const float*, const float*, const float*,
                                 const float*, const float*, float*, int, int, int, int, float,
-                                hipStream_t);
+                                int, int, int, hipStream_t);
 template int triattn_fwd<bf16_t>(const bf16_t*, const bf16_t*, const bf16_t*, const bf16_t*,
                                  const bf16_t*, const bf16_t*, bf16_t*, int, int, int, int, float,
-                                 hipStream_t);
+                                 int, int, int, hipStream_t);
 
 }  // namespace ptx

@@ -4,7 +4,9 @@ Below a few hundred tokens the forward pass is bound by the host: a block issues
 kernel launches and the GPU finishes them faster than Python can enqueue them.  `Graphed`
 records one forward pass of a `PairformerBlock` / `PairformerStack` into a HIP graph (through
 `torch.cuda.CUDAGraph`, which also captures the second stream the stack uses for the single
-track) and replays it for every later call with the same shapes and dtypes.
+track) and replays it for every later call with the same shapes and dtypes (and, for a single
+pair mask, the same class of mask: padding at the end with the same number of valid tokens, or
+any other mask - the class decides which attention kernels a forward pass launches).
 
     fast = protenix_amd.Graphed(stack)          # stack: eval mode, on the GPU
     s, z = fast(s, z, pair_mask)                # first call per shape: warm-up + capture
@@ -23,6 +25,8 @@ from typing import Dict, Optional, Tuple
 import torch
 import torch.nn as nn
 
+from . import ops
+
 
 class Graphed:
     def __init__(self, module: nn.Module, warmup: int = 2) -> None:
@@ -33,10 +37,21 @@ class Graphed:
         self._entries: Dict[tuple, tuple] = {}
 
     @staticmethod
-    def _key(s, z, pair_mask) -> tuple:
+    def _mask_class(z, pair_mask) -> tuple:
+        """The class of the mask that decides which kernels run (ops.mask_class): a recording
+        is made for one class and replayed for masks of that class only."""
+        if pair_mask is None or not pair_mask.is_cuda:
+            return (False, None)
+        n = z.shape[-2]
+        if pair_mask.numel() != n * n:
+            return (False, None)      # a batch of masks: the general kernels
+        return (False, ops.mask_class(pair_mask.view(n, n))[1])
+
+    @classmethod
+    def _key(cls, s, z, pair_mask) -> tuple:
         def sig(t):
             return None if t is None else (tuple(t.shape), t.dtype, t.device.index)
-        return (sig(s), sig(z), sig(pair_mask))
+        return (sig(s), sig(z), sig(pair_mask), cls._mask_class(z, pair_mask))
 
     def _capture(self, s, z, pair_mask) -> tuple:
         if not z.is_cuda:
@@ -56,8 +71,12 @@ class Graphed:
         torch.cuda.synchronize(z.device)
         z_io.copy_(z)
         graph = torch.cuda.CUDAGraph()
-        with torch.no_grad(), torch.cuda.graph(graph):
-            s_out, z_out = self.module(s_in, z_io, m_in, inplace_safe=True)
+        ops.capture_mask_class = self._mask_class(z, pair_mask)
+        try:
+            with torch.no_grad(), torch.cuda.graph(graph):
+                s_out, z_out = self.module(s_in, z_io, m_in, inplace_safe=True)
+        finally:
+            ops.capture_mask_class = None
         return graph, s_in, z_io, m_in, s_out, z_out
 
     def __call__(self, s: Optional[torch.Tensor], z: torch.Tensor,

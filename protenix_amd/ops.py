@@ -174,10 +174,59 @@ def _workspace(shape, dtype, device) -> torch.Tensor:
 _mask_cache: list = []
 
 
-def _mask_for(mask: Optional[torch.Tensor], z: torch.Tensor, dtype: Optional[torch.dtype] = None,
-              transpose: bool = False) -> Optional[torch.Tensor]:
+# Pair masks of padded batches are m (x) m with the padding at the end: the triangle attention
+# then runs its valid rows over the valid keys without a mask (see triangle_attention).  False
+# hands every mask to the kernels as it is (tests compare the two).
+prefix_mask_enabled = True
+
+
+def _mask_key(mask: torch.Tensor) -> tuple:
+    return (mask.untyped_storage().data_ptr(), mask.storage_offset(), tuple(mask.shape), tuple(mask.stride()),
+            mask.dtype, mask.device, mask._version)
+
+
+_class_cache: list = []     # (key, mask, (all ones, n_valid or None)), most recent first
+# While a HIP graph is being recorded nothing can be looked at: the class the recording is made
+# for, set by its owner (graph.py), who replays it only for masks of that class.
+capture_mask_class: Optional[tuple] = None
+
+
+def mask_class(mask: Optional[torch.Tensor]) -> tuple:
+    """(all ones, n_valid) of a 2-D pair mask on the GPU: n_valid is the number of valid tokens if
+    the mask is m (x) m with m = n_valid ones followed by zeros (0 < n_valid < n), else None.
+    Computed on the device, fetched with one synchronisation per mask (not per call) and kept
+    with the mask's storage, view geometry and version counter."""
     if mask is None:
-        return None
+        return (True, None)
+    if torch.cuda.is_current_stream_capturing():
+        return capture_mask_class or (False, None)
+    if not mask.is_cuda or mask.dim() != 2 or mask.shape[0] != mask.shape[1] or mask.shape[0] == 0:
+        return (bool((mask == 1).all()), None)
+    key = _mask_key(mask)
+    for i, (k, _, cls) in enumerate(_class_cache):
+        if k == key:
+            if i:
+                _class_cache.insert(0, _class_cache.pop(i))
+            return cls
+    row, col = mask[0, :], mask[:, 0]
+    nv = row.float().sum()
+    steps = (row[1:] > row[:-1]).any() if row.numel() > 1 else torch.zeros((), dtype=torch.bool, device=mask.device)
+    prefix = ((mask == col[:, None] * row[None, :]).all() & (row == col).all()
+              & ((row == 0) | (row == 1)).all() & ~steps)
+    ones, prefix, nv = torch.stack([(mask == 1).all().float(), prefix.float(), nv]).tolist()
+    cls = (bool(ones), int(nv) if prefix and 0 < int(nv) < mask.shape[0] else None)
+    _class_cache.insert(0, (key, mask, cls))
+    del _class_cache[8:]
+    return cls
+
+
+def _mask_for(mask: Optional[torch.Tensor], z: torch.Tensor, dtype: Optional[torch.dtype] = None,
+              transpose: bool = False, classify: bool = False):
+    """The mask in the kernels' dtype (None for a mask of all ones); with `classify`, also the
+    number of valid tokens n_valid if the mask is m (x) m with m = n_valid ones followed by
+    zeros (0 < n_valid < n), else None."""
+    if mask is None:
+        return (None, None) if classify else None
     dtype = dtype or z.dtype
 
     def convert() -> torch.Tensor:
@@ -185,25 +234,27 @@ def _mask_for(mask: Optional[torch.Tensor], z: torch.Tensor, dtype: Optional[tor
         return out.transpose(-1, -2).contiguous() if transpose else out.contiguous()
 
     # Under stream capture the conversion is part of what is recorded: a replay must convert the
-    # mask it is given then, so nothing is looked up, examined or kept.
+    # mask it is given then, so nothing is looked up, examined or kept (the class is the one the
+    # recording was announced for; a mask of all ones is then still loaded and applied, which
+    # changes no bit).
     if not z.is_cuda or torch.cuda.is_current_stream_capturing():
-        return convert()
-    key = (mask.untyped_storage().data_ptr(), mask.storage_offset(), tuple(mask.shape), tuple(mask.stride()),
-           mask.dtype, mask.device, mask._version, dtype, z.device, transpose)
+        n_valid = capture_mask_class[1] if (z.is_cuda and capture_mask_class) else None
+        return (convert(), n_valid) if classify else convert()
+    # A mask of all ones changes no bit of any result (x * 1, logit + 0): it is handed on as
+    # "no mask", which spares the kernels its loads.
+    ones, n_valid = mask_class(mask)
+    if ones:
+        return (None, None) if classify else None
+    key = _mask_key(mask) + (dtype, z.device, transpose)
     for i, (k, _, out) in enumerate(_mask_cache):
         if k == key:
             if i:
                 _mask_cache.insert(0, _mask_cache.pop(i))
-            return out
+            return (out, n_valid) if classify else out
     out = convert()
-    # A mask of all ones changes no bit of any result (x * 1, logit + 0): it is handed on as
-    # "no mask", which spares the kernels its loads.  Looking costs one synchronisation per
-    # mask (not per call).
-    if bool((out == 1).all()):
-        out = None
     _mask_cache.insert(0, (key, mask, out))
     del _mask_cache[8:]
-    return out
+    return (out, n_valid) if classify else out
 
 
 def triangle_multiplication(z: torch.Tensor, mask: Optional[torch.Tensor], w: dict, incoming: bool,
@@ -258,7 +309,9 @@ def triangle_attention(z: torch.Tensor, mask: Optional[torch.Tensor], w: dict, h
     dt, st = _dt_stream(z, cd), _stream()
     pitch = key_pitch(n)
     # (ending node: the key mask of logical row i is mask[:, i]; a transposed copy makes it a row)
-    mask = _mask_for(mask, z, cd, transpose=transposed)
+    mask, n_valid = _mask_for(mask, z, cd, transpose=transposed, classify=True)
+    if not prefix_mask_enabled:
+        n_valid = None
     dev = z.device
     # attention-core layouts (see include/protenix_amd.h): q, gate, output head-major; K, V^T
     # and the triangle bias in fragment-ordered key tiles
@@ -276,9 +329,18 @@ def triangle_attention(z: torch.Tensor, mask: Optional[torch.Tensor], w: dict, h
               _ptr(w["w_b"]), _ptr(q), _ptr(k), _ptr(vt), None if late_gate else _ptr(g), _ptr(tb),
               n, c, heads, d, pitch, int(transposed), eps, dt, st)
         # o overwrites g: each element of g is read once, by the thread that then writes o there
-        _call("triattn_fwd", lib.ptx_triattn_fwd, _ptr(q), _ptr(k), _ptr(vt),
-              None if late_gate else _ptr(g), _ptr(tb), _ptr(mask), _ptr(g), n, heads, d, pitch, 0,
-              float(inf), dt, st)
+        if mask is not None and n_valid is not None:
+            # mask = m (x) m, padding at the end: the valid rows attend the valid keys with no
+            # mask at all (a masked key of such a row has weight exactly zero in the reference);
+            # the padded rows, all of whose keys are masked, go through the masked path
+            for rows, mk, nk in (((0, n_valid), None, n_valid), ((n_valid, n - n_valid), mask, n)):
+                _call("triattn_fwd", lib.ptx_triattn_fwd_rows, _ptr(q), _ptr(k), _ptr(vt),
+                      None if late_gate else _ptr(g), _ptr(tb), _ptr(mk), _ptr(g), n, heads, d, pitch,
+                      0, float(inf), rows[0], rows[1], nk, dt, st)
+        else:
+            _call("triattn_fwd", lib.ptx_triattn_fwd, _ptr(q), _ptr(k), _ptr(vt),
+                  None if late_gate else _ptr(g), _ptr(tb), _ptr(mask), _ptr(g), n, heads, d, pitch, 0,
+                  float(inf), dt, st)
         del q, k, vt, tb
         if out is None:
             out = torch.empty_like(z)

@@ -69,5 +69,7 @@ def test_graphed_replays_convert_the_mask_they_are_given():
             s_ref, z_ref = st(s, z, m)
             s_got, z_got = fast(s, z, m)
         assert torch.equal(z_got, z_ref) and torch.equal(s_got, s_ref)
-    assert len(fast.shapes()) == 1
+    # one recording for the masks the general kernels take (all ones, random holes) and one for
+    # the padded tail of 9 tokens, whose valid rows run without a mask
+    assert len(fast.shapes()) == 2
 
