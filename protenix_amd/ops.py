@@ -176,8 +176,11 @@ _mask_cache: list = []
 
 # Pair masks of padded batches are m (x) m with the padding at the end: the triangle attention
 # then runs its valid rows over the valid keys without a mask (see triangle_attention).  False
-# hands every mask to the kernels as it is (tests compare the two).
+# hands every mask to the kernels as it is (tests compare the two).  Below some 600 tokens the
+# second launch costs what the first one saves (measured: 113 against 108 us at N = 256, 331
+# against 328 at 512, 750 against 775 at 768, 1.42 against 1.59 ms at 1024).
 prefix_mask_enabled = True
+prefix_mask_min_n = 600
 
 
 def _mask_key(mask: torch.Tensor) -> tuple:
@@ -220,13 +223,19 @@ def mask_class(mask: Optional[torch.Tensor]) -> tuple:
     return cls
 
 
+def padded_tail(mask: Optional[torch.Tensor], n: int) -> Optional[int]:
+    """n_valid if the triangle attention treats this [n, n] mask as a padded tail (two launches:
+    valid rows over valid keys without a mask, padded rows with it), else None."""
+    if mask is None or not prefix_mask_enabled or n < prefix_mask_min_n:
+        return None
+    return mask_class(mask)[1]
+
+
 def _mask_for(mask: Optional[torch.Tensor], z: torch.Tensor, dtype: Optional[torch.dtype] = None,
-              transpose: bool = False, classify: bool = False):
-    """The mask in the kernels' dtype (None for a mask of all ones); with `classify`, also the
-    number of valid tokens n_valid if the mask is m (x) m with m = n_valid ones followed by
-    zeros (0 < n_valid < n), else None."""
+              transpose: bool = False) -> Optional[torch.Tensor]:
+    """The mask in the kernels' dtype, or None for a mask of all ones."""
     if mask is None:
-        return (None, None) if classify else None
+        return None
     dtype = dtype or z.dtype
 
     def convert() -> torch.Tensor:
@@ -234,27 +243,24 @@ def _mask_for(mask: Optional[torch.Tensor], z: torch.Tensor, dtype: Optional[tor
         return out.transpose(-1, -2).contiguous() if transpose else out.contiguous()
 
     # Under stream capture the conversion is part of what is recorded: a replay must convert the
-    # mask it is given then, so nothing is looked up, examined or kept (the class is the one the
-    # recording was announced for; a mask of all ones is then still loaded and applied, which
-    # changes no bit).
+    # mask it is given then, so nothing is looked up, examined or kept (a mask of all ones is
+    # then still loaded and applied, which changes no bit).
     if not z.is_cuda or torch.cuda.is_current_stream_capturing():
-        n_valid = capture_mask_class[1] if (z.is_cuda and capture_mask_class) else None
-        return (convert(), n_valid) if classify else convert()
+        return convert()
     # A mask of all ones changes no bit of any result (x * 1, logit + 0): it is handed on as
     # "no mask", which spares the kernels its loads.
-    ones, n_valid = mask_class(mask)
-    if ones:
-        return (None, None) if classify else None
+    if mask_class(mask)[0]:
+        return None
     key = _mask_key(mask) + (dtype, z.device, transpose)
     for i, (k, _, out) in enumerate(_mask_cache):
         if k == key:
             if i:
                 _mask_cache.insert(0, _mask_cache.pop(i))
-            return (out, n_valid) if classify else out
+            return out
     out = convert()
     _mask_cache.insert(0, (key, mask, out))
     del _mask_cache[8:]
-    return (out, n_valid) if classify else out
+    return out
 
 
 def triangle_multiplication(z: torch.Tensor, mask: Optional[torch.Tensor], w: dict, incoming: bool,
@@ -309,9 +315,8 @@ def triangle_attention(z: torch.Tensor, mask: Optional[torch.Tensor], w: dict, h
     dt, st = _dt_stream(z, cd), _stream()
     pitch = key_pitch(n)
     # (ending node: the key mask of logical row i is mask[:, i]; a transposed copy makes it a row)
-    mask, n_valid = _mask_for(mask, z, cd, transpose=transposed, classify=True)
-    if not prefix_mask_enabled:
-        n_valid = None
+    n_valid = padded_tail(mask, n)
+    mask = _mask_for(mask, z, cd, transpose=transposed)
     dev = z.device
     # attention-core layouts (see include/protenix_amd.h): q, gate, output head-major; K, V^T
     # and the triangle bias in fragment-ordered key tiles

@@ -69,7 +69,31 @@ def test_graphed_replays_convert_the_mask_they_are_given():
             s_ref, z_ref = st(s, z, m)
             s_got, z_got = fast(s, z, m)
         assert torch.equal(z_got, z_ref) and torch.equal(s_got, s_ref)
-    # one recording for the masks the general kernels take (all ones, random holes) and one for
-    # the padded tail of 9 tokens, whose valid rows run without a mask
-    assert len(fast.shapes()) == 2
+    assert len(fast.shapes()) == 1
+
+
+def test_graphed_padded_tail_has_its_own_recording():
+    """Where the eager call runs a padded-tail mask as two attention launches, so does a recording
+    (same bits), and masks of another class get another recording."""
+    keep = P.ops.prefix_mask_min_n
+    P.ops.prefix_mask_min_n = 0
+    try:
+        st = _stack(BF16, n_blocks=2)
+        fast = P.Graphed(st)
+        n = 72
+        s, z, _ = O.make_inputs(n, seed=3, dtype=BF16)
+        s, z = s.cuda(), z.cuda()
+        masks = [O.make_inputs(n, n_pad=9)[2], torch.ones(1, n, n), O.make_inputs(n, n_pad=9)[2],
+                 O.make_inputs(n, n_pad=20)[2],
+                 (torch.rand(1, n, n, generator=torch.Generator().manual_seed(1)) > 0.3).float()]
+        for m in masks:
+            m = m.cuda()
+            with torch.no_grad():
+                s_ref, z_ref = st(s, z, m)
+                s_got, z_got = fast(s, z, m)
+            assert torch.equal(z_got, z_ref) and torch.equal(s_got, s_ref)
+        # 63 valid tokens, 52 valid tokens, everything else
+        assert len(fast.shapes()) == 3
+    finally:
+        P.ops.prefix_mask_min_n = keep
 

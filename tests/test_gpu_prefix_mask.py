@@ -14,6 +14,15 @@ from tests.util import oracle_and_product, pad_mask, rel_err, tol
 pytestmark = pytest.mark.gpu
 
 
+@pytest.fixture(autouse=True)
+def _every_size():
+    """The two-range path at every N (the host side takes it from some 600 tokens on)."""
+    keep = ops.prefix_mask_min_n
+    ops.prefix_mask_min_n = 0
+    yield
+    ops.prefix_mask_min_n = keep
+
+
 def _run(prod, z, mask, mixed, prefix):
     keep = ops.prefix_mask_enabled
     ops.prefix_mask_enabled = prefix
@@ -24,6 +33,19 @@ def _run(prod, z, mask, mixed, prefix):
     finally:
         ops.prefix_mask_enabled = keep
         ops._mask_cache.clear()
+
+
+def test_short_rows_keep_one_launch():
+    ops.prefix_mask_min_n = 600
+    _, prod = oracle_and_product(O.TriangleAttention, P.TriangleAttention, 128, 32, 4, dtype=torch.bfloat16)
+    z = torch.randn(1, 96, 96, 128).to(torch.bfloat16).cuda()
+    ops.kernel_timer = {}
+    try:
+        with torch.no_grad():
+            prod(z, pad_mask(96, 10).cuda())
+        assert len(ops.kernel_timer["triattn_fwd"]) == 1
+    finally:
+        ops.kernel_timer = None
 
 
 @pytest.mark.parametrize("mode", ["bf16", "mixed", "fp32"])
