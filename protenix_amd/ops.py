@@ -195,29 +195,30 @@ capture_mask_class: Optional[tuple] = None
 
 
 def mask_class(mask: Optional[torch.Tensor]) -> tuple:
-    """(all ones, n_valid) of a 2-D pair mask on the GPU: n_valid is the number of valid tokens if
-    the mask is m (x) m with m = n_valid ones followed by zeros (0 < n_valid < n), else None.
-    Computed on the device, fetched with one synchronisation per mask (not per call) and kept
-    with the mask's storage, view geometry and version counter."""
+    """(all ones, n_valid) of a pair mask: n_valid is the number of valid tokens if the mask is
+    [n, n] = m (x) m with m = n_valid ones followed by zeros (0 < n_valid < n), else None.
+    Computed where the mask lives, fetched with one synchronisation per mask (not per call) and
+    kept with the mask's storage, view geometry and version counter."""
     if mask is None:
         return (True, None)
-    if torch.cuda.is_current_stream_capturing():
+    if mask.is_cuda and torch.cuda.is_current_stream_capturing():
         return capture_mask_class or (False, None)
-    if not mask.is_cuda or mask.dim() != 2 or mask.shape[0] != mask.shape[1] or mask.shape[0] == 0:
-        return (bool((mask == 1).all()), None)
     key = _mask_key(mask)
     for i, (k, _, cls) in enumerate(_class_cache):
         if k == key:
             if i:
                 _class_cache.insert(0, _class_cache.pop(i))
             return cls
-    row, col = mask[0, :], mask[:, 0]
-    nv = row.float().sum()
-    steps = (row[1:] > row[:-1]).any() if row.numel() > 1 else torch.zeros((), dtype=torch.bool, device=mask.device)
-    prefix = ((mask == col[:, None] * row[None, :]).all() & (row == col).all()
-              & ((row == 0) | (row == 1)).all() & ~steps)
-    ones, prefix, nv = torch.stack([(mask == 1).all().float(), prefix.float(), nv]).tolist()
-    cls = (bool(ones), int(nv) if prefix and 0 < int(nv) < mask.shape[0] else None)
+    if mask.dim() != 2 or mask.shape[0] != mask.shape[1] or mask.shape[0] == 0:
+        cls = (bool((mask == 1).all()), None)
+    else:
+        row, col = mask[0, :], mask[:, 0]
+        nv = row.float().sum()
+        steps = (row[1:] > row[:-1]).any() if row.numel() > 1 else torch.zeros((), dtype=torch.bool, device=mask.device)
+        prefix = ((mask == col[:, None] * row[None, :]).all() & (row == col).all()
+                  & ((row == 0) | (row == 1)).all() & ~steps)
+        ones, prefix, nv = torch.stack([(mask == 1).all().float(), prefix.float(), nv]).tolist()
+        cls = (bool(ones), int(nv) if prefix and 0 < int(nv) < mask.shape[0] else None)
     _class_cache.insert(0, (key, mask, cls))
     del _class_cache[8:]
     return cls

@@ -150,3 +150,51 @@ def test_product_state_dict_is_the_reference_checkpoint_layout():
     sd = P.PairformerBlock(c_s=0).state_dict()
     assert not any(k.startswith(("attention_pair_bias", "single_transition")) for k in sd)
     assert len(sd) == len(_BLOCK_KEYS) - 16
+
+
+def test_mask_class_finds_a_padded_tail_and_nothing_else():
+    """ops.mask_class: (all ones, n_valid); n_valid only for m (x) m with the zeros of m at the
+    end (the reference's pair_mask of a padded batch, loss.py:589)."""
+    import torch
+    from protenix_amd import ops
+
+    def outer(v):
+        return v[:, None] * v[None, :]
+
+    v = torch.ones(8)
+    assert ops.mask_class(None) == (True, None)
+    assert ops.mask_class(outer(v)) == (True, None)
+    v[5:] = 0
+    tail = outer(v)
+    assert ops.mask_class(tail) == (False, 5)
+    assert ops.mask_class(tail.to(torch.bfloat16)) == (False, 5)
+    hole = torch.ones(8)
+    hole[2:4] = 0
+    assert ops.mask_class(outer(hole)) == (False, None)            # padding not at the end
+    head = torch.ones(8)
+    head[:3] = 0
+    assert ops.mask_class(outer(head)) == (False, None)            # padding at the front
+    spoilt = tail.clone()
+    spoilt[0, 7] = 1
+    assert ops.mask_class(spoilt) == (False, None)                 # not m (x) m
+    spoilt = tail.clone()
+    spoilt[6, 6] = 1
+    assert ops.mask_class(spoilt) == (False, None)
+    assert ops.mask_class(tail * 0.5) == (False, None)             # not 0 / 1
+    assert ops.mask_class(torch.zeros(4, 4)) == (False, None)      # no valid token
+    assert ops.mask_class(torch.ones(1, 4, 4)) == (True, None)     # batched: all-ones check only
+    # an entry follows the version counter of the tensor it was made for
+    m = outer(torch.ones(6))
+    assert ops.mask_class(m) == (True, None)
+    m[:, 4:] = 0
+    m[4:, :] = 0
+    assert ops.mask_class(m) == (False, 4)
+    # the attention takes the two-launch path from prefix_mask_min_n tokens on
+    assert ops.padded_tail(tail, 8) is None
+    keep = ops.prefix_mask_min_n
+    ops.prefix_mask_min_n = 0
+    try:
+        assert ops.padded_tail(tail, 8) == 5
+        assert ops.padded_tail(outer(hole), 8) is None
+    finally:
+        ops.prefix_mask_min_n = keep
