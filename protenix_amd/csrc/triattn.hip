@@ -332,7 +332,8 @@ __global__ __launch_bounds__((NWQ * 64), (sizeof(T) == 2 ? 16 / NWQ : 2)) void t
     out.alpha = alpha;
     return true;
   };
-  auto process_tile = [&](int tile, V8 (&tb)[2][2]) {
+  auto process_tile = [&](auto tail_tag, int tile, V8 (&tb)[2][2]) {
+    constexpr bool LAST_PARTIAL = decltype(tail_tag)::value;   // the one tile with keys beyond n_keys
     static_assert(R == 1, "the register budget of four waves per SIMD holds one row per wave");
     const int buf = tile % 3;
     const int key0 = tile * kKeyTile;
@@ -340,7 +341,10 @@ __global__ __launch_bounds__((NWQ * 64), (sizeof(T) == 2 ? 16 / NWQ : 2)) void t
     // are the lanes with bit 4 == u
     uint64_t mb_mask = 0ull;
     if constexpr (has_mask) mb_mask = __builtin_amdgcn_ballot_w64(lds_mb[buf][0][lane] != 0.0f);
-    const bool tail_tile = MK != kMaskNone && key0 + kKeyTile > nk;   // uniform
+    // keys of this tile that take part (uniform; 64 or more: all).  Half u holds the keys
+    // 16u .. 16u+15 and 32+16u .. 32+16u+15 of the tile: complete from 48 + 16u keys on, empty
+    // (and left out altogether) up to 16u.
+    const int tile_keys = LAST_PARTIAL ? nk - key0 : kKeyTile;
     // the unmasked paths of one half: optimistic against the reference the earlier tiles left,
     // classic if there is none yet or the optimistic one had to give up
     auto unmasked_half = [&](auto tail_tag, int u, HalfOut& out) -> bool {
@@ -358,6 +362,8 @@ __global__ __launch_bounds__((NWQ * 64), (sizeof(T) == 2 ? 16 / NWQ : 2)) void t
     for (int u = 0; u < 2; ++u) {
       HalfOut out;
       bool rescale = true;
+      const bool tail_tile = LAST_PARTIAL && tile_keys < 48 + 16 * u;
+      if (LAST_PARTIAL && tile_keys <= 16 * u) continue;
       // this half's keys are those of lanes with bit 4 == u
       if (has_mask && (mb_mask & (u ? 0xffff0000ffff0000ull : 0x0000ffff0000ffffull)) != 0ull) {
         if (tail_tile) half_row(std::integral_constant<int, kMasked>{}, std::true_type{}, buf, u, key0, tb[u], out);
@@ -381,9 +387,9 @@ __global__ __launch_bounds__((NWQ * 64), (sizeof(T) == 2 ? 16 / NWQ : 2)) void t
   // Tile t+2 travels global -> registers -> LDS while tile t is processed; the bias tile of
   // t+1 is requested into the bias registers once tile t has consumed them.
   V8 tbias[2][2];
-  auto step = [&](int tile) {
+  auto step = [&](auto tail_tag, int tile) {
     fetch(tile + 2);
-    process_tile(tile, tbias);
+    process_tile(tail_tag, tile, tbias);
     stash(tile + 2);
     __syncthreads();
   };
@@ -394,7 +400,13 @@ __global__ __launch_bounds__((NWQ * 64), (sizeof(T) == 2 ? 16 / NWQ : 2)) void t
   fetch(1);
   stash(1);
   __syncthreads();
-  for (int tile = 0; tile < n_tiles; ++tile) step(tile);
+  // the tiles whose keys all take part, in a loop that knows nothing of a partial tile (with
+  // its tests in the loop every tile was 7 % slower), then the partial one if there is one
+  const int n_full = MK == kMaskNone ? n_tiles : nk / kKeyTile;
+  for (int tile = 0; tile < n_full; ++tile) step(std::false_type{}, tile);
+  if constexpr (MK != kMaskNone) {
+    if (n_full < n_tiles) step(std::true_type{}, n_full);
+  }
 
   // ---- normalise, gate, store: lane <-> query, register e <-> d = acc_row(e, g) ----
   // o may alias gate: every gate load is issued before the first store.
