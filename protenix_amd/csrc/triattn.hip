@@ -264,8 +264,7 @@ __global__ __launch_bounds__((NWQ * 64), (sizeof(T) == 2 ? 16 / NWQ : 2)) void t
 #pragma unroll
         for (int t = 0; t < 8; ++t) {
           const float mbv = t < 4 ? m0[t & 3] : m1[t & 3];
-          const float v = (s[8 * c + t] * kLn2 + mbv) + b[t] * kLn2;
-          s[8 * c + t] = mbv == -INFINITY ? -INFINITY : v;
+          s[8 * c + t] = (s[8 * c + t] * kLn2 + mbv) + b[t] * kLn2;
         }
       }
     }
