@@ -296,9 +296,11 @@ __global__ __launch_bounds__((NWQ * 64), (sizeof(T) == 2 ? 16 / NWQ : 2)) void t
 #pragma unroll
       for (int e = 0; e < 16; ++e) s[e] = fast_exp2(s[e] + nml);
     } else {
+      // (no key with a finite logit yet: -inf minus a finite stand-in is -inf, weight 0, where
+      // -inf minus -inf would not be a number)
+      const float mref = fmaxf(m_run[0], -3.0e38f);
 #pragma unroll
-      for (int e = 0; e < 16; ++e)
-        s[e] = m_run[0] == -INFINITY ? 0.0f : fast_exp2((s[e] - m_run[0]) * kLog2e);
+      for (int e = 0; e < 16; ++e) s[e] = fast_exp2((s[e] - mref) * kLog2e);
     }
     float psum = 0.0f;
 #pragma unroll
