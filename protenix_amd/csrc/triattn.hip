@@ -162,7 +162,7 @@ __global__ __launch_bounds__((NWQ * 64), (sizeof(T) == 2 ? 16 / NWQ : 2)) void t
   auto stash = [&](int tile) {
     const int buf = tile % 3;
     const int key0 = tile * kKeyTile;
-    const bool tail = key0 + kKeyTile > nk;   // uniform
+    const bool tail = MK != kMaskNone && key0 + kKeyTile > nk;   // uniform (kMaskNone: whole tiles only)
 #pragma unroll
     for (int j = 0; j < FPW; ++j) {
       const int fid = wave * FPW + j;
