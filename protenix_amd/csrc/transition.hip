@@ -160,11 +160,22 @@ __global__ __launch_bounds__((TrCfg<T, KS>::NW * 64), 2) void transition_fused_k
         load_to_lds16_s<0>(fb, lane_off + 16 * pc, lds_address(&lds_w[buf][frag][pc][0]));
     }
   };
-  auto read_frag = [&](int buf, int frag) {
+  // A chunk buffer is read through this lane's LDS address of its first fragment, formed once
+  // per chunk and made opaque: the fragment number is then the immediate offset of the LDS read.
+  // (Left to itself the compiler keeps one address register per fragment and forms every
+  // address with two vector adds from a buffer offset it tracks in scalar registers: 44 adds
+  // per chunk next to the 104 instructions of the activation, and 25 registers.)
+  typedef __attribute__((address_space(3))) const u32x4_t* BufPtr;
+  auto buf_ptr = [&](int buf) -> BufPtr {
+    uint32_t a = (uint32_t)(uintptr_t)(BufPtr)&lds_w[buf][0][0][lane];
+    asm volatile("" : "+v"(a));
+    return (BufPtr)(uintptr_t)a;
+  };
+  auto read_frag = [&](BufPtr base, int frag) {
     V8 v;
     u32x4_t* d = reinterpret_cast<u32x4_t*>(&v);
 #pragma unroll
-    for (int pc = 0; pc < PIECES; ++pc) d[pc] = lds_w[buf][frag][pc][lane];
+    for (int pc = 0; pc < PIECES; ++pc) d[pc] = base[(frag * PIECES + pc) * kWave];
     return v;
   };
 
@@ -200,8 +211,8 @@ __global__ __launch_bounds__((TrCfg<T, KS>::NW * 64), 2) void transition_fused_k
   // the activation of the previous chunk (`prev`) between its MFMAs when ACT.  Fragments
   // are read from LDS one K step before they are used; the last step fetches the first
   // W_o fragment of the GEMM2 that follows (buffer `tail_buf`) and returns it.
-  auto gemm1 = [&](auto act_tag, int buf, f32x16 (&cur)[RB][2], f32x16 (&prev)[RB][2],
-                   int tail_buf) {
+  auto gemm1 = [&](auto act_tag, BufPtr buf, f32x16 (&cur)[RB][2], f32x16 (&prev)[RB][2],
+                   BufPtr tail_buf) {
     constexpr bool ACT = decltype(act_tag)::value;
     V8 wa = read_frag(buf, 0), wb = read_frag(buf, KS);
 #pragma unroll
@@ -230,7 +241,7 @@ __global__ __launch_bounds__((TrCfg<T, KS>::NW * 64), 2) void transition_fused_k
     return wa;
   };
   // GEMM2 of the chunk whose W_o fragments sit in buffer `buf`; `wo` is its first fragment.
-  auto gemm2 = [&](int buf, V8 wo) {
+  auto gemm2 = [&](BufPtr buf, V8 wo) {
 #pragma unroll
     for (int s2 = 0; s2 < 2 * NOB; ++s2) {
       const int u = s2 / NOB, ob = s2 % NOB;
@@ -248,15 +259,18 @@ __global__ __launch_bounds__((TrCfg<T, KS>::NW * 64), 2) void transition_fused_k
   auto iteration = [&](int j, f32x16 (&cur)[RB][2], f32x16 (&prev)[RB][2]) {
     ring_barrier<(D - 1) * G::DMA_PER_CHUNK>();
     dma_chunk(j + D);
-    const int pbuf = (j + NBUF - 1) % NBUF;
-    const V8 wo = gemm1(std::true_type{}, j % NBUF, cur, prev, pbuf);
+    const BufPtr cbuf = buf_ptr(j % NBUF), pbuf = buf_ptr((j + NBUF - 1) % NBUF);
+    const V8 wo = gemm1(std::true_type{}, cbuf, cur, prev, pbuf);
     gemm2(pbuf, wo);
   };
 
   // chunk 0: GEMM1 only
   ring_barrier<(D - 1) * G::DMA_PER_CHUNK>();
   dma_chunk(D);
-  gemm1(std::false_type{}, 0, ab0, ab1, 0);
+  {
+    const BufPtr b0 = buf_ptr(0);
+    gemm1(std::false_type{}, b0, ab0, ab1, b0);
+  }
   // chunks 1 .. n_chunks-1 (n_chunks is even): GEMM1(j), activation and GEMM2 of j-1
   int j = 1;
   for (; j + 1 < n_chunks; j += 2) {
@@ -292,7 +306,10 @@ __global__ __launch_bounds__((TrCfg<T, KS>::NW * 64), 2) void transition_fused_k
   // drain: activation and GEMM2 of the last chunk
 #pragma unroll
   for (int kk = 0; kk < KS; ++kk) act_part(kk, ab1);
-  gemm2((n_chunks - 1) % NBUF, read_frag((n_chunks - 1) % NBUF, 2 * KS));
+  {
+    const BufPtr lbuf = buf_ptr((n_chunks - 1) % NBUF);
+    gemm2(lbuf, read_frag(lbuf, 2 * KS));
+  }
 
   // ---- epilogue: out rows through the per-wave staging tile (reuses the chunk buffers once
   // every wave is past its last fragment read and all loads have landed) ----
