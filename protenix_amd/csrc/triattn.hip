@@ -57,8 +57,10 @@ struct AttnAux {
   int n_keys;             // keys 0 .. n_keys-1 take part (n_keys <= n; the rest count as masked)
 };
 
-// Rows of the pair tensor handled by one wave: one (more would share the bias tile, but do not
-// fit the register budget).
+// Rows of the pair tensor handled by one wave: one.  Two share the bias tile (half the bias
+// stream from the L2, one conversion per logit for both) at 131 registers, which leaves three
+// waves per SIMD instead of four: 416 - 420 us per launch at N = 768 against 412 (the kernel
+// below takes any R; R = 2 was measured with the same code).
 #define PTX_ATTN_ROWS 1
 
 // NWQ waves per workgroup (4 or 8), each with 32 queries: the workgroup's waves share the staged
@@ -74,7 +76,7 @@ struct AttnAux {
 // n_keys set to -inf (kMaskTail; kMaskNone where the keys fill whole tiles).
 enum { kMaskNone = 0, kMaskTail = 1, kMaskGiven = 2 };
 template <typename T, int R, int NWQ, int MK>
-__global__ __launch_bounds__((NWQ * 64), (sizeof(T) == 2 ? 16 / NWQ : 2)) void triattn_fwd_kernel(
+__global__ __launch_bounds__((NWQ * 64), (sizeof(T) == 2 ? (R == 1 ? 16 : 12) / NWQ : 2)) void triattn_fwd_kernel(
     const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ vt,
     const T* gate, const T* __restrict__ bias, const T* __restrict__ mask,
     T* o, int n, int heads, int key_pitch, int mask_transposed, float inf,
@@ -234,33 +236,34 @@ __global__ __launch_bounds__((NWQ * 64), (sizeof(T) == 2 ? 16 / NWQ : 2)) void t
   // mask values found there, are replaced by -inf before the softmax (weight zero).  The other
   // keys of such a tile take the same path as in any other tile, so a mask of all ones gives
   // the bits that no mask gives.
-  auto half_row = [&](auto mode_tag, auto tail_tag, int buf, int u, int key0, V8 (&tbh)[2],
-                      HalfOut& out) -> bool {
+  // `r`: which of the wave's R rows; `tbf`: the half's bias tile in fp32 (converted once per
+  // half, for all R rows: they share the query block and with it the bias).
+  auto half_row = [&](auto mode_tag, auto tail_tag, int r, int buf, int u, int key0, V8 (&tbh)[2],
+                      const f32x16& tbf, HalfOut& out) -> bool {
     constexpr int MODE = decltype(mode_tag)::value;
     constexpr bool MASKED = MODE == kMasked;
     constexpr bool TAIL = decltype(tail_tag)::value;
     V8 kf[2];
 #pragma unroll
-    for (int kk = 0; kk < 2; ++kk) kf[kk] = lds_kv[buf][0][u * 2 + kk][lane];
+    for (int kk = 0; kk < 2; ++kk) kf[kk] = lds_kv[buf][r][u * 2 + kk][lane];
     f32x16 s;
     if constexpr (!MASKED) {
       // S^T starts from the bias, the C operand of the first product: register e of this lane
       // <-> element e of its 16 stored values (16-bit: one conversion per logit, which with
       // four waves per SIMD costs less than adding the bias on the matrix pipe)
-      const f32x8 b0 = to_f32(tbh[0]), b1 = to_f32(tbh[1]);
-      s = __builtin_shufflevector(b0, b1, 0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15);
+      s = tbf;
     } else {
 #pragma unroll
       for (int e = 0; e < 16; ++e) s[e] = 0.0f;
     }
 #pragma unroll
-    for (int kk = 0; kk < 2; ++kk) mma32(s, kf[kk], qf[0][kk]);
+    for (int kk = 0; kk < 2; ++kk) mma32(s, kf[kk], qf[r][kk]);
     if constexpr (MASKED) {
 #pragma unroll
       for (int c = 0; c < 2; ++c) {
         const f32x8 b = to_f32(tbh[c]);
-        const f32x4 m0 = *reinterpret_cast<const f32x4*>(&lds_mb[buf][0][32 * g + 16 * u + 8 * c]);
-        const f32x4 m1 = *reinterpret_cast<const f32x4*>(&lds_mb[buf][0][32 * g + 16 * u + 8 * c + 4]);
+        const f32x4 m0 = *reinterpret_cast<const f32x4*>(&lds_mb[buf][r][32 * g + 16 * u + 8 * c]);
+        const f32x4 m1 = *reinterpret_cast<const f32x4*>(&lds_mb[buf][r][32 * g + 16 * u + 8 * c + 4]);
 #pragma unroll
         for (int t = 0; t < 8; ++t) {
           const float mbv = t < 4 ? m0[t & 3] : m1[t & 3];
@@ -283,22 +286,22 @@ __global__ __launch_bounds__((NWQ * 64), (sizeof(T) == 2 ? 16 / NWQ : 2)) void t
       mt = fmaxf(mt, swap32(mt));
       if (!MASKED) mt *= kLn2;
       // (a half whose keys all lie beyond n has mt = -inf: the reference stays where it is)
-      float m_new = fmaxf(m_run[0], mt);
+      float m_new = fmaxf(m_run[r], mt);
       if (!MASKED && (__builtin_amdgcn_ballot_w64(!(fabsf(m_new) < kZeroReferenceLimit)) & q_ok_mask) == 0ull) m_new = 0.0f;
-      alpha = m_new == -INFINITY ? 1.0f : fast_exp2((m_run[0] - m_new) * kLog2e);
-      m_run[0] = m_new;
+      alpha = m_new == -INFINITY ? 1.0f : fast_exp2((m_run[r] - m_new) * kLog2e);
+      m_run[r] = m_new;
     }
     if constexpr (MODE == kOptimisticZero) {
 #pragma unroll
       for (int e = 0; e < 16; ++e) s[e] = fast_exp2(s[e]);
     } else if constexpr (!MASKED) {
-      const float nml = -m_run[0] * kLog2e;
+      const float nml = -m_run[r] * kLog2e;
 #pragma unroll
       for (int e = 0; e < 16; ++e) s[e] = fast_exp2(s[e] + nml);
     } else {
       // (no key with a finite logit yet: -inf minus a finite stand-in is -inf, weight 0, where
       // -inf minus -inf would not be a number)
-      const float mref = fmaxf(m_run[0], -3.0e38f);
+      const float mref = fmaxf(m_run[r], -3.0e38f);
 #pragma unroll
       for (int e = 0; e < 16; ++e) s[e] = fast_exp2((s[e] - mref) * kLog2e);
     }
@@ -335,53 +338,61 @@ __global__ __launch_bounds__((NWQ * 64), (sizeof(T) == 2 ? 16 / NWQ : 2)) void t
   };
   auto process_tile = [&](auto tail_tag, int tile, V8 (&tb)[2][2]) {
     constexpr bool LAST_PARTIAL = decltype(tail_tag)::value;   // the one tile with keys beyond n_keys
-    static_assert(R == 1, "the register budget of four waves per SIMD holds one row per wave");
     const int buf = tile % 3;
     const int key0 = tile * kKeyTile;
-    // keys of the tile with a non-zero mask bias, as a lane mask (key <-> lane); half u's keys
-    // are the lanes with bit 4 == u
-    uint64_t mb_mask = 0ull;
-    if constexpr (has_mask) mb_mask = __builtin_amdgcn_ballot_w64(lds_mb[buf][0][lane] != 0.0f);
+    // keys of the tile with a non-zero mask bias, per row, as a lane mask (key <-> lane); half
+    // u's keys are the lanes with bit 4 == u
+    uint64_t mb_mask[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      mb_mask[r] = 0ull;
+      if constexpr (has_mask) mb_mask[r] = __builtin_amdgcn_ballot_w64(lds_mb[buf][r][lane] != 0.0f);
+    }
     // keys of this tile that take part (uniform; 64 or more: all).  Half u holds the keys
     // 16u .. 16u+15 and 32+16u .. 32+16u+15 of the tile: complete from 48 + 16u keys on, empty
     // (and left out altogether) up to 16u.
     const int tile_keys = LAST_PARTIAL ? nk - key0 : kKeyTile;
-    // the unmasked paths of one half: optimistic against the reference the earlier tiles left,
-    // classic if there is none yet or the optimistic one had to give up
-    auto unmasked_half = [&](auto tail_tag, int u, HalfOut& out) -> bool {
-      bool done = false;
-      if (tile != 0 || u != 0) {
-        if ((__builtin_amdgcn_ballot_w64(m_run[0] != 0.0f) & q_ok_mask) == 0ull)
-          done = half_row(std::integral_constant<int, kOptimisticZero>{}, tail_tag, buf, u, key0, tb[u], out);
-        else
-          done = half_row(std::integral_constant<int, kOptimistic>{}, tail_tag, buf, u, key0, tb[u], out);
-      }
-      if (!done) half_row(std::integral_constant<int, kClassic>{}, tail_tag, buf, u, key0, tb[u], out);
-      return !done;   // classic: O and l are rescaled first
-    };
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
-      HalfOut out;
-      bool rescale = true;
       const bool tail_tile = LAST_PARTIAL && tile_keys < 48 + 16 * u;
       if (LAST_PARTIAL && tile_keys <= 16 * u) continue;
-      // this half's keys are those of lanes with bit 4 == u
-      if (has_mask && (mb_mask & (u ? 0xffff0000ffff0000ull : 0x0000ffff0000ffffull)) != 0ull) {
-        if (tail_tile) half_row(std::integral_constant<int, kMasked>{}, std::true_type{}, buf, u, key0, tb[u], out);
-        else half_row(std::integral_constant<int, kMasked>{}, std::false_type{}, buf, u, key0, tb[u], out);
-      } else if (tail_tile) {
-        rescale = unmasked_half(std::true_type{}, u, out);
-      } else {
-        rescale = unmasked_half(std::false_type{}, u, out);
-      }
-      if (rescale) {
+      const f32x8 b0 = to_f32(tb[u][0]), b1 = to_f32(tb[u][1]);
+      const f32x16 tbf = __builtin_shufflevector(b0, b1, 0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15);
 #pragma unroll
-        for (int e = 0; e < 16; ++e) acc_o[0][e] *= out.alpha;
-        l_run[0] *= out.alpha;
-      }
-      l_run[0] += out.psum;
+      for (int r = 0; r < R; ++r) {
+        // the unmasked paths of one half: optimistic against the reference the earlier tiles
+        // left, classic if there is none yet or the optimistic one had to give up
+        auto unmasked_half = [&](auto ttag, HalfOut& out) -> bool {
+          bool done = false;
+          if (tile != 0 || u != 0) {
+            if ((__builtin_amdgcn_ballot_w64(m_run[r] != 0.0f) & q_ok_mask) == 0ull)
+              done = half_row(std::integral_constant<int, kOptimisticZero>{}, ttag, r, buf, u, key0, tb[u], tbf, out);
+            else
+              done = half_row(std::integral_constant<int, kOptimistic>{}, ttag, r, buf, u, key0, tb[u], tbf, out);
+          }
+          if (!done) half_row(std::integral_constant<int, kClassic>{}, ttag, r, buf, u, key0, tb[u], tbf, out);
+          return !done;   // classic: O and l are rescaled first
+        };
+        HalfOut out;
+        bool rescale = true;
+        // this half's keys are those of lanes with bit 4 == u
+        if (has_mask && (mb_mask[r] & (u ? 0xffff0000ffff0000ull : 0x0000ffff0000ffffull)) != 0ull) {
+          if (tail_tile) half_row(std::integral_constant<int, kMasked>{}, std::true_type{}, r, buf, u, key0, tb[u], tbf, out);
+          else half_row(std::integral_constant<int, kMasked>{}, std::false_type{}, r, buf, u, key0, tb[u], tbf, out);
+        } else if (tail_tile) {
+          rescale = unmasked_half(std::true_type{}, out);
+        } else {
+          rescale = unmasked_half(std::false_type{}, out);
+        }
+        if (rescale) {
 #pragma unroll
-      for (int c = 0; c < 2; ++c) mma32(acc_o[0], lds_kv[buf][0][4 + u * 2 + c][lane], out.pf[c]);
+          for (int e = 0; e < 16; ++e) acc_o[r][e] *= out.alpha;
+          l_run[r] *= out.alpha;
+        }
+        l_run[r] += out.psum;
+#pragma unroll
+        for (int c = 0; c < 2; ++c) mma32(acc_o[r], lds_kv[buf][r][4 + u * 2 + c][lane], out.pf[c]);
+      }
     }
     fetch_bias(tile + 1, tb);
   };
