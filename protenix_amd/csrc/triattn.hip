@@ -53,15 +53,11 @@ struct AttnAux {
   int mask_is_bias;
   float* lse;             // or null
   int64_t lh, li, lj;     // element strides of lse: head, row, query
-  int row0;               // first row of this launch (a launch may cover a range of the rows)
+  int row0, row_end;      // rows row0 .. row_end-1 are this launch's (a launch may cover a range)
   int n_keys;             // keys 0 .. n_keys-1 take part (n_keys <= n; the rest count as masked)
 };
 
-// Rows of the pair tensor handled by one wave: one.  Two share the bias tile (half the bias
-// stream from the L2, one conversion per logit for both) at 131 registers, which leaves three
-// waves per SIMD instead of four: 416 - 420 us per launch at N = 768 against 412 (the kernel
-// below takes any R; R = 2 was measured with the same code).
-#define PTX_ATTN_ROWS 1
+// Rows of the pair tensor handled by one wave: R = 1 or 2, chosen per launch (triattn_fwd_ex).
 
 // NWQ waves per workgroup (4 or 8), each with 32 queries: the workgroup's waves share the staged
 // K / V^T tiles, so with 8 every wave moves one fragment per tile instead of two.
@@ -76,7 +72,7 @@ struct AttnAux {
 // n_keys set to -inf (kMaskTail; kMaskNone where the keys fill whole tiles).
 enum { kMaskNone = 0, kMaskTail = 1, kMaskGiven = 2 };
 template <typename T, int R, int NWQ, int MK>
-__global__ __launch_bounds__((NWQ * 64), (sizeof(T) == 2 ? (R == 1 ? 16 : 12) / NWQ : 2)) void triattn_fwd_kernel(
+__global__ __launch_bounds__((NWQ * 64), (sizeof(T) == 2 ? (R == 1 ? 16 / NWQ : (NWQ == 8 ? 2 : 3)) : 2)) void triattn_fwd_kernel(
     const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ vt,
     const T* gate, const T* __restrict__ bias, const T* __restrict__ mask,
     T* o, int n, int heads, int key_pitch, int mask_transposed, float inf,
@@ -440,10 +436,10 @@ __global__ __launch_bounds__((NWQ * 64), (sizeof(T) == 2 ? (R == 1 ? 16 : 12) / 
   for (int r = 0; r < R; ++r) {
     const float l_tot = l_run[r] + swap32(l_run[r]);
     const float inv = fast_rcp(l_tot);
-    if (ax.lse && g == 0 && q0 + ln < n && i0 + r < n_rows)
+    if (ax.lse && g == 0 && q0 + ln < n && i0 + r < ax.row_end)
       ax.lse[h * ax.lh + (int64_t)(i0 + r) * ax.li + (int64_t)qi_again * ax.lj] =
           m_run[r] * kLog2e + __builtin_amdgcn_logf(l_tot);   // v_log_f32 is log2
-    if (q0 + ln < n && i0 + r < n_rows) {
+    if (q0 + ln < n && i0 + r < ax.row_end) {
 #pragma unroll
       for (int c = 0; c < 4; ++c) {
         f32x4 ov;
@@ -479,21 +475,38 @@ int triattn_fwd_ex(const T* q, const T* k, const T* vt, const T* g, const T* tri
                    int64_t sj, float* lse, int64_t lh, int64_t li, int64_t lj, int row_begin,
                    int row_count, int n_keys, hipStream_t stream) {
   if (n == 0 || n_rows == 0 || row_count == 0) return 0;
-  AttnAux ax = {sh, si, sj, n_rows, mask_is_bias, lse, lh, li, lj, row_begin, n_keys};
-  constexpr int R = PTX_ATTN_ROWS;
+  AttnAux ax = {sh, si, sj, n_rows, mask_is_bias, lse, lh, li, lj, row_begin, row_begin + row_count, n_keys};
   // 8-wave workgroups for long rows (measured: +2 % at n = 768, even at 1024, -2.6 % at 1536,
   // -2.2 % at 2048), where their 256 queries divide n or n is large enough for the idle waves
   // of the last one not to matter
   const bool wide = sizeof(T) == 2 && ((n % 256 == 0 && n >= 1536) || n >= 2048);
-  const int n_qtiles = wide ? (n + 255) / 256 : (n + 127) / 128;
+  // Two rows per wave, in 8-wave workgroups (16-bit, whole key tiles, no mask): the two rows
+  // share the query block and with it the bias tile - one load and one conversion per logit for
+  // both, half the bias stream from the L2 - at 123 registers, so that four waves still share a
+  // SIMD (with a mask or a partial tile the kernel needs 131 to 160 and loses a wave; with four
+  // waves per workgroup the K / V tiles of two rows leave room for three workgroups only: no
+  // gain).  Per launch: 395 -> 356 us at n = 768 in the trunk; in a loop of attention updates
+  // -7 % at n = 512, -3 % at 768, -11 % at 1536, -13 % at 2048, but +10 to +25 % where 256
+  // queries do not divide n (256, 384, 640) and waves of the last workgroup idle.
+  const bool r2 = sizeof(T) == 2 && !mask && n_keys % kKeyTile == 0 && n % 256 == 0 && n >= 512 &&
+                  row_count >= 2;
+  const int n_qtiles = (wide || r2) ? (n + 255) / 256 : (n + 127) / 128;
+  const int R = r2 ? 2 : 1;
   const int n_rowgroups = (row_count + R - 1) / R;
   const int64_t total = (int64_t)heads * n_rowgroups * n_qtiles;
   const int64_t per_xcd = (total + 7) / 8;
-#define PTX_ATTN_LAUNCH(NWQ, MK)                                                                  \
-  triattn_fwd_kernel<T, R, NWQ, MK><<<dim3((unsigned)(per_xcd * 8)), dim3(NWQ * 64), 0, stream>>>( \
+  const int mk = mask ? kMaskGiven : n_keys % kKeyTile ? kMaskTail : kMaskNone;
+#define PTX_ATTN_LAUNCH_R(RR, NWQ, MK)                                                            \
+  triattn_fwd_kernel<T, RR, NWQ, MK><<<dim3((unsigned)(per_xcd * 8)), dim3(NWQ * 64), 0, stream>>>( \
       q, k, vt, g, tri_bias, mask, o, n, heads, key_pitch, mask_transposed, inf, n_qtiles,        \
       n_rowgroups, total, ax)
-  const int mk = mask ? kMaskGiven : n_keys % kKeyTile ? kMaskTail : kMaskNone;
+#define PTX_ATTN_LAUNCH(NWQ, MK) PTX_ATTN_LAUNCH_R(1, NWQ, MK)
+  if (r2) {
+    if constexpr (sizeof(T) == 2) {
+      PTX_ATTN_LAUNCH_R(2, 8, kMaskNone);
+    }
+    return 0;
+  }
   if (wide) {
     if (mk == kMaskGiven) PTX_ATTN_LAUNCH(8, kMaskGiven);
     else if (mk == kMaskTail) PTX_ATTN_LAUNCH(8, kMaskTail);
@@ -504,6 +517,7 @@ int triattn_fwd_ex(const T* q, const T* k, const T* vt, const T* g, const T* tri
     else PTX_ATTN_LAUNCH(4, kMaskNone);
   }
 #undef PTX_ATTN_LAUNCH
+#undef PTX_ATTN_LAUNCH_R
   return 0;
 }
 

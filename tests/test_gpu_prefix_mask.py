@@ -152,3 +152,41 @@ def test_rows_entry_refusals():
     assert lib.ptx_triattn_fwd_rows(*args, 64, 4, 32, 64, 0, 1e9, 0, 64, 0, 1, None) == 1
     # an empty range is no work
     assert lib.ptx_triattn_fwd_rows(*args, 64, 4, 32, 64, 0, 1e9, 10, 0, 64, 1, None) == 0
+
+
+@pytest.mark.parametrize("n", [512, 130])
+@pytest.mark.parametrize("rows", [(0, 512), (3, 5), (7, 1), (100, 33), (509, 3)])
+def test_rows_entry_writes_its_rows_only(n, rows):
+    """ptx_triattn_fwd_rows on a range of rows (odd counts, odd starts: at n = 512 the core takes
+    two rows per wave) gives those rows of ptx_triattn_fwd's result bit for bit and leaves every
+    other row of o alone."""
+    r0, cnt = rows
+    r0, cnt = min(r0, n - 1), min(cnt, n - min(r0, n - 1))
+    lib = P._lib.load()
+    bf = torch.bfloat16
+    g = torch.Generator().manual_seed(n)
+    z = torch.randn(n, n, 128, generator=g).to(bf).cuda()
+
+    def w(*s):
+        return (torch.randn(*s, generator=g) / s[-1] ** 0.5).to(bf).cuda()
+
+    ln_w, ln_b = torch.ones(128, dtype=bf).cuda(), torch.zeros(128, dtype=bf).cuda()
+    wq, wk, wv, wg, wb = w(128, 128), w(128, 128), w(128, 128), w(128, 128), w(4, 128)
+    pitch = lib.ptx_key_pitch(n)
+    q = torch.empty(4, n, n, 32, dtype=bf, device="cuda")
+    gate = torch.empty_like(q)
+    k = torch.empty(lib.ptx_triattn_kv_elems(n, 4), dtype=bf, device="cuda")
+    vt = torch.empty_like(k)
+    tb = torch.empty(lib.ptx_triattn_bias_elems(n, 4), dtype=bf, device="cuda")
+    st = torch.cuda.current_stream().cuda_stream
+    p = lambda t: t.data_ptr()
+    assert lib.ptx_triattn_project(p(z), p(ln_w), p(ln_b), p(wq), p(wk), p(wv), p(wg), p(wb), p(q), p(k), p(vt),
+                                   p(gate), p(tb), n, 128, 4, 32, pitch, 0, 1e-5, 1, st) == 0
+    full = torch.empty_like(q)
+    assert lib.ptx_triattn_fwd(p(q), p(k), p(vt), p(gate), p(tb), None, p(full), n, 4, 32, pitch, 0, 1e9, 1, st) == 0
+    part = torch.full_like(q, 7.0)
+    assert lib.ptx_triattn_fwd_rows(p(q), p(k), p(vt), p(gate), p(tb), None, p(part), n, 4, 32, pitch, 0, 1e9,
+                                    r0, cnt, n, 1, st) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(part[:, r0:r0 + cnt], full[:, r0:r0 + cnt])
+    assert (part[:, :r0] == 7.0).all() and (part[:, r0 + cnt:] == 7.0).all()
