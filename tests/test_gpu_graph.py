@@ -55,7 +55,7 @@ def test_graphed_block_without_single_track():
 
 def test_graphed_replays_convert_the_mask_they_are_given():
     """The pair mask's converted copy is kept between eager calls; a graph must not bake in the
-    copy (or the "all ones: no mask" verdict) of the mask it was captured with."""
+    copy (or the "all ones: no mask" decision) of the mask it was captured with."""
     st = _stack(BF16, n_blocks=2)
     fast = P.Graphed(st)
     n = 72
