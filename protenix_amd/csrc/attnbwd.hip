@@ -16,6 +16,7 @@
 // registers, parks it in LDS row-major and (for the operands a product needs with the walking
 // index in the K slots: K^T for dQ, Q^T and dO^T for dK / dV) transposed, and every wave reads
 // its MFMA fragments from there.
+#include <type_traits>
 #include "common.h"
 #include "kernels.h"
 
@@ -70,6 +71,14 @@ __device__ __forceinline__ f32x8 load_bias8(const T* row, int kb, int s, bool ve
 
 }  // namespace
 
+// 16-bit kernels double-buffer their shared tiles (one barrier a step) and are held to three
+// workgroups per compute unit where rows are 8-aligned; fp32 tiles are twice as large and stay
+// single-buffered (two barriers a step).
+template <typename T, bool VEC> struct BwdCfg {
+  static constexpr int kBuffers = sizeof(T) == 2 ? 2 : 1;
+  static constexpr int kMinBlocks = sizeof(T) == 2 ? (VEC ? 3 : 2) : 1;
+};
+
 // Delta[i][j][h] = sum_d O * dO
 template <typename T>
 __global__ __launch_bounds__(256) void attn_bwd_delta_kernel(BwdParams p) {
@@ -111,12 +120,17 @@ template <typename T> struct TilePiece {
 // dQ: a workgroup takes 128 queries of one (row, head), a wave 32 of them, and walks over the
 // key blocks; K, V and K^T are shared.  Works on S^T: lane <-> query, register <-> key, so the
 // biases arrive as 8 consecutive keys per load and the row statistics are per-lane scalars.
+// The biases are the initial value of the S^T accumulator and -Delta that of dP^T, so that a
+// logit costs one multiply-add, one exponential and one multiply.  Lanes whose query lies
+// beyond s repeat query s - 1 and store nothing; keys beyond s exist in the last block only,
+// which has its own copy of the step.  The shared tiles are double-buffered: one barrier a step.
 template <typename T, bool VEC>
-__global__ __launch_bounds__(256) void attn_bwd_dq_kernel(BwdParams p) {
+__global__ __launch_bounds__(256, (BwdCfg<T, VEC>::kMinBlocks)) void attn_bwd_dq_kernel(BwdParams p) {
   typedef typename Vec8<T>::type V8;
   typedef typename Vec4<T>::type V4;
-  __shared__ __attribute__((aligned(32))) T rm[2][32 * kTP];   // K, V
-  __shared__ __attribute__((aligned(32))) T tr[1][32 * kTP];   // K^T
+  constexpr int NB = BwdCfg<T, VEC>::kBuffers;
+  __shared__ __attribute__((aligned(32))) T rm[NB][2][32 * kTP];   // K, V
+  __shared__ __attribute__((aligned(32))) T tr[NB][1][32 * kTP];   // K^T
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, ln = lane & 31, g = lane >> 5;
   const int s = p.s, H = p.heads;
   constexpr bool vec = VEC;   // rows of s keys are 8-aligned
@@ -125,7 +139,10 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_kernel(BwdParams p) {
   const int qi = min(q0 + ln, s - 1);
   const bool q_ok = q0 + ln < s;
   const T* b2row = (const T*)p.b2 + ((int64_t)h * s + qi) * s;
-  const T* b1row = p.b1 ? (const T*)p.b1 + (int64_t)i * s : nullptr;
+  // (without a Bias1 the loads go to Bias2's row and count for nothing: a load under a branch
+  // would make every wait for memory a wait for all of it)
+  const T* b1row = p.b1 ? (const T*)p.b1 + (int64_t)i * s : b2row;
+  const float b1on = p.b1 ? 1.0f : 0.0f;
 
   V8 qf[2], dof[2];
 #pragma unroll
@@ -133,48 +150,54 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_kernel(BwdParams p) {
     qf[kk] = load8<T>((const T*)p.q + elem(p, i, qi, h) + 16 * kk + 8 * g);
     dof[kk] = load8<T>((const T*)p.dout + elem(p, i, qi, h) + 16 * kk + 8 * g);
   }
-  const float mq = p.lse[((int64_t)i * s + qi) * H + h];
-  const float dq_ = p.delta[((int64_t)i * s + qi) * H + h];
+  const float neg_mq = -p.lse[((int64_t)i * s + qi) * H + h];
+  const float neg_dq = -p.delta[((int64_t)i * s + qi) * H + h];
   f32x16 acc;
 #pragma unroll
   for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
 
   TilePiece<T> piece;
   V8 b1n[2], b2n[2];
+  // (the compiler barriers keep the loads where they are written, a step ahead of their use:
+  // left alone, the compiler moves them down to the use and waits there)
   auto fetch = [&](int key0) {
     piece.fetch(p, p.k, p.v, i, key0, h, tid);
+    asm volatile("" ::: "memory");
+  };
+  auto fetch_bias = [&](int key0) {
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks) {
       b2n[ks] = load_bias8_raw<T>(b2row, key0 + 16 * ks + 8 * g, s, vec);
-      b1n[ks] = b1row ? load_bias8_raw<T>(b1row, key0 + 16 * ks + 8 * g, s, vec) : zero_frag<T>();
+      b1n[ks] = load_bias8_raw<T>(b1row, key0 + 16 * ks + 8 * g, s, vec);
     }
+    asm volatile("" ::: "memory");
   };
-  fetch(0);
-  for (int key0 = 0; key0 < s; key0 += 32) {
-    piece.park(rm, tr, 1, tid);
-    f32x8 b1f[2], b2f[2];
-#pragma unroll
-    for (int ks = 0; ks < 2; ++ks) {
-      b1f[ks] = to_f32(b1n[ks]);
-      b2f[ks] = to_f32(b2n[ks]);
-    }
-    __syncthreads();
-    if (key0 + 32 < s) fetch(key0 + 32);   // in flight while this step computes
-
+  // one block of 32 keys out of buffer `buf`; TAIL: the block holds keys beyond s.  The biases
+  // of the next block are requested as soon as this block's sit in the accumulator.
+  auto step = [&](auto tail_tag, int buf, int key0, int next_key0) {
+    constexpr bool TAIL = decltype(tail_tag)::value;
     V8 kf[2], vf[2], ktf[2];
 #pragma unroll
     for (int kk = 0; kk < 2; ++kk) {
-      kf[kk] = load8<T>(&rm[0][perm_row(ln) * kTP + 16 * kk + 8 * g]);
-      vf[kk] = load8<T>(&rm[1][perm_row(ln) * kTP + 16 * kk + 8 * g]);
-      ktf[kk] = load8<T>(&tr[0][ln * kTP + 16 * kk + 8 * g]);
+      kf[kk] = load8<T>(&rm[buf][0][perm_row(ln) * kTP + 16 * kk + 8 * g]);
+      vf[kk] = load8<T>(&rm[buf][1][perm_row(ln) * kTP + 16 * kk + 8 * g]);
+      ktf[kk] = load8<T>(&tr[buf][0][ln * kTP + 16 * kk + 8 * g]);
     }
     f32x16 st, dp;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) st[r] = dp[r] = 0.0f;
+    for (int ks = 0; ks < 2; ++ks) {
+      const f32x8 b1f = to_f32(b1n[ks]), b2f = to_f32(b2n[ks]);
+#pragma unroll
+      for (int t = 0; t < 8; ++t) {
+        st[8 * ks + t] = b1f[t] * b1on + b2f[t];
+        dp[8 * ks + t] = neg_dq;
+      }
+    }
+    fetch_bias(next_key0);
 #pragma unroll
     for (int kk = 0; kk < 2; ++kk) {
-      mma32(st, kf[kk], qf[kk]);    // S^T[key][query]
-      mma32(dp, vf[kk], dof[kk]);   // dP^T[key][query]
+      mma32(st, kf[kk], qf[kk]);    // S^T[key][query] (+ biases)
+      mma32(dp, vf[kk], dof[kk]);   // dP^T[key][query] - Delta
     }
     V8 dsf[2];
 #pragma unroll
@@ -183,18 +206,35 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_kernel(BwdParams p) {
 #pragma unroll
       for (int t = 0; t < 8; ++t) {
         const int r = 8 * ks + t;
-        // (q.k + Bias1) + Bias2, the order of the forward
-        const float x = (st[r] + b1f[ks][t]) + b2f[ks][t];
-        const float pr = (key0 + reg_index(r, g) < s && q_ok) ? fast_exp2(x * kBwdLog2e - mq) : 0.0f;
-        ds[t] = pr * (dp[r] - dq_);
+        float pr = fast_exp2(st[r] * kBwdLog2e + neg_mq);
+        if (TAIL) pr = key0 + reg_index(r, g) < s ? pr : 0.0f;
+        ds[t] = pr * dp[r];
       }
       dsf[ks] = from_f32<T>(ds);
     }
     // dQ^T[d][query] += K^T[d][key] dS^T[key][query]: lane <-> query, register <-> d
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks) mma32(acc, ktf[ks], dsf[ks]);
-    __syncthreads();   // every wave is done with the tiles before the next step's are parked
+  };
+
+  // Block t is computed out of buffer t & 1 while block t + 1 waits in registers (fetched a
+  // step earlier) and is parked into the other buffer, which every wave has left at the
+  // barrier that ended step t - 1.
+  const int n_steps = (s + 31) >> 5;
+  const int n_full = s >> 5;
+  fetch(0);
+  fetch_bias(0);
+  piece.park(rm[0], tr[0], 1, tid);
+  __syncthreads();
+  fetch(min(1, n_steps - 1) * 32);
+  for (int t = 0; t < n_full; ++t) {
+    step(std::false_type{}, t % NB, t * 32, min(t + 1, n_steps - 1) * 32);
+    if (NB == 1) __syncthreads();
+    piece.park(rm[(t + 1) % NB], tr[(t + 1) % NB], 1, tid);
+    __syncthreads();
+    fetch(min(t + 2, n_steps - 1) * 32);
   }
+  if (n_full < n_steps) step(std::true_type{}, n_full % NB, n_full * 32, n_full * 32);
   if (q_ok) {
     T* dst = (T*)p.dq + elem(p, i, qi, h);
 #pragma unroll
@@ -210,15 +250,19 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_kernel(BwdParams p) {
 // dK and dV: a workgroup takes 128 keys of one (row, head), a wave 32 of them, and walks over
 // the query blocks; Q, dO, their transposes and the queries' statistics are shared.  Works on
 // S (not S^T): lane <-> key, register <-> query.  Each wave's Bias2 tile is loaded with the
-// lane on the query (8 keys per load) and turned through its own LDS tile.
+// lane on the query (8 keys per load) and turned through its own LDS tile; with Bias1 added it
+// is the initial value of the S accumulator, -Delta that of dP.  Lanes whose key lies beyond s
+// repeat key s - 1 and store nothing; queries beyond s exist in the last block only, which has
+// its own copy of the step.  Everything shared is double-buffered: one barrier a step.
 template <typename T, bool VEC>
-__global__ __launch_bounds__(256) void attn_bwd_kv_kernel(BwdParams p) {
+__global__ __launch_bounds__(256, (BwdCfg<T, VEC>::kMinBlocks)) void attn_bwd_kv_kernel(BwdParams p) {
   typedef typename Vec8<T>::type V8;
   typedef typename Vec4<T>::type V4;
-  __shared__ __attribute__((aligned(32))) T rm[2][32 * kTP];    // Q, dO
-  __shared__ __attribute__((aligned(32))) T tr[2][32 * kTP];    // Q^T, dO^T
-  __shared__ __attribute__((aligned(32))) T b2t[4][32 * kTP];   // per wave: Bias2 as [key][query]
-  __shared__ __attribute__((aligned(32))) float stats[2][32];   // log-sum-exp, Delta of the 32 queries
+  constexpr int NB = BwdCfg<T, VEC>::kBuffers;
+  __shared__ __attribute__((aligned(32))) T rm[NB][2][32 * kTP];    // Q, dO
+  __shared__ __attribute__((aligned(32))) T tr[NB][2][32 * kTP];    // Q^T, dO^T
+  __shared__ __attribute__((aligned(32))) T b2t[NB][4][32 * kTP];   // per wave: Bias2 as [key][query]
+  __shared__ __attribute__((aligned(32))) float stats[NB][2][32];   // -log-sum-exp, -Delta of the 32 queries
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, ln = lane & 31, g = lane >> 5;
   const int s = p.s, H = p.heads;
   constexpr bool vec = VEC;
@@ -233,7 +277,7 @@ __global__ __launch_bounds__(256) void attn_bwd_kv_kernel(BwdParams p) {
     vf[kk] = load8<T>((const T*)p.v + elem(p, i, kc, h) + 16 * kk + 8 * g);
   }
   const float b1v = p.b1 ? to_f32(((const T*)p.b1)[(int64_t)i * s + kc]) : 0.0f;
-  const float* stat_src = g == 0 ? p.lse : p.delta;   // wave 0 fetches the statistics
+  const float* stat_src = g == 0 ? p.lse : p.delta;   // every wave fetches, wave 0 publishes
   f32x16 acc_dk, acc_dv;
 #pragma unroll
   for (int r = 0; r < 16; ++r) acc_dk[r] = acc_dv[r] = 0.0f;
@@ -244,65 +288,91 @@ __global__ __launch_bounds__(256) void attn_bwd_kv_kernel(BwdParams p) {
   auto fetch = [&](int q0) {
     piece.fetch(p, p.q, p.dout, i, q0, h, tid);
     const int ql = min(q0 + ln, s - 1);
-    if (wave == 0) stat = stat_src[((int64_t)i * s + ql) * H + h];
+    stat = stat_src[((int64_t)i * s + ql) * H + h];
     const T* b2row = (const T*)p.b2 + ((int64_t)h * s + ql) * s;
     b2a = load_bias8_raw<T>(b2row, key0 + 16 * g, s, vec);
     b2b = load_bias8_raw<T>(b2row, key0 + 16 * g + 8, s, vec);
+    asm volatile("" ::: "memory");   // the loads are issued here, a step ahead of their use
   };
-  fetch(0);
-  for (int q0 = 0; q0 < s; q0 += 32) {
-    piece.park(rm, tr, 2, tid);
-    if (wave == 0) stats[g][ln] = stat;
+  auto park = [&](int buf) {
+    piece.park(rm[buf], tr[buf], 2, tid);
+    if (wave == 0) stats[buf][g][ln] = -stat;
 #pragma unroll
     for (int t = 0; t < 8; ++t) {
-      b2t[wave][(16 * g + t) * kTP + ln] = b2a[t];
-      b2t[wave][(16 * g + 8 + t) * kTP + ln] = b2b[t];
+      b2t[buf][wave][(16 * g + t) * kTP + ln] = b2a[t];
+      b2t[buf][wave][(16 * g + 8 + t) * kTP + ln] = b2b[t];
     }
-    __syncthreads();
-    if (q0 + 32 < s) fetch(q0 + 32);   // in flight while this step computes
-
+  };
+  // one block of 32 queries out of buffer `buf`; TAIL: the block holds queries beyond s
+  auto step = [&](auto tail_tag, int buf, int q0) {
+    constexpr bool TAIL = decltype(tail_tag)::value;
     V8 qf[2], dof[2];
 #pragma unroll
     for (int kk = 0; kk < 2; ++kk) {
-      qf[kk] = load8<T>(&rm[0][perm_row(ln) * kTP + 16 * kk + 8 * g]);
-      dof[kk] = load8<T>(&rm[1][perm_row(ln) * kTP + 16 * kk + 8 * g]);
+      qf[kk] = load8<T>(&rm[buf][0][perm_row(ln) * kTP + 16 * kk + 8 * g]);
+      dof[kk] = load8<T>(&rm[buf][1][perm_row(ln) * kTP + 16 * kk + 8 * g]);
     }
     f32x16 sm, dp;
+    f32x8 nlse[2];
 #pragma unroll
-    for (int r = 0; r < 16; ++r) sm[r] = dp[r] = 0.0f;
+    for (int ks = 0; ks < 2; ++ks) {
+      const int qb = 16 * ks + 8 * g;   // queries q0 + qb .. + 7 sit in registers 8 ks .. 8 ks + 7
+      nlse[ks] = *reinterpret_cast<const f32x8*>(&stats[buf][0][qb]);
+      const f32x8 ndel = *reinterpret_cast<const f32x8*>(&stats[buf][1][qb]);
+      const f32x8 b28 = to_f32(load8<T>(&b2t[buf][wave][ln * kTP + qb]));
+#pragma unroll
+      for (int t = 0; t < 8; ++t) {
+        sm[8 * ks + t] = b1v + b28[t];
+        dp[8 * ks + t] = ndel[t];
+      }
+    }
 #pragma unroll
     for (int kk = 0; kk < 2; ++kk) {
-      mma32(sm, qf[kk], kf[kk]);    // S[query][key]: lane <-> key, register <-> query
-      mma32(dp, dof[kk], vf[kk]);   // dP[query][key]
+      mma32(sm, qf[kk], kf[kk]);    // S[query][key] (+ biases): lane <-> key, register <-> query
+      mma32(dp, dof[kk], vf[kk]);   // dP[query][key] - Delta
     }
     V8 pf[2], dsf[2];
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks) {
-      const int qb = 16 * ks + 8 * g;   // queries q0 + qb .. + 7 sit in registers 8 ks .. 8 ks + 7
-      const f32x8 lse8 = *reinterpret_cast<const f32x8*>(&stats[0][qb]);
-      const f32x8 del8 = *reinterpret_cast<const f32x8*>(&stats[1][qb]);
-      const f32x8 b28 = to_f32(load8<T>(&b2t[wave][ln * kTP + qb]));
+      const int qb = 16 * ks + 8 * g;
       f32x8 pv, dv;
 #pragma unroll
       for (int t = 0; t < 8; ++t) {
         const int r = 8 * ks + t;
-        const float x = (sm[r] + b1v) + b28[t];   // (q.k + Bias1) + Bias2, the order of the forward
-        const float pr = (q0 + qb + t < s && k_ok) ? fast_exp2(x * kBwdLog2e - lse8[t]) : 0.0f;
+        float pr = fast_exp2(sm[r] * kBwdLog2e + nlse[ks][t]);
+        if (TAIL) pr = q0 + qb + t < s ? pr : 0.0f;
         pv[t] = pr;
-        dv[t] = pr * (dp[r] - del8[t]);
+        dv[t] = pr * dp[r];
       }
       pf[ks] = from_f32<T>(pv);
       dsf[ks] = from_f32<T>(dv);
     }
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks) {
-      const V8 qtf = load8<T>(&tr[0][ln * kTP + 16 * ks + 8 * g]);
-      const V8 dotf = load8<T>(&tr[1][ln * kTP + 16 * ks + 8 * g]);
+      const V8 qtf = load8<T>(&tr[buf][0][ln * kTP + 16 * ks + 8 * g]);
+      const V8 dotf = load8<T>(&tr[buf][1][ln * kTP + 16 * ks + 8 * g]);
       mma32(acc_dv, dotf, pf[ks]);    // dV^T[d][key] += dO^T[d][query] P[query][key]
       mma32(acc_dk, qtf, dsf[ks]);    // dK^T[d][key] += Q^T[d][query] dS[query][key]
     }
-    __syncthreads();   // every wave is done with the tiles before the next step's are parked
+  };
+
+  // Block t is computed out of buffer t & 1 while block t + 1 waits in registers (fetched a
+  // step earlier) and is parked into the other buffer, which every wave has left at the
+  // barrier that ended step t - 1.
+  const int n_steps = (s + 31) >> 5;
+  const int n_full = s >> 5;
+  fetch(0);
+  park(0);
+  __syncthreads();
+  fetch(min(1, n_steps - 1) * 32);
+  for (int t = 0; t < n_full; ++t) {
+    step(std::false_type{}, t % NB, t * 32);
+    if (NB == 1) __syncthreads();
+    park((t + 1) % NB);
+    __syncthreads();
+    fetch(min(t + 2, n_steps - 1) * 32);
   }
+  if (n_full < n_steps) step(std::true_type{}, n_full % NB, n_full * 32);
   if (k_ok) {
     T* dk = (T*)p.dk + elem(p, i, kc, h);
     T* dv = (T*)p.dv + elem(p, i, kc, h);
@@ -322,11 +392,15 @@ __global__ __launch_bounds__(256) void attn_bwd_kv_kernel(BwdParams p) {
 
 // dBias2: a workgroup takes 64 queries x 64 keys of one head, a wave one 32 x 32 quadrant, and
 // walks over the rows; the two Q / dO tiles and the two K / V tiles of a row are shared.
-// Works on S^T like dQ.  Bias2 itself does not change along the walk and stays in registers.
+// Works on S^T like dQ.  Bias2 itself does not change along the walk and stays in registers;
+// a row's Bias1 is added to it for the initial value of the S^T accumulator, -Delta is that of
+// dP^T.  Nothing in the walk looks at s: queries and keys beyond it repeat the last one, and
+// what accumulates for them is not stored.
 template <typename T, bool VEC>
-__global__ __launch_bounds__(256) void attn_bwd_db2_kernel(BwdParams p) {
+__global__ __launch_bounds__(256, (BwdCfg<T, VEC>::kMinBlocks)) void attn_bwd_db2_kernel(BwdParams p) {
   typedef typename Vec8<T>::type V8;
-  __shared__ __attribute__((aligned(32))) T tiles[4][64 * kTP];   // Q, dO (64 queries), K, V (64 keys)
+  constexpr int NB = BwdCfg<T, VEC>::kBuffers;
+  __shared__ __attribute__((aligned(32))) T tiles[NB][4][64 * kTP];   // Q, dO (64 queries), K, V (64 keys)
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, ln = lane & 31, g = lane >> 5;
   const int s = p.s, H = p.heads;
   constexpr bool vec = VEC;
@@ -340,6 +414,10 @@ __global__ __launch_bounds__(256) void attn_bwd_db2_kernel(BwdParams p) {
   f32x8 b2f[2];
 #pragma unroll
   for (int ks = 0; ks < 2; ++ks) b2f[ks] = load_bias8<T>(b2row, key0 + 16 * ks + 8 * g, s, vec);
+  // (without a Bias1 the loads go to Bias2's row and count for nothing: no load under a branch)
+  const T* b1base = p.b1 ? (const T*)p.b1 : b2row;
+  const int64_t b1pitch = p.b1 ? s : 0;
+  const float b1on = p.b1 ? 1.0f : 0.0f;
   f32x16 acc;
 #pragma unroll
   for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
@@ -358,39 +436,51 @@ __global__ __launch_bounds__(256) void attn_bwd_db2_kernel(BwdParams p) {
     dq_n = p.delta[((int64_t)i * s + qi) * H + h];
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks)
-      b1n[ks] = p.b1 ? load_bias8_raw<T>((const T*)p.b1 + (int64_t)i * s, key0 + 16 * ks + 8 * g, s, vec)
-                     : zero_frag<T>();
+      b1n[ks] = load_bias8_raw<T>(b1base + i * b1pitch, key0 + 16 * ks + 8 * g, s, vec);
   };
+  // Row i is computed out of buffer i % NB while row i + 1, fetched a step earlier, is parked
+  // (two buffers: into the other one, which every wave left at the last barrier).
+  const int last = p.n_rows - 1;
   fetch(0);
+#pragma unroll
+  for (int w = 0; w < 4; ++w) store8<T>(&tiles[0][w][crow * kTP + cc], piece[w]);
+  float neg_mq = -mq_n, neg_dq = -dq_n;
+  V8 b1c[2] = {b1n[0], b1n[1]};
+  __syncthreads();
   for (int i = 0; i < p.n_rows; ++i) {
-#pragma unroll
-    for (int w = 0; w < 4; ++w) store8<T>(&tiles[w][crow * kTP + cc], piece[w]);
-    const float mq = mq_n, dq_ = dq_n;
-    f32x8 b1f[2];
-#pragma unroll
-    for (int ks = 0; ks < 2; ++ks) b1f[ks] = to_f32(b1n[ks]);
-    __syncthreads();
-    if (i + 1 < p.n_rows) fetch(i + 1);   // in flight while this step computes
-
+    const int buf = i % NB;
+    fetch(min(i + 1, last));
+    asm volatile("" ::: "memory");   // the loads are issued here, a step ahead of their use
     f32x16 st, dp;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) st[r] = dp[r] = 0.0f;
+    for (int ks = 0; ks < 2; ++ks) {
+      const f32x8 b1f = to_f32(b1c[ks]);
+#pragma unroll
+      for (int t = 0; t < 8; ++t) {
+        st[8 * ks + t] = b1f[t] * b1on + b2f[ks][t];
+        dp[8 * ks + t] = neg_dq;
+      }
+    }
 #pragma unroll
     for (int kk = 0; kk < 2; ++kk) {
-      const V8 qf = load8<T>(&tiles[0][(32 * wq + ln) * kTP + 16 * kk + 8 * g]);
-      const V8 dof = load8<T>(&tiles[1][(32 * wq + ln) * kTP + 16 * kk + 8 * g]);
-      const V8 kf = load8<T>(&tiles[2][(32 * wk + perm_row(ln)) * kTP + 16 * kk + 8 * g]);
-      const V8 vf = load8<T>(&tiles[3][(32 * wk + perm_row(ln)) * kTP + 16 * kk + 8 * g]);
-      mma32(st, kf, qf);    // S^T[key][query]
-      mma32(dp, vf, dof);   // dP^T[key][query]
+      const V8 qf = load8<T>(&tiles[buf][0][(32 * wq + ln) * kTP + 16 * kk + 8 * g]);
+      const V8 dof = load8<T>(&tiles[buf][1][(32 * wq + ln) * kTP + 16 * kk + 8 * g]);
+      const V8 kf = load8<T>(&tiles[buf][2][(32 * wk + perm_row(ln)) * kTP + 16 * kk + 8 * g]);
+      const V8 vf = load8<T>(&tiles[buf][3][(32 * wk + perm_row(ln)) * kTP + 16 * kk + 8 * g]);
+      mma32(st, kf, qf);    // S^T[key][query] (+ biases)
+      mma32(dp, vf, dof);   // dP^T[key][query] - Delta
     }
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const float x = (st[r] + b1f[r >> 3][r & 7]) + b2f[r >> 3][r & 7];
-      const float pr = (key0 + reg_index(r, g) < s && q_ok) ? fast_exp2(x * kBwdLog2e - mq) : 0.0f;
-      acc[r] += pr * (dp[r] - dq_);
-    }
-    __syncthreads();   // every wave is done with the tiles before the next row's are parked
+    for (int r = 0; r < 16; ++r) acc[r] += fast_exp2(st[r] * kBwdLog2e + neg_mq) * dp[r];
+    if (NB == 1) __syncthreads();
+    // the next row: tiles into LDS, its statistics and Bias1 into this step's places
+#pragma unroll
+    for (int w = 0; w < 4; ++w) store8<T>(&tiles[(i + 1) % NB][w][crow * kTP + cc], piece[w]);
+    neg_mq = -mq_n;
+    neg_dq = -dq_n;
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) b1c[ks] = b1n[ks];
+    __syncthreads();
   }
   if (q_ok) {
     T* dst = (T*)p.db2 + ((int64_t)h * s + qi) * s;
