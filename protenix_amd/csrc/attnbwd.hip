@@ -422,21 +422,30 @@ __global__ __launch_bounds__(256, (BwdCfg<T, VEC>::kMinBlocks)) void attn_bwd_db
 #pragma unroll
   for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
 
-  // thread t: 8 channels (t & 3) of row t >> 2 of each of the four 64-row tiles
+  // thread t: 8 channels (t & 3) of row t >> 2 of each of the four 64-row tiles.  Along the
+  // walk only the row's base address changes, the same for all lanes: what a lane adds to it
+  // is formed once.
   const int crow = tid >> 2, cc = 8 * (tid & 3);
-  const int cq = min(qs0 + crow, s - 1), ck = min(ks0 + crow, s - 1);
+  const unsigned off_q = ((unsigned)min(qs0 + crow, s - 1) * H + h) * 32 + cc;
+  const unsigned off_k = ((unsigned)min(ks0 + crow, s - 1) * H + h) * 32 + cc;
+  const unsigned off_stat = (unsigned)qi * H + h;
+  unsigned off_b1[2];
+#pragma unroll
+  for (int ks = 0; ks < 2; ++ks) off_b1[ks] = vec ? min(key0 + 16 * ks + 8 * g, s - 8) : 0;
+  const int64_t row_elems = (int64_t)s * H * 32, row_stats = (int64_t)s * H;
   V8 piece[4], b1n[2];
   float mq_n = 0.0f, dq_n = 0.0f;
   auto fetch = [&](int i) {
-    piece[0] = load8<T>((const T*)p.q + elem(p, i, cq, h) + cc);
-    piece[1] = load8<T>((const T*)p.dout + elem(p, i, cq, h) + cc);
-    piece[2] = load8<T>((const T*)p.k + elem(p, i, ck, h) + cc);
-    piece[3] = load8<T>((const T*)p.v + elem(p, i, ck, h) + cc);
-    mq_n = p.lse[((int64_t)i * s + qi) * H + h];
-    dq_n = p.delta[((int64_t)i * s + qi) * H + h];
+    piece[0] = load8<T>((const T*)p.q + i * row_elems + off_q);
+    piece[1] = load8<T>((const T*)p.dout + i * row_elems + off_q);
+    piece[2] = load8<T>((const T*)p.k + i * row_elems + off_k);
+    piece[3] = load8<T>((const T*)p.v + i * row_elems + off_k);
+    mq_n = (p.lse + i * row_stats)[off_stat];
+    dq_n = (p.delta + i * row_stats)[off_stat];
+    const T* b1row = b1base + i * b1pitch;
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks)
-      b1n[ks] = load_bias8_raw<T>(b1base + i * b1pitch, key0 + 16 * ks + 8 * g, s, vec);
+      b1n[ks] = vec ? load8<T>(b1row + off_b1[ks]) : load_bias8_raw<T>(b1row, key0 + 16 * ks + 8 * g, s, false);
   };
   // Row i is computed out of buffer i % NB while row i + 1, fetched a step earlier, is parked
   // (two buffers: into the other one, which every wave left at the last barrier).
