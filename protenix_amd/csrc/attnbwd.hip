@@ -71,12 +71,13 @@ __device__ __forceinline__ f32x8 load_bias8(const T* row, int kb, int s, bool ve
 
 }  // namespace
 
-// 16-bit kernels double-buffer their shared tiles (one barrier a step) and are held to three
-// workgroups per compute unit where rows are 8-aligned; fp32 tiles are twice as large and stay
-// single-buffered (two barriers a step).
+// 16-bit kernels double-buffer their shared tiles (one barrier a step) and are held to the
+// registers of three waves per SIMD where rows are 8-aligned; fp32 tiles are twice as
+// large and stay single-buffered (two barriers a step).
 template <typename T, bool VEC> struct BwdCfg {
   static constexpr int kBuffers = sizeof(T) == 2 ? 2 : 1;
-  static constexpr int kMinBlocks = sizeof(T) == 2 ? (VEC ? 3 : 2) : 1;
+  // (the second argument of __launch_bounds__: waves per SIMD the register budget allows for)
+  static constexpr int kMinWaves = sizeof(T) == 2 ? (VEC ? 3 : 2) : 1;
 };
 
 // Delta[i][j][h] = sum_d O * dO
@@ -125,12 +126,13 @@ template <typename T> struct TilePiece {
 // beyond s repeat query s - 1 and store nothing; keys beyond s exist in the last block only,
 // which has its own copy of the step.  The shared tiles are double-buffered: one barrier a step.
 template <typename T, bool VEC>
-__global__ __launch_bounds__(256, (BwdCfg<T, VEC>::kMinBlocks)) void attn_bwd_dq_kernel(BwdParams p) {
+__global__ __launch_bounds__(256, (BwdCfg<T, VEC>::kMinWaves)) void attn_bwd_dq_kernel(BwdParams p) {
   typedef typename Vec8<T>::type V8;
   typedef typename Vec4<T>::type V4;
   constexpr int NB = BwdCfg<T, VEC>::kBuffers;
   __shared__ __attribute__((aligned(32))) T rm[NB][2][32 * kTP];   // K, V
   __shared__ __attribute__((aligned(32))) T tr[NB][1][32 * kTP];   // K^T
+  __shared__ __attribute__((aligned(32))) T b2s[NB][128 * kTP];    // Bias2 of the 128 queries x 32 keys
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, ln = lane & 31, g = lane >> 5;
   const int s = p.s, H = p.heads;
   constexpr bool vec = VEC;   // rows of s keys are 8-aligned
@@ -138,10 +140,9 @@ __global__ __launch_bounds__(256, (BwdCfg<T, VEC>::kMinBlocks)) void attn_bwd_dq
   const int q0 = (blockIdx.x * 4 + wave) * 32;
   const int qi = min(q0 + ln, s - 1);
   const bool q_ok = q0 + ln < s;
-  const T* b2row = (const T*)p.b2 + ((int64_t)h * s + qi) * s;
-  // (without a Bias1 the loads go to Bias2's row and count for nothing: a load under a branch
-  // would make every wait for memory a wait for all of it)
-  const T* b1row = p.b1 ? (const T*)p.b1 + (int64_t)i * s : b2row;
+  // (without a Bias1 the loads go to a row of Bias2 and count for nothing: a load under a
+  // branch would make every wait for memory a wait for all of it)
+  const T* b1row = p.b1 ? (const T*)p.b1 + (int64_t)i * s : (const T*)p.b2 + (int64_t)h * s * s;
   const float b1on = p.b1 ? 1.0f : 0.0f;
 
   V8 qf[2], dof[2];
@@ -156,20 +157,32 @@ __global__ __launch_bounds__(256, (BwdCfg<T, VEC>::kMinBlocks)) void attn_bwd_dq
 #pragma unroll
   for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
 
+  // Bias2 comes in through LDS like the tiles: four neighbouring lanes read the 64 bytes a
+  // query's row has for the block (a lane reading 16 bytes of its own query's row touches as
+  // many cache lines per load as it has lanes, and the texture path was busy 96 % of the time).
   TilePiece<T> piece;
   V8 b1n[2], b2n[2];
+  const int b2col = 8 * (tid & 3);
+  const T* b2rows[2];
+#pragma unroll
+  for (int j = 0; j < 2; ++j)
+    b2rows[j] = (const T*)p.b2 + ((int64_t)h * s + min((int)blockIdx.x * 128 + 64 * j + (tid >> 2), s - 1)) * s;
   // (the compiler barriers keep the loads where they are written, a step ahead of their use:
   // left alone, the compiler moves them down to the use and waits there)
   auto fetch = [&](int key0) {
     piece.fetch(p, p.k, p.v, i, key0, h, tid);
+#pragma unroll
+    for (int j = 0; j < 2; ++j) b2n[j] = load_bias8_raw<T>(b2rows[j], key0 + b2col, s, vec);
     asm volatile("" ::: "memory");
+  };
+  auto park = [&](int buf) {
+    piece.park(rm[buf], tr[buf], 1, tid);
+#pragma unroll
+    for (int j = 0; j < 2; ++j) store8<T>(&b2s[buf][(64 * j + (tid >> 2)) * kTP + b2col], b2n[j]);
   };
   auto fetch_bias = [&](int key0) {
 #pragma unroll
-    for (int ks = 0; ks < 2; ++ks) {
-      b2n[ks] = load_bias8_raw<T>(b2row, key0 + 16 * ks + 8 * g, s, vec);
-      b1n[ks] = load_bias8_raw<T>(b1row, key0 + 16 * ks + 8 * g, s, vec);
-    }
+    for (int ks = 0; ks < 2; ++ks) b1n[ks] = load_bias8_raw<T>(b1row, key0 + 16 * ks + 8 * g, s, vec);
     asm volatile("" ::: "memory");
   };
   // one block of 32 keys out of buffer `buf`; TAIL: the block holds keys beyond s.  The biases
@@ -186,7 +199,8 @@ __global__ __launch_bounds__(256, (BwdCfg<T, VEC>::kMinBlocks)) void attn_bwd_dq
     f32x16 st, dp;
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks) {
-      const f32x8 b1f = to_f32(b1n[ks]), b2f = to_f32(b2n[ks]);
+      const f32x8 b1f = to_f32(b1n[ks]);
+      const f32x8 b2f = to_f32(load8<T>(&b2s[buf][(32 * wave + ln) * kTP + 16 * ks + 8 * g]));
 #pragma unroll
       for (int t = 0; t < 8; ++t) {
         st[8 * ks + t] = b1f[t] * b1on + b2f[t];
@@ -224,13 +238,13 @@ __global__ __launch_bounds__(256, (BwdCfg<T, VEC>::kMinBlocks)) void attn_bwd_dq
   const int n_full = s >> 5;
   fetch(0);
   fetch_bias(0);
-  piece.park(rm[0], tr[0], 1, tid);
+  park(0);
   __syncthreads();
   fetch(min(1, n_steps - 1) * 32);
   for (int t = 0; t < n_full; ++t) {
     step(std::false_type{}, t % NB, t * 32, min(t + 1, n_steps - 1) * 32);
     if (NB == 1) __syncthreads();
-    piece.park(rm[(t + 1) % NB], tr[(t + 1) % NB], 1, tid);
+    park((t + 1) % NB);
     __syncthreads();
     fetch(min(t + 2, n_steps - 1) * 32);
   }
@@ -255,7 +269,7 @@ __global__ __launch_bounds__(256, (BwdCfg<T, VEC>::kMinBlocks)) void attn_bwd_dq
 // repeat key s - 1 and store nothing; queries beyond s exist in the last block only, which has
 // its own copy of the step.  Everything shared is double-buffered: one barrier a step.
 template <typename T, bool VEC>
-__global__ __launch_bounds__(256, (BwdCfg<T, VEC>::kMinBlocks)) void attn_bwd_kv_kernel(BwdParams p) {
+__global__ __launch_bounds__(256, (BwdCfg<T, VEC>::kMinWaves)) void attn_bwd_kv_kernel(BwdParams p) {
   typedef typename Vec8<T>::type V8;
   typedef typename Vec4<T>::type V4;
   constexpr int NB = BwdCfg<T, VEC>::kBuffers;
@@ -397,7 +411,7 @@ __global__ __launch_bounds__(256, (BwdCfg<T, VEC>::kMinBlocks)) void attn_bwd_kv
 // dP^T.  Nothing in the walk looks at s: queries and keys beyond it repeat the last one, and
 // what accumulates for them is not stored.
 template <typename T, bool VEC>
-__global__ __launch_bounds__(256, (BwdCfg<T, VEC>::kMinBlocks)) void attn_bwd_db2_kernel(BwdParams p) {
+__global__ __launch_bounds__(256, (BwdCfg<T, VEC>::kMinWaves)) void attn_bwd_db2_kernel(BwdParams p) {
   typedef typename Vec8<T>::type V8;
   constexpr int NB = BwdCfg<T, VEC>::kBuffers;
   __shared__ __attribute__((aligned(32))) T tiles[NB][4][64 * kTP];   // Q, dO (64 queries), K, V (64 keys)
