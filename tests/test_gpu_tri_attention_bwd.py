@@ -63,6 +63,22 @@ def test_gradients_against_autograd_of_the_torch_path(dtype, B, N, S, H, n_maske
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("N,S", [(5, 96), (3, 50)])
+def test_no_bias1_is_a_bias1_of_zeros(dtype, N, S):
+    """Without a mask bias the kernels read a row of Bias2 in its place and weigh it with zero:
+    same gradients as with a Bias1 of zeros, and as the torch path's."""
+    q, k, v, b1, b2, do = _operands(1, N, S, 2, dtype, seed=S)
+    want = _autograd_reference(q, k, v, b1, b2, do)
+    with_zeros = _product(q, k, v, b1, b2, do)
+    qc, kc, vc, b2c = (t.cuda().requires_grad_(True) for t in (q, k, v, b2))
+    P.TriAttentionFunction.apply(qc, kc, vc, None, b2c).backward(do.cuda())
+    for name, g, z, w in zip(("dQ", "dK", "dV", "dBias2"), (qc.grad, kc.grad, vc.grad, b2c.grad),
+                             with_zeros[1:], want[1:]):
+        assert torch.equal(g, z), name
+        assert rel_err(g, w) <= tol(dtype), name
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_bias2_broadcast_over_the_batch_and_not_requiring_grad(dtype):
     ops = _operands(2, 16, 40, 4, dtype, seed=9, n_masked=3, b2_batch=1)
     want = _autograd_reference(*ops)
