@@ -80,6 +80,27 @@ template <typename T, bool VEC> struct BwdCfg {
   static constexpr int kMinWaves = sizeof(T) == 2 ? (VEC ? 3 : 2) : 1;
 };
 
+// 16-bit tiles are parked in LDS row-major only; an operand that a product needs with the
+// tile's rows in the K slots is read with the transposing LDS load of gfx950
+// (ds_read_b64_tr_b16: the 16 lanes of a block hand in the addresses of 4 x 16 elements, 4
+// lanes per row, and lane j of the block gets column j of the 4 rows).  Two of them: the lane
+// gets column col0 + lane % 16 of rows row0 .. row0 + 7.  fp32 has no such load and keeps
+// transposed copies of its tiles.
+template <typename T> struct Turned {
+  static constexpr bool value = sizeof(T) == 2;
+};
+__device__ __forceinline__ bf16x8 load8_turned(const bf16_t* tile, int pitch, int row0, int col0, int lane) {
+  typedef short v4s __attribute__((ext_vector_type(4)));
+  typedef short v8s __attribute__((ext_vector_type(8)));
+  typedef __attribute__((address_space(3))) v4s* LdsV4;
+  const int i = lane & 15;
+  const bf16_t* a = tile + (row0 + (i >> 2)) * pitch + col0 + 4 * (i & 3);
+  const v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsV4)a);
+  const v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsV4)(a + 4 * pitch));
+  return __builtin_bit_cast(bf16x8, (v8s)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+}
+__device__ __forceinline__ f32x8 load8_turned(const float*, int, int, int, int) { return f32x8{}; }   // (never called)
+
 // Delta[i][j][h] = sum_d O * dO
 template <typename T>
 __global__ __launch_bounds__(256) void attn_bwd_delta_kernel(BwdParams p) {
@@ -107,13 +128,14 @@ template <typename T> struct TilePiece {
     const int row = min(pos0 + ((tid & 127) >> 2), p.s - 1);
     v = load8<T>((const T*)(tid >> 7 ? b : a) + elem(p, i, row, h) + 8 * (tid & 3));
   }
-  // row-major into rm[tid >> 7]; with `tr`, transposed ([channel][row]) into tr[tid >> 7] as well
-  __device__ __forceinline__ void park(T (*rm)[32 * kTP], T (*tr)[32 * kTP], int n_tr, int tid) const {
+  // row-major into rm[tid >> 7]; the first n_tr tiles also transposed ([channel][row]) into
+  // tr + (tid >> 7) * 32 * kTP
+  __device__ __forceinline__ void park(T (*rm)[32 * kTP], T* tr, int n_tr, int tid) const {
     const int which = tid >> 7, row = (tid & 127) >> 2, c0 = 8 * (tid & 3);
     store8<T>(&rm[which][row * kTP + c0], v);
     if (which < n_tr) {
 #pragma unroll
-      for (int t = 0; t < 8; ++t) tr[which][(c0 + t) * kTP + row] = v[t];
+      for (int t = 0; t < 8; ++t) tr[which * 32 * kTP + (c0 + t) * kTP + row] = v[t];
     }
   }
 };
@@ -131,7 +153,8 @@ __global__ __launch_bounds__(256, (BwdCfg<T, VEC>::kMinWaves)) void attn_bwd_dq_
   typedef typename Vec4<T>::type V4;
   constexpr int NB = BwdCfg<T, VEC>::kBuffers;
   __shared__ __attribute__((aligned(32))) T rm[NB][2][32 * kTP];   // K, V
-  __shared__ __attribute__((aligned(32))) T tr[NB][1][32 * kTP];   // K^T
+  constexpr bool TURN = Turned<T>::value;
+  __shared__ __attribute__((aligned(32))) T tr[TURN ? 8 : NB * 32 * kTP];   // K^T (fp32 only)
   __shared__ __attribute__((aligned(32))) T b2s[NB][128 * kTP];    // Bias2 of the 128 queries x 32 keys
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, ln = lane & 31, g = lane >> 5;
   const int s = p.s, H = p.heads;
@@ -176,7 +199,7 @@ __global__ __launch_bounds__(256, (BwdCfg<T, VEC>::kMinWaves)) void attn_bwd_dq_
     asm volatile("" ::: "memory");
   };
   auto park = [&](int buf) {
-    piece.park(rm[buf], tr[buf], 1, tid);
+    piece.park(rm[buf], tr + (TURN ? 0 : buf * 32 * kTP), TURN ? 0 : 1, tid);
 #pragma unroll
     for (int j = 0; j < 2; ++j) store8<T>(&b2s[buf][(64 * j + (tid >> 2)) * kTP + b2col], b2n[j]);
   };
@@ -194,7 +217,8 @@ __global__ __launch_bounds__(256, (BwdCfg<T, VEC>::kMinWaves)) void attn_bwd_dq_
     for (int kk = 0; kk < 2; ++kk) {
       kf[kk] = load8<T>(&rm[buf][0][perm_row(ln) * kTP + 16 * kk + 8 * g]);
       vf[kk] = load8<T>(&rm[buf][1][perm_row(ln) * kTP + 16 * kk + 8 * g]);
-      ktf[kk] = load8<T>(&tr[buf][0][ln * kTP + 16 * kk + 8 * g]);
+      ktf[kk] = TURN ? load8_turned(rm[buf][0], kTP, 16 * kk + 8 * g, 16 * ((lane >> 4) & 1), lane)
+                     : load8<T>(&tr[TURN ? 0 : buf * 32 * kTP + ln * kTP + 16 * kk + 8 * g]);
     }
     f32x16 st, dp;
 #pragma unroll
@@ -263,9 +287,9 @@ __global__ __launch_bounds__(256, (BwdCfg<T, VEC>::kMinWaves)) void attn_bwd_dq_
 
 // dK and dV: a workgroup takes 128 keys of one (row, head), a wave 32 of them, and walks over
 // the query blocks; Q, dO, their transposes and the queries' statistics are shared.  Works on
-// S (not S^T): lane <-> key, register <-> query.  Each wave's Bias2 tile is loaded with the
-// lane on the query (8 keys per load) and turned through its own LDS tile; with Bias1 added it
-// is the initial value of the S accumulator, -Delta that of dP.  Lanes whose key lies beyond s
+// S (not S^T): lane <-> key, register <-> query.  Bias2 is loaded along the queries' rows (8
+// keys per load) and turned on its way through LDS; with Bias1 added it is the initial value
+// of the S accumulator, -Delta that of dP.  Lanes whose key lies beyond s
 // repeat key s - 1 and store nothing; queries beyond s exist in the last block only, which has
 // its own copy of the step.  Everything shared is double-buffered: one barrier a step.
 template <typename T, bool VEC>
@@ -274,8 +298,12 @@ __global__ __launch_bounds__(256, (BwdCfg<T, VEC>::kMinWaves)) void attn_bwd_kv_
   typedef typename Vec4<T>::type V4;
   constexpr int NB = BwdCfg<T, VEC>::kBuffers;
   __shared__ __attribute__((aligned(32))) T rm[NB][2][32 * kTP];    // Q, dO
-  __shared__ __attribute__((aligned(32))) T tr[NB][2][32 * kTP];    // Q^T, dO^T
-  __shared__ __attribute__((aligned(32))) T b2t[NB][4][32 * kTP];   // per wave: Bias2 as [key][query]
+  constexpr bool TURN = Turned<T>::value;
+  __shared__ __attribute__((aligned(32))) T tr[TURN ? 8 : NB * 2 * 32 * kTP];   // Q^T, dO^T (fp32 only)
+  // Bias2 of the step: fp32 per wave as [key][query]; 16-bit one tile [query][128 keys] for
+  // the workgroup, as it was loaded
+  constexpr int kB2P = 136;   // pitch of the 16-bit tile (elements)
+  __shared__ __attribute__((aligned(32))) T b2t[NB][TURN ? 32 * kB2P : 4 * 32 * kTP];
   __shared__ __attribute__((aligned(32))) float stats[NB][2][32];   // -log-sum-exp, -Delta of the 32 queries
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, ln = lane & 31, g = lane >> 5;
   const int s = p.s, H = p.heads;
@@ -298,23 +326,33 @@ __global__ __launch_bounds__(256, (BwdCfg<T, VEC>::kMinWaves)) void attn_bwd_kv_
 
   TilePiece<T> piece;
   float stat = 0.0f;
-  V8 b2a, b2b;   // lane (ln, g): Bias2 of query q0 + ln for keys key0 + 16 g .. + 15
+  // fp32: lane (ln, g) loads Bias2 of query q0 + ln for this wave's keys key0 + 16 g .. + 15.
+  // 16-bit: thread t loads keys 8 (t & 7) .. + 7 of both halves of the workgroup's 128 keys for
+  // query q0 + (t >> 3): eight neighbouring lanes read one 128-byte line (a lane per query
+  // touches as many lines per load as it has lanes).
+  V8 b2a, b2b;
+  const int b2q = TURN ? tid >> 3 : ln;
+  const int b2k = TURN ? (int)blockIdx.x * 128 + 8 * (tid & 7) : key0 + 16 * g;
   auto fetch = [&](int q0) {
     piece.fetch(p, p.q, p.dout, i, q0, h, tid);
-    const int ql = min(q0 + ln, s - 1);
-    stat = stat_src[((int64_t)i * s + ql) * H + h];
-    const T* b2row = (const T*)p.b2 + ((int64_t)h * s + ql) * s;
-    b2a = load_bias8_raw<T>(b2row, key0 + 16 * g, s, vec);
-    b2b = load_bias8_raw<T>(b2row, key0 + 16 * g + 8, s, vec);
+    stat = stat_src[((int64_t)i * s + min(q0 + ln, s - 1)) * H + h];
+    const T* b2row = (const T*)p.b2 + ((int64_t)h * s + min(q0 + b2q, s - 1)) * s;
+    b2a = load_bias8_raw<T>(b2row, b2k, s, vec);
+    b2b = load_bias8_raw<T>(b2row, b2k + (TURN ? 64 : 8), s, vec);
     asm volatile("" ::: "memory");   // the loads are issued here, a step ahead of their use
   };
   auto park = [&](int buf) {
-    piece.park(rm[buf], tr[buf], 2, tid);
+    piece.park(rm[buf], tr + (TURN ? 0 : buf * 2 * 32 * kTP), TURN ? 0 : 2, tid);
     if (wave == 0) stats[buf][g][ln] = -stat;
+    if (TURN) {
+      store8<T>(&b2t[buf][b2q * kB2P + 8 * (tid & 7)], b2a);
+      store8<T>(&b2t[buf][b2q * kB2P + 8 * (tid & 7) + 64], b2b);
+    } else {
 #pragma unroll
-    for (int t = 0; t < 8; ++t) {
-      b2t[buf][wave][(16 * g + t) * kTP + ln] = b2a[t];
-      b2t[buf][wave][(16 * g + 8 + t) * kTP + ln] = b2b[t];
+      for (int t = 0; t < 8; ++t) {
+        b2t[buf][wave * 32 * kTP + (16 * g + t) * kTP + ln] = b2a[t];
+        b2t[buf][wave * 32 * kTP + (16 * g + 8 + t) * kTP + ln] = b2b[t];
+      }
     }
   };
   // one block of 32 queries out of buffer `buf`; TAIL: the block holds queries beyond s
@@ -333,7 +371,8 @@ __global__ __launch_bounds__(256, (BwdCfg<T, VEC>::kMinWaves)) void attn_bwd_kv_
       const int qb = 16 * ks + 8 * g;   // queries q0 + qb .. + 7 sit in registers 8 ks .. 8 ks + 7
       nlse[ks] = *reinterpret_cast<const f32x8*>(&stats[buf][0][qb]);
       const f32x8 ndel = *reinterpret_cast<const f32x8*>(&stats[buf][1][qb]);
-      const f32x8 b28 = to_f32(load8<T>(&b2t[buf][wave][ln * kTP + qb]));
+      const f32x8 b28 = to_f32(TURN ? load8_turned(b2t[buf], kB2P, qb, 32 * wave + 16 * ((lane >> 4) & 1), lane)
+                                    : load8<T>(&b2t[buf][wave * 32 * kTP + ln * kTP + qb]));
 #pragma unroll
       for (int t = 0; t < 8; ++t) {
         sm[8 * ks + t] = b1v + b28[t];
@@ -363,8 +402,10 @@ __global__ __launch_bounds__(256, (BwdCfg<T, VEC>::kMinWaves)) void attn_bwd_kv_
     }
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks) {
-      const V8 qtf = load8<T>(&tr[buf][0][ln * kTP + 16 * ks + 8 * g]);
-      const V8 dotf = load8<T>(&tr[buf][1][ln * kTP + 16 * ks + 8 * g]);
+      const V8 qtf = TURN ? load8_turned(rm[buf][0], kTP, 16 * ks + 8 * g, 16 * ((lane >> 4) & 1), lane)
+                          : load8<T>(&tr[TURN ? 0 : (buf * 2 + 0) * 32 * kTP + ln * kTP + 16 * ks + 8 * g]);
+      const V8 dotf = TURN ? load8_turned(rm[buf][1], kTP, 16 * ks + 8 * g, 16 * ((lane >> 4) & 1), lane)
+                           : load8<T>(&tr[TURN ? 0 : (buf * 2 + 1) * 32 * kTP + ln * kTP + 16 * ks + 8 * g]);
       mma32(acc_dv, dotf, pf[ks]);    // dV^T[d][key] += dO^T[d][query] P[query][key]
       mma32(acc_dk, qtf, dsf[ks]);    // dK^T[d][key] += Q^T[d][query] dS[query][key]
     }
