@@ -5,17 +5,19 @@
 //   P = 2^(S log2 e - M),  S = Q K^T + Bias1 + Bias2,  Delta = rowsum(O * dO),
 //   dS = P * (dO V^T - Delta)
 // it produces  dV = P^T dO,  dK = dS^T Q,  dQ = dS K,  dBias2[h] = sum over rows of dS.
-// Four kernels, as in the reference (preprocess, dK/dV, dQ, dBias2); P is recomputed, the
+// Three kernels - dQ, which also forms Delta (the reference's preprocess kernel) and leaves it
+// for the others, dK/dV, dBias2 - where the reference has four; P is recomputed, the
 // logits are never stored.  One wave owns a 32 x 32 block of (query, key) pairs and walks over
 // the other index; every product runs on MFMA with fp32 accumulation (conventions of
 // common.h).  The register <-> index permutation of single.hip makes the recomputed P and dS
 // usable as MFMA operands as they sit in the accumulators.
 // What bounds these kernels is the operand stream out of L2 (6 to 8 KB per block pair when
-// every wave fetches its own), so the four waves of a workgroup take neighbouring blocks and
-// share the tiles that walk: the workgroup loads each tile once, one step ahead, into
-// registers, parks it in LDS row-major and (for the operands a product needs with the walking
-// index in the K slots: K^T for dQ, Q^T and dO^T for dK / dV) transposed, and every wave reads
-// its MFMA fragments from there.
+// every wave fetches its own) and the cache lines each load touches, so the four waves of a
+// workgroup take neighbouring blocks and share the tiles that walk: the workgroup loads each
+// tile once, one step ahead, into registers, parks it in LDS row-major, and every wave reads
+// its MFMA fragments from there - also those a product needs with the walking index in the K
+// slots (K^T for dQ, Q^T and dO^T for dK / dV), which 16-bit tiles give through the
+// transposing LDS load and fp32 tiles through a transposed copy.
 #include <type_traits>
 #include "common.h"
 #include "kernels.h"
@@ -101,24 +103,6 @@ __device__ __forceinline__ bf16x8 load8_turned(const bf16_t* tile, int pitch, in
 }
 __device__ __forceinline__ f32x8 load8_turned(const float*, int, int, int, int) { return f32x8{}; }   // (never called)
 
-// Delta[i][j][h] = sum_d O * dO
-template <typename T>
-__global__ __launch_bounds__(256) void attn_bwd_delta_kernel(BwdParams p) {
-  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  const int64_t total = (int64_t)p.n_rows * p.s * p.heads;
-  if (idx >= total) return;
-  const T* o = (const T*)p.o + idx * 32;
-  const T* d = (const T*)p.dout + idx * 32;
-  float acc = 0.0f;
-#pragma unroll
-  for (int c = 0; c < 4; ++c) {
-    const f32x8 a = to_f32(load8<T>(o + 8 * c)), b = to_f32(load8<T>(d + 8 * c));
-#pragma unroll
-    for (int t = 0; t < 8; ++t) acc += a[t] * b[t];
-  }
-  p.delta[idx] = acc;
-}
-
 // The workgroup's 256 threads load two [32 rows][32 channels] tiles (rows `pos0 ..` of tensors
 // a and b at (row i, head h)): thread t takes 8 channels of one row of one tile.
 template <typename T> struct TilePiece {
@@ -175,7 +159,19 @@ __global__ __launch_bounds__(256, (BwdCfg<T, VEC>::kMinWaves)) void attn_bwd_dq_
     dof[kk] = load8<T>((const T*)p.dout + elem(p, i, qi, h) + 16 * kk + 8 * g);
   }
   const float neg_mq = -p.lse[((int64_t)i * s + qi) * H + h];
-  const float neg_dq = -p.delta[((int64_t)i * s + qi) * H + h];
+  // Delta = sum_d O * dO of this lane's query, formed here (the lane holds half of the query's
+  // channels, the other half-wave the rest) and left in p.delta for the two kernels that follow
+  float delta = 0.0f;
+#pragma unroll
+  for (int kk = 0; kk < 2; ++kk) {
+    const f32x8 of = to_f32(load8<T>((const T*)p.o + elem(p, i, qi, h) + 16 * kk + 8 * g));
+    const f32x8 df = to_f32(dof[kk]);
+#pragma unroll
+    for (int t = 0; t < 8; ++t) delta += of[t] * df[t];
+  }
+  delta += swap32(delta);
+  if (g == 0 && q_ok) p.delta[((int64_t)i * s + qi) * H + h] = delta;
+  const float neg_dq = -delta;
   f32x16 acc;
 #pragma unroll
   for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
@@ -571,17 +567,15 @@ int triattn_bwd(const void* q, const void* k, const void* v, const void* b1, con
                 void* db2, float* delta, int n_rows, int s, int heads, hipStream_t stream) {
   if (n_rows == 0 || s == 0 || heads == 0) return 0;
   BwdParams p = {q, k, v, o, dout, b1, b2, lse, delta, dq, dk, dv, db2, n_rows, s, heads};
-  const int64_t total = (int64_t)n_rows * s * heads;
   const unsigned blocks = (unsigned)((s + 31) / 32);
-  attn_bwd_delta_kernel<T><<<dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream>>>(p);
   const dim3 walk((blocks + 3) / 4, heads, n_rows), pairs((blocks + 1) / 2, heads, (blocks + 1) / 2);
   if ((s & 7) == 0) {
+    attn_bwd_dq_kernel<T, true><<<walk, dim3(256), 0, stream>>>(p);   // (writes Delta: first)
     attn_bwd_kv_kernel<T, true><<<walk, dim3(256), 0, stream>>>(p);
-    attn_bwd_dq_kernel<T, true><<<walk, dim3(256), 0, stream>>>(p);
     if (db2) attn_bwd_db2_kernel<T, true><<<pairs, dim3(256), 0, stream>>>(p);
   } else {
-    attn_bwd_kv_kernel<T, false><<<walk, dim3(256), 0, stream>>>(p);
     attn_bwd_dq_kernel<T, false><<<walk, dim3(256), 0, stream>>>(p);
+    attn_bwd_kv_kernel<T, false><<<walk, dim3(256), 0, stream>>>(p);
     if (db2) attn_bwd_db2_kernel<T, false><<<pairs, dim3(256), 0, stream>>>(p);
   }
   return 0;
