@@ -151,6 +151,21 @@ __global__ __launch_bounds__(256, (BwdCfg<T, VEC>::kMinWaves)) void attn_bwd_dq_
   // branch would make every wait for memory a wait for all of it)
   const T* b1row = p.b1 ? (const T*)p.b1 + (int64_t)i * s : (const T*)p.b2 + (int64_t)h * s * s;
   const float b1on = p.b1 ? 1.0f : 0.0f;
+  // 16-bit: the biases reach the S^T accumulator on the matrix pipe, which these kernels leave
+  // idle four fifths of the time, instead of being converted and added on the vector ALU:
+  //   Bias2  S^T += E * B2, B2 the block's [key][query] values as they lie in LDS for this
+  //          lane's query (B operand: slots <-> keys), E the 0/1 matrix that sends key j to
+  //          the accumulator row that stands for it (row m <-> key perm_row(m));
+  //   Bias1  S^T += b * 1^T: Bias1 of the row's key in K slot 0 of one more product, against
+  //          a B operand with 1 in that slot (0 without a Bias1).  Products with 1 are exact.
+  constexpr bool MMB = sizeof(T) == 2;
+  V8 e_frag[2], one_frag;
+#pragma unroll
+  for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+    for (int t = 0; t < 8; ++t) e_frag[kk][t] = (T)(perm_row(ln) == 16 * kk + 8 * g + t ? 1.0f : 0.0f);
+#pragma unroll
+  for (int t = 0; t < 8; ++t) one_frag[t] = (T)(t == 0 && g == 0 ? b1on : 0.0f);
 
   V8 qf[2], dof[2];
 #pragma unroll
@@ -181,6 +196,7 @@ __global__ __launch_bounds__(256, (BwdCfg<T, VEC>::kMinWaves)) void attn_bwd_dq_
   // many cache lines per load as it has lanes, and the texture path was busy 96 % of the time).
   TilePiece<T> piece;
   V8 b1n[2], b2n[2];
+  T b1m = (T)0.0f;   // (16-bit) Bias1 of key perm_row(ln) of the block
   const int b2col = 8 * (tid & 3);
   const T* b2rows[2];
 #pragma unroll
@@ -200,8 +216,12 @@ __global__ __launch_bounds__(256, (BwdCfg<T, VEC>::kMinWaves)) void attn_bwd_dq_
     for (int j = 0; j < 2; ++j) store8<T>(&b2s[buf][(64 * j + (tid >> 2)) * kTP + b2col], b2n[j]);
   };
   auto fetch_bias = [&](int key0) {
+    if (MMB) {
+      b1m = b1row[min(key0 + perm_row(ln), s - 1)];
+    } else {
 #pragma unroll
-    for (int ks = 0; ks < 2; ++ks) b1n[ks] = load_bias8_raw<T>(b1row, key0 + 16 * ks + 8 * g, s, vec);
+      for (int ks = 0; ks < 2; ++ks) b1n[ks] = load_bias8_raw<T>(b1row, key0 + 16 * ks + 8 * g, s, vec);
+    }
     asm volatile("" ::: "memory");
   };
   // one block of 32 keys out of buffer `buf`; TAIL: the block holds keys beyond s.  The biases
@@ -218,21 +238,37 @@ __global__ __launch_bounds__(256, (BwdCfg<T, VEC>::kMinWaves)) void attn_bwd_dq_
     }
     f32x16 st, dp;
 #pragma unroll
-    for (int ks = 0; ks < 2; ++ks) {
-      const f32x8 b1f = to_f32(b1n[ks]);
-      const f32x8 b2f = to_f32(load8<T>(&b2s[buf][(32 * wave + ln) * kTP + 16 * ks + 8 * g]));
+    for (int r = 0; r < 16; ++r) dp[r] = neg_dq;
+    if constexpr (MMB) {
+      V8 b1a;
 #pragma unroll
-      for (int t = 0; t < 8; ++t) {
-        st[8 * ks + t] = b1f[t] * b1on + b2f[t];
-        dp[8 * ks + t] = neg_dq;
+      for (int t = 0; t < 8; ++t) b1a[t] = (T)0.0f;
+      b1a[0] = (g == 0 && b1on != 0.0f) ? b1m : (T)0.0f;
+      V8 b2v[2];
+#pragma unroll
+      for (int ks = 0; ks < 2; ++ks) b2v[ks] = load8<T>(&b2s[buf][(32 * wave + ln) * kTP + 16 * ks + 8 * g]);
+      fetch_bias(next_key0);
+#pragma unroll
+      for (int r = 0; r < 16; ++r) st[r] = 0.0f;
+#pragma unroll
+      for (int kk = 0; kk < 2; ++kk) mma32(st, kf[kk], qf[kk]);      // S^T[key][query]
+#pragma unroll
+      for (int kk = 0; kk < 2; ++kk) mma32(st, e_frag[kk], b2v[kk]);  // + Bias2
+      mma32(st, b1a, one_frag);                                        // + Bias1
+    } else {
+#pragma unroll
+      for (int ks = 0; ks < 2; ++ks) {
+        const f32x8 b1f = to_f32(b1n[ks]);
+        const f32x8 b2f = to_f32(load8<T>(&b2s[buf][(32 * wave + ln) * kTP + 16 * ks + 8 * g]));
+#pragma unroll
+        for (int t = 0; t < 8; ++t) st[8 * ks + t] = b1f[t] * b1on + b2f[t];
       }
-    }
-    fetch_bias(next_key0);
+      fetch_bias(next_key0);
 #pragma unroll
-    for (int kk = 0; kk < 2; ++kk) {
-      mma32(st, kf[kk], qf[kk]);    // S^T[key][query] (+ biases)
-      mma32(dp, vf[kk], dof[kk]);   // dP^T[key][query] - Delta
+      for (int kk = 0; kk < 2; ++kk) mma32(st, kf[kk], qf[kk]);    // S^T[key][query] (+ biases)
     }
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk) mma32(dp, vf[kk], dof[kk]);   // dP^T[key][query] - Delta
     V8 dsf[2];
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks) {
@@ -486,6 +522,17 @@ __global__ __launch_bounds__(256, (BwdCfg<T, VEC>::kMinWaves)) void attn_bwd_db2
   const int64_t row_elems = (int64_t)s * H * 32, row_stats = (int64_t)s * H;
   V8 piece[4], b1n[2];
   float mq_n = 0.0f, dq_n = 0.0f;
+  // 16-bit: Bias1 reaches the accumulator on the matrix pipe (see the dQ kernel): one value
+  // per lane, that of the key its accumulator row stands for, in K slot 0 of one more product
+  constexpr bool MMB = sizeof(T) == 2;
+  const unsigned off_b1m = min(key0 + perm_row(ln), s - 1);
+  T b1m_n = (T)0.0f;
+  V8 one_frag;
+#pragma unroll
+  for (int t = 0; t < 8; ++t) one_frag[t] = (T)(t == 0 && g == 0 ? b1on : 0.0f);
+  f32x16 b2acc;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) b2acc[r] = b2f[r >> 3][r & 7];
   auto fetch = [&](int i) {
     piece[0] = load8<T>((const T*)p.q + i * row_elems + off_q);
     piece[1] = load8<T>((const T*)p.dout + i * row_elems + off_q);
@@ -494,9 +541,13 @@ __global__ __launch_bounds__(256, (BwdCfg<T, VEC>::kMinWaves)) void attn_bwd_db2
     mq_n = (p.lse + i * row_stats)[off_stat];
     dq_n = (p.delta + i * row_stats)[off_stat];
     const T* b1row = b1base + i * b1pitch;
+    if (MMB) {
+      b1m_n = b1row[off_b1m];
+    } else {
 #pragma unroll
-    for (int ks = 0; ks < 2; ++ks)
-      b1n[ks] = vec ? load8<T>(b1row + off_b1[ks]) : load_bias8_raw<T>(b1row, key0 + 16 * ks + 8 * g, s, false);
+      for (int ks = 0; ks < 2; ++ks)
+        b1n[ks] = vec ? load8<T>(b1row + off_b1[ks]) : load_bias8_raw<T>(b1row, key0 + 16 * ks + 8 * g, s, false);
+    }
   };
   // Row i is computed out of buffer i % NB while row i + 1, fetched a step earlier, is parked
   // (two buffers: into the other one, which every wave left at the last barrier).
@@ -506,6 +557,7 @@ __global__ __launch_bounds__(256, (BwdCfg<T, VEC>::kMinWaves)) void attn_bwd_db2
   for (int w = 0; w < 4; ++w) store8<T>(&tiles[0][w][crow * kTP + cc], piece[w]);
   float neg_mq = -mq_n, neg_dq = -dq_n;
   V8 b1c[2] = {b1n[0], b1n[1]};
+  T b1m = b1m_n;
   __syncthreads();
   for (int i = 0; i < p.n_rows; ++i) {
     const int buf = i % NB;
@@ -513,12 +565,20 @@ __global__ __launch_bounds__(256, (BwdCfg<T, VEC>::kMinWaves)) void attn_bwd_db2
     asm volatile("" ::: "memory");   // the loads are issued here, a step ahead of their use
     f32x16 st, dp;
 #pragma unroll
-    for (int ks = 0; ks < 2; ++ks) {
-      const f32x8 b1f = to_f32(b1c[ks]);
+    for (int r = 0; r < 16; ++r) dp[r] = neg_dq;
+    if constexpr (MMB) {
+      V8 b1a;
 #pragma unroll
-      for (int t = 0; t < 8; ++t) {
-        st[8 * ks + t] = b1f[t] * b1on + b2f[ks][t];
-        dp[8 * ks + t] = neg_dq;
+      for (int t = 0; t < 8; ++t) b1a[t] = (T)0.0f;
+      b1a[0] = (g == 0 && b1on != 0.0f) ? b1m : (T)0.0f;
+      st = b2acc;
+      mma32(st, b1a, one_frag);   // Bias2 + Bias1
+    } else {
+#pragma unroll
+      for (int ks = 0; ks < 2; ++ks) {
+        const f32x8 b1f = to_f32(b1c[ks]);
+#pragma unroll
+        for (int t = 0; t < 8; ++t) st[8 * ks + t] = b1f[t] * b1on + b2f[ks][t];
       }
     }
 #pragma unroll
@@ -540,6 +600,7 @@ __global__ __launch_bounds__(256, (BwdCfg<T, VEC>::kMinWaves)) void attn_bwd_db2
     neg_dq = -dq_n;
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks) b1c[ks] = b1n[ks];
+    b1m = b1m_n;
     __syncthreads();
   }
   if (q_ok) {
