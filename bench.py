@@ -278,7 +278,7 @@ def main() -> int:
                     "bwd_frac_mfma": round(1280.0 * 768 ** 3 / (bm * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4),
                     "algorithmic": "backward: 5 products of 2 * 768^3 * 4 * 32 flop (dV, dP, dS^T Q, dS K, "
                                    "and the logits once); the kernels recompute the logits and dP in each of "
-                                   "three passes, 10 products executed",
+                                   "three passes, 10 products executed, and add the biases on the matrix pipe",
                     "workload": "TriAttentionFunction.apply + backward (dQ, dK, dV, dBias2); fwd_ms includes "
                                 "the scaling of Q and the repack of the operands into the core's tile order"}
                 del qkv, qo, ko, vo, do, b1o, b2o, oo
