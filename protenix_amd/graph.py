@@ -45,7 +45,7 @@ class Graphed:
         n = z.shape[-2]
         if pair_mask.numel() != n * n:
             return (False, None)      # a batch of masks: the general kernels
-        return (False, ops.padded_tail(pair_mask.view(n, n), n))
+        return (False, ops.padded_tail(pair_mask.reshape(n, n), n))
 
     @classmethod
     def _key(cls, s, z, pair_mask) -> tuple:

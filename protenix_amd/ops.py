@@ -183,7 +183,15 @@ prefix_mask_enabled = True
 prefix_mask_min_n = 600
 
 
-def _mask_key(mask: torch.Tensor) -> tuple:
+_CACHE_ENTRIES = 64      # masks kept per cache: a batch of pair masks has one entry per element
+
+
+def _mask_key(mask: torch.Tensor) -> Optional[tuple]:
+    """Identity of a mask's contents for the caches below, or None for a mask that cannot be
+    cached: a tensor made under torch.inference_mode() has no version counter, so an in-place
+    change of it would go unseen; such masks are converted and classified on every call."""
+    if mask.is_inference():
+        return None
     return (mask.untyped_storage().data_ptr(), mask.storage_offset(), tuple(mask.shape), tuple(mask.stride()),
             mask.dtype, mask.device, mask._version)
 
@@ -204,7 +212,7 @@ def mask_class(mask: Optional[torch.Tensor]) -> tuple:
     if mask.is_cuda and torch.cuda.is_current_stream_capturing():
         return capture_mask_class or (False, None)
     key = _mask_key(mask)
-    for i, (k, _, cls) in enumerate(_class_cache):
+    for i, (k, _, cls) in enumerate(_class_cache if key is not None else ()):
         if k == key:
             if i:
                 _class_cache.insert(0, _class_cache.pop(i))
@@ -219,8 +227,9 @@ def mask_class(mask: Optional[torch.Tensor]) -> tuple:
                   & ((row == 0) | (row == 1)).all() & ~steps)
         ones, prefix, nv = torch.stack([(mask == 1).all().float(), prefix.float(), nv]).tolist()
         cls = (bool(ones), int(nv) if prefix and 0 < int(nv) < mask.shape[0] else None)
-    _class_cache.insert(0, (key, mask, cls))
-    del _class_cache[8:]
+    if key is not None:
+        _class_cache.insert(0, (key, mask, cls))
+        del _class_cache[_CACHE_ENTRIES:]
     return cls
 
 
@@ -252,7 +261,10 @@ def _mask_for(mask: Optional[torch.Tensor], z: torch.Tensor, dtype: Optional[tor
     # "no mask", which spares the kernels its loads.
     if mask_class(mask)[0]:
         return None
-    key = _mask_key(mask) + (dtype, z.device, transpose)
+    key = _mask_key(mask)
+    if key is None:
+        return convert()
+    key = key + (dtype, z.device, transpose)
     for i, (k, _, out) in enumerate(_mask_cache):
         if k == key:
             if i:
@@ -260,7 +272,7 @@ def _mask_for(mask: Optional[torch.Tensor], z: torch.Tensor, dtype: Optional[tor
             return out
     out = convert()
     _mask_cache.insert(0, (key, mask, out))
-    del _mask_cache[8:]
+    del _mask_cache[2 * _CACHE_ENTRIES:]
     return out
 
 

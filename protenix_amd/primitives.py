@@ -14,7 +14,6 @@ from typing import Optional
 
 import torch
 import torch.nn as nn
-import torch.nn.functional as F
 
 from . import ops
 from .layer_norm import LayerNorm, _forward_only
@@ -37,6 +36,7 @@ class Linear(nn.Linear):
         self.precision = precision
         self.initializer = initializer
         super().__init__(in_features, out_features, bias=bias, device=device, dtype=dtype)
+        self._cache = _WeightCache()
         self._init_params()
 
     @torch.no_grad()
@@ -57,10 +57,25 @@ class Linear(nn.Linear):
             raise ValueError(f"Invalid initializer: {self.initializer}.")
 
     def forward(self, input: torch.Tensor) -> torch.Tensor:  # noqa: A002
-        d = input.dtype
-        cd = self.precision if self.precision is not None else d
-        b = self.bias.to(cd) if self.bias is not None else None
-        return F.linear(input.to(cd), self.weight.to(cd), b).to(d)
+        """primitives.py:83-98 on the HIP kernel of the single track: with `precision`, the
+        product is formed in that dtype (autocast ignored) and returned in the input's dtype;
+        without, in the input's dtype, or in the autocast dtype for an fp32 input under
+        torch.autocast (as F.linear would).  GPU tensors, float32 / bfloat16, in_features a
+        multiple of 16 and out_features of 8; anything else raises - no library GEMM stands in."""
+        _forward_only(input, module=self)
+        ops._dev(input, "input")
+        if self.precision is not None:
+            cd, od = self.precision, input.dtype
+        else:
+            cd = ops.autocast_compute_dtype(input) or input.dtype
+            od = cd
+        if cd not in (torch.float32, torch.bfloat16):
+            raise RuntimeError(f"protenix_amd.Linear: unsupported arithmetic dtype {cd} "
+                               "(float32 or bfloat16)")
+        w, b = self._cache.get((self.weight, self.bias), cd, input.device, lambda: (
+            _cv(self.weight, cd, input.device), _cv(self.bias, cd, input.device)))
+        out = ops.linear(input.to(cd), w, b)
+        return out if out.dtype == od else out.to(od)
 
 
 LinearNoBias = partial(Linear, bias=False)
@@ -98,7 +113,6 @@ class Transition(nn.Module):
         self.linear_no_bias = LinearNoBias(n * c_in, c_in, initializer="zeros")
         self._cache = _WeightCache()
         self._cache_ab = _WeightCache()
-        self._cache_lib = _WeightCache()
 
     def _weights(self, dtype, device) -> dict:
         ps = (self.layernorm1.weight, self.layernorm1.bias, self.linear_no_bias_a.weight,
@@ -138,28 +152,19 @@ class Transition(nn.Module):
             # the autocast dtype, like the reference's last linear)
             return out if (add or cd == x.dtype) else out.to(cd)
         # other widths (the single track, c_in = 384): HIP LayerNorm, SwiGLU and output kernels
+        if any(l.precision is not None for l in (self.linear_no_bias_a, self.linear_no_bias_b,
+                                                 self.linear_no_bias)):
+            raise RuntimeError("protenix_amd.Transition: linear layers with a `precision` override "
+                               "are not supported")
+        if not (self.c_in % 16 == 0 and (self.n * self.c_in) % 16 == 0
+                and x.dtype in (torch.float32, torch.bfloat16)):
+            raise RuntimeError(
+                f"protenix_amd.Transition: unsupported shape c_in={self.c_in} n={self.n} dtype={x.dtype} "
+                "(c_in a multiple of 16, float32 or bfloat16)")
         y = self.layernorm1(x)
-        plain = all(l.precision is None for l in (self.linear_no_bias_a, self.linear_no_bias_b,
-                                                  self.linear_no_bias))
-        if (plain and not torch.is_grad_enabled() and x.is_cuda and self.c_in % 16 == 0
-                and (self.n * self.c_in) % 16 == 0 and x.dtype in (torch.float32, torch.bfloat16)):
-            ps = (self.linear_no_bias_a.weight, self.linear_no_bias_b.weight, self.linear_no_bias.weight)
-            w_a, w_b, w_o = self._cache_ab.get(ps, y.dtype, y.device, lambda: tuple(
-                _cv(p, y.dtype, y.device) for p in ps))
-            h = ops.swiglu(y, w_a, w_b)
-            u = ops.linear(h, w_o, res=x if add else None)
-            return u if _residual_out is None else _residual_out.copy_(u)
-        # library GEMMs (a and b as one GEMM on the stacked weights)
-        if (not torch.is_grad_enabled() and self.linear_no_bias_a.precision is None
-                and self.linear_no_bias_b.precision is None):
-            ps = (self.linear_no_bias_a.weight, self.linear_no_bias_b.weight)
-            w_ab = self._cache_lib.get(ps, y.dtype, y.device, lambda: torch.cat(
-                [_cv(p, y.dtype, y.device) for p in ps], 0).contiguous())
-            a, b = F.linear(y, w_ab).chunk(2, dim=-1)
-            h = F.silu(a) * b
-        else:
-            h = F.silu(self.linear_no_bias_a(y)) * self.linear_no_bias_b(y)
-        u = self.linear_no_bias(h)
-        if _residual_out is not None:
-            return _residual_out.copy_(x + u) if _residual_out is not x else x.add_(u)
-        return x + u if add else u
+        ps = (self.linear_no_bias_a.weight, self.linear_no_bias_b.weight, self.linear_no_bias.weight)
+        w_a, w_b, w_o = self._cache_ab.get(ps, y.dtype, y.device, lambda: tuple(
+            _cv(p, y.dtype, y.device) for p in ps))
+        h = ops.swiglu(y, w_a, w_b)
+        u = ops.linear(h, w_o, res=x if add else None)
+        return u if _residual_out is None else _residual_out.copy_(u)

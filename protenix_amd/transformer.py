@@ -60,61 +60,58 @@ class Attention(nn.Module):
             return torch.cat([wq, wk, wg, wv], 0).contiguous(), bq
         return self._cache_in.get(ps, dtype, device, make)
 
-    def _hip_eligible(self, q_x: torch.Tensor, kv_x: torch.Tensor) -> bool:
-        plain = all(l is not None and l.precision is None for l in
-                    (self.linear_q, self.linear_k, self.linear_v, self.linear_g, self.linear_o))
-        return (q_x is kv_x and plain and q_x.is_cuda and self.c_q == self.c_k == self.c_v
-                and self.c_q % 16 == 0 and self.c_hidden % 8 == 0 and self.c_hidden <= 32
-                and q_x.dtype in (torch.float32, torch.bfloat16) and not torch.is_grad_enabled())
+    def _check_supported(self, q_x: torch.Tensor, kv_x: torch.Tensor) -> None:
+        """The HIP kernels cover self-attention with a gate on float32 / bfloat16 GPU tensors,
+        c_q a multiple of 16, head width 8, 16, 24 or 32 and 3 * heads * width a multiple of 32
+        (the transposed tail of the stacked projection).  Anything else raises: no library
+        GEMM or softmax stands in."""
+        why = None
+        if q_x is not kv_x:
+            why = "q_x and kv_x must be the same tensor (self-attention)"
+        elif any(l is None or l.precision is not None for l in
+                 (self.linear_q, self.linear_k, self.linear_v, self.linear_g, self.linear_o)):
+            why = "needs the gate and linear layers without a `precision` override"
+        elif not (self.c_q == self.c_k == self.c_v and self.c_q % 16 == 0):
+            why = f"c_q = c_k = c_v, a multiple of 16 (got {self.c_q}, {self.c_k}, {self.c_v})"
+        elif not (self.c_hidden % 8 == 0 and self.c_hidden <= 32
+                  and (3 * self.num_heads * self.c_hidden) % 32 == 0):
+            why = (f"head width 8, 16, 24 or 32 with 3 * heads * width a multiple of 32 "
+                   f"(got {self.num_heads} x {self.c_hidden})")
+        elif q_x.dtype not in (torch.float32, torch.bfloat16):
+            why = f"float32 or bfloat16 tensors (got {q_x.dtype})"
+        if why is not None:
+            raise RuntimeError(f"protenix_amd.Attention: unsupported configuration: {why}")
 
     def forward(self, q_x: torch.Tensor, kv_x: torch.Tensor,
                 attn_bias: Optional[torch.Tensor] = None, residual: Optional[torch.Tensor] = None,
                 **_unused) -> torch.Tensor:
         """Attention update of q_x; with `residual`, residual + update (added in the output
-        projection's epilogue)."""
+        projection's epilogue).  Three HIP kernels per batch element: stacked projection
+        (q | k | gate row-major, v transposed), flash-style attention with the pair bias and
+        the gate, output projection (+ residual).  Logits and softmax are fp32 and never
+        materialised (the reference upcasts q, k and the bias and relies on autocast for v,
+        primitives.py:255-270; here v is fp32 in the kernel as well)."""
+        _forward_only(q_x, attn_bias, residual, module=self)
+        ops._dev(q_x, "q_x")
+        self._check_supported(q_x, kv_x)
         H, d = self.num_heads, self.c_hidden
-        if self._hip_eligible(q_x, kv_x):
-            # Three HIP kernels per batch element: stacked projection (q | k | gate row-major,
-            # v transposed), flash-style attention with the pair bias and the gate, output
-            # projection (+ residual).  Logits and softmax are fp32 and never materialised.
-            w, bq = self._fused_in(q_x.dtype, q_x.device)
-            w_o = self._cache_out.get((self.linear_o.weight,), q_x.dtype, q_x.device,
-                                      lambda: _cv(self.linear_o.weight, q_x.dtype, q_x.device))
-            n, c = q_x.shape[-2], q_x.shape[-1]
-            xb = q_x.reshape(-1, n, c)
-            if not xb.is_contiguous():
-                xb = xb.contiguous()
-            bb = None
-            if attn_bias is not None:
-                bb = attn_bias.expand(*q_x.shape[:-2], H, n, n).reshape(-1, H, n, n)
-            outs = []
-            for i in range(xb.shape[0]):
-                qkg, vt = ops.linear_split(xb[i], w, bq, H * d, 3 * H * d)
-                outs.append(ops.single_attention(qkg, vt, None if bb is None else bb[i], H, d,
-                                                 1.0 / math.sqrt(d)))
-            o = outs[0] if len(outs) == 1 else torch.stack(outs)
-            return ops.linear(o.view(*q_x.shape[:-1], H * d), w_o, res=residual)
-        q = self.linear_q(q_x).unflatten(-1, (H, -1)).transpose(-2, -3)
-        k = self.linear_k(kv_x).unflatten(-1, (H, -1)).transpose(-2, -3)
-        v = self.linear_v(kv_x).unflatten(-1, (H, -1)).transpose(-2, -3)
-        q = q / math.sqrt(self.c_hidden)
-        # logits, softmax and the weighted sum in fp32 (the reference upcasts q, k
-        # and the bias and relies on autocast for v; here v is upcast as well)
-        dt = q.dtype
-        # (shielded from autocast, which would run both products in its own dtype again - as
-        # the reference shields its non-SDPA branch, primitives.py:269)
-        with torch.autocast("cuda", enabled=False):
-            w = torch.matmul(q.float(), k.float().transpose(-1, -2))
-            if attn_bias is not None:
-                if attn_bias.dim() != w.dim():
-                    attn_bias = attn_bias.unsqueeze(-3)
-                w = w + attn_bias.float()
-            w = torch.softmax(w, dim=-1)
-            o = torch.matmul(w, v.float()).to(dt).transpose(-2, -3)
-        if self.linear_g is not None:
-            o = o * torch.sigmoid(self.linear_g(q_x)).unflatten(-1, (H, -1))
-        out = self.linear_o(o.flatten(-2))
-        return out if residual is None else residual + out
+        w, bq = self._fused_in(q_x.dtype, q_x.device)
+        w_o = self._cache_out.get((self.linear_o.weight,), q_x.dtype, q_x.device,
+                                  lambda: _cv(self.linear_o.weight, q_x.dtype, q_x.device))
+        n, c = q_x.shape[-2], q_x.shape[-1]
+        xb = q_x.reshape(-1, n, c)
+        if not xb.is_contiguous():
+            xb = xb.contiguous()
+        bb = None
+        if attn_bias is not None:
+            bb = attn_bias.expand(*q_x.shape[:-2], H, n, n).reshape(-1, H, n, n)
+        outs = []
+        for i in range(xb.shape[0]):
+            qkg, vt = ops.linear_split(xb[i], w, bq, H * d, 3 * H * d)
+            outs.append(ops.single_attention(qkg, vt, None if bb is None else bb[i], H, d,
+                                             1.0 / math.sqrt(d)))
+        o = outs[0] if len(outs) == 1 else torch.stack(outs)
+        return ops.linear(o.view(*q_x.shape[:-1], H * d), w_o, res=residual)
 
 
 class AttentionPairBias(nn.Module):

@@ -154,4 +154,5 @@ def test_config5_stack_48_blocks_n2048_pad64():
     assert torch.isfinite(z_full).all() and torch.isfinite(s_full.float()).all()
     e = rel_err(z_crop, z_full)
     print(f"48 blocks, N = 2048, 64 padded: full vs cropped z {e:.2e}")
-    assert e <= TOL_BF16
+    # masked keys contribute exact zeros in the same summation order: bit for bit
+    assert torch.equal(z_crop.float().cpu(), z_full), f"padded keys leak: {e:.2e}"

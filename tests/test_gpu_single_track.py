@@ -11,7 +11,7 @@ import torch.nn.functional as F
 import protenix_amd as P
 from oracle import pairformer_oracle as O
 from protenix_amd import ops
-from tests.util import oracle_and_product, rel_err, tol
+from tests.util import TOL_BF16, oracle_and_product, rel_err, tol
 
 pytestmark = pytest.mark.gpu
 DTYPES = [torch.float32, torch.bfloat16]
@@ -118,6 +118,73 @@ def test_attention_pair_bias_module_runs_on_the_hip_kernels(dtype, n):
     assert {"layernorm", "swiglu", "linear"} <= seen
     assert rel_err(got, want) <= tol(dtype)
     assert rel_err(got_res, a.float() + want) <= tol(dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_linear_module_runs_on_the_hip_kernel(dtype):
+    """primitives.Linear called on its own (primitives.py:83-98): the HIP kernel, with and
+    without bias, with a `precision` override, on batched input, under autocast."""
+    x = _rand(3, 50, 384, dtype=dtype, seed=21)
+    for bias in (True, False):
+        lin = P.primitives.Linear(384, 136, bias=bias)
+        with torch.no_grad():
+            lin.weight.copy_(_rand(136, 384, dtype=dtype, seed=22, scale=1 / math.sqrt(384)).float())
+            if bias:
+                lin.bias.copy_(_rand(136, dtype=dtype, seed=23).float())
+        want = F.linear(x.float(), lin.weight.float(), lin.bias.float() if bias else None)
+        lin = lin.to("cuda", dtype).eval()
+        ops.kernel_timer = {}
+        try:
+            with torch.no_grad():
+                got = lin(x.cuda())
+            # frozen parameters, grad mode on: still the HIP kernel
+            lin.requires_grad_(False)
+            got2 = lin(x.cuda())
+            assert len(ops.kernel_timer.get("linear", ())) == 2
+        finally:
+            ops.kernel_timer = None
+        assert got.dtype == dtype and got.shape == (3, 50, 136)
+        assert rel_err(got, want) <= tol(dtype) and torch.equal(got, got2)
+    # precision override: fp32 product of a bf16 input, result in the input's dtype
+    lin = P.primitives.Linear(384, 136, bias=False, precision=torch.float32).to("cuda").eval()
+    with torch.no_grad():
+        y = lin(x.to(torch.bfloat16).cuda())
+        want = F.linear(x.to(torch.bfloat16).float(), lin.weight.float().cpu())
+    assert y.dtype == torch.bfloat16 and rel_err(y, want) <= TOL_BF16
+    # fp32 input and parameters under autocast: bf16 arithmetic and result, as F.linear gives
+    lin = P.primitives.Linear(384, 136).to("cuda").eval()
+    with torch.no_grad(), torch.autocast("cuda", dtype=torch.bfloat16):
+        y = lin(x.float().cuda())
+    assert y.dtype == torch.bfloat16
+    want = F.linear(x.float(), lin.weight.float().cpu(), lin.bias.float().cpu())
+    assert rel_err(y, want) <= TOL_BF16
+    with pytest.raises(RuntimeError, match="forward-only"):
+        P.primitives.Linear(384, 136).to("cuda")(x.float().cuda())
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_single_track_with_frozen_parameters_and_grad_mode_on(dtype):
+    """Eval mode with frozen parameters outside torch.no_grad(): the same HIP kernels and the
+    same bits as under no_grad (there is no second implementation to fall into)."""
+    n = 100
+    ref, prod = oracle_and_product(O.AttentionPairBias, P.AttentionPairBias, has_s=False,
+                                   create_offset_ln_z=True, n_heads=16, c_a=384, c_z=128, dtype=dtype)
+    reft, prodt = oracle_and_product(O.Transition, P.Transition, 384, 4, dtype=dtype)
+    g = torch.Generator().manual_seed(3)
+    a, z = torch.randn(1, n, 384, generator=g).to(dtype), torch.randn(1, n, n, 128, generator=g).to(dtype)
+    with torch.no_grad():
+        want, want_t = prod(a.cuda(), None, z.cuda()), prodt(a.cuda())
+    prod.requires_grad_(False)
+    prodt.requires_grad_(False)
+    assert torch.is_grad_enabled()
+    ops.kernel_timer = {}
+    try:
+        got, got_t = prod(a.cuda(), None, z.cuda()), prodt(a.cuda())
+        seen = set(ops.kernel_timer)
+    finally:
+        ops.kernel_timer = None
+    assert {"pair_bias", "layernorm", "linear", "single_attention", "swiglu"} <= seen
+    assert torch.equal(got, want) and torch.equal(got_t, want_t)
 
 
 def test_refusals():

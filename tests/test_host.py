@@ -198,3 +198,65 @@ def test_mask_class_finds_a_padded_tail_and_nothing_else():
         assert ops.padded_tail(outer(hole), 8) is None
     finally:
         ops.prefix_mask_min_n = keep
+
+
+def test_mask_class_takes_inference_mode_masks_and_large_batches():
+    """A mask made under torch.inference_mode() has no version counter: it is classified on
+    every call instead of being cached (an in-place change of it could not be noticed), and
+    the caches hold every element of a batch of masks larger than eight."""
+    import torch
+    from protenix_amd import ops
+
+    with torch.inference_mode():
+        v = torch.ones(8)
+        v[6:] = 0
+        m = v[:, None] * v[None, :]
+        assert m.is_inference()
+        assert ops.mask_class(m) == (False, 6)
+        m[:, 5:] = 0
+        m[5:, :] = 0
+        assert ops.mask_class(m) == (False, 5)
+        z = torch.zeros(8, 8, 4)
+        out = ops._mask_for(m, z, torch.float32, transpose=True)
+        assert out.dtype == torch.float32 and torch.equal(out, m.t())
+    # a batch of 12 masks, looked at twice: the second look finds every entry
+    batch = torch.ones(12, 8, 8)
+    for i in range(12):
+        batch[i, :, 8 - i % 4 - 1:] = 0
+        batch[i, 8 - i % 4 - 1:, :] = 0
+    first = [ops.mask_class(batch[i]) for i in range(12)]
+    assert first == [(False, 8 - i % 4 - 1) for i in range(12)]
+    keys = {ops._mask_key(batch[i]) for i in range(12)}
+    assert keys <= {k for k, _, _ in ops._class_cache}
+
+
+def test_modules_refuse_what_the_kernels_do_not_cover_instead_of_falling_back():
+    """No library GEMM or softmax stands in for a HIP kernel: CPU tensors, a `precision`
+    override inside the fused modules, unsupported head shapes and cross-attention raise."""
+    import pytest
+    import torch
+    import protenix_amd as P
+    from protenix_amd.primitives import Linear, Transition
+    from protenix_amd.transformer import Attention
+
+    with torch.no_grad():
+        with pytest.raises(RuntimeError, match="no CPU fallback"):
+            Linear(16, 8)(torch.zeros(4, 16))
+        with pytest.raises(RuntimeError, match="no CPU fallback"):
+            Attention(32, 32, 32, 8, 4).eval()(torch.zeros(4, 32), torch.zeros(4, 32))
+        att = Attention(48, 48, 48, 24, 2).eval()       # 3 * 2 * 24 = 144: not a multiple of 32
+        x = torch.zeros(4, 48)
+        with pytest.raises(RuntimeError, match="unsupported configuration"):
+            att._check_supported(x, x)
+        with pytest.raises(RuntimeError, match="self-attention"):
+            Attention(32, 32, 32, 8, 4)._check_supported(x, x.clone())
+        Attention(384, 384, 384, 24, 16)._check_supported(x, x)      # the block's own shape
+        tr = Transition(384, 4).eval()
+        tr.linear_no_bias_a.precision = torch.float32
+        with pytest.raises(RuntimeError, match="precision"):
+            tr(torch.zeros(4, 384))
+    import inspect
+    from protenix_amd import primitives, transformer
+    for mod in (primitives, transformer):
+        src = inspect.getsource(mod)
+        assert "torch.nn.functional" not in src and "torch.softmax(" not in src and "torch.matmul(" not in src
