@@ -368,6 +368,15 @@ PTX_API int ptx_single_attention_fwd(const void* q, const void* k, const void* v
                    const void* bias, int bias_f32, void* out, int n, int heads, int d, int64_t ld,
                    int64_t ldt, int64_t ldo, float scale, int dtype, void* stream);
 
+/*
+ * Measurement aid with no counterpart in the reference: streams `bytes` (a multiple of 16)
+ * through the GPU with plain 16-byte accesses - a copy (src and dst), a read-only pass (dst
+ * NULL) or a write-only pass (src NULL), with non-temporal accesses when nontemporal = 1.  Its
+ * rate on a tensor of a kernel's size is the ceiling that kernel's achieved HBM bandwidth is
+ * reported against (bench.py, `hbm_ceiling`); src and dst must not overlap.
+ */
+PTX_API int ptx_hbm_stream(const void* src, void* dst, int64_t bytes, int nontemporal, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

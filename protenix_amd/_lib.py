@@ -52,6 +52,7 @@ SIGNATURES = {
     "ptx_swiglu_fwd": (_i, [_p, _p, _p, _p, _i, _i, _i, _i, _p]),
     "ptx_single_attention_fwd": (_i, [_p, _p, _p, _p, _p, _i, _p, _i, _i, _i, _l, _l, _l, _f, _i, _p]),
     "ptx_pair_bias_fwd": (_i, [_p] * 5 + [_i, _i, _i, _i, _f, _i, _p]),
+    "ptx_hbm_stream": (_i, [_p, _p, _l, _i, _p]),
 }
 
 _lock = threading.Lock()

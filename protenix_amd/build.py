@@ -14,7 +14,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libprotenix_amd.so")
-SOURCES = ["api.hip", "layernorm.hip", "rowgemm.hip", "triattn.hip", "attnpack.hip", "attnbwd.hip", "attnout.hip", "ntgemm.hip", "transition.hip", "single.hip"]
+SOURCES = ["api.hip", "layernorm.hip", "rowgemm.hip", "triattn.hip", "attnpack.hip", "attnbwd.hip", "attnout.hip", "ntgemm.hip", "transition.hip", "single.hip", "stream.hip"]
 # per-source extra flags (none: the attention core's redo checks of the form !(x < limit) are
 # what catches a NaN logit, so it is built with NaNs honoured like everything else)
 EXTRA_FLAGS = {}

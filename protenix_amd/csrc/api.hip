@@ -624,4 +624,16 @@ PTX_API int ptx_pair_bias_fwd(const void* z, const void* ln_w, const void* ln_b,
   return after_launch("pair_bias");
 }
 
+PTX_API int ptx_hbm_stream(const void* src, void* dst, int64_t bytes, int nontemporal, void* stream) {
+  PTX_REQUIRE(bytes >= 0 && bytes % 16 == 0, PTX_ERR_BAD_ARG,
+              "hbm_stream: bytes=%lld must be a non-negative multiple of 16", (long long)bytes);
+  PTX_REQUIRE(bytes <= ((int64_t)1 << 40), PTX_ERR_UNSUPPORTED, "hbm_stream: more than 1 TiB");
+  if (bytes == 0) return PTX_OK;
+  PTX_REQUIRE(src || dst, PTX_ERR_BAD_ARG, "hbm_stream: src and dst are both null");
+  PTX_REQUIRE(aligned16(src) && aligned16(dst), PTX_ERR_BAD_ARG,
+              "hbm_stream: pointers must be 16-byte aligned");
+  ptx::hbm_stream(src, dst, bytes, nontemporal, (hipStream_t)stream);
+  return after_launch("hbm_stream");
+}
+
 }  // extern "C"

@@ -119,4 +119,7 @@ int triattn_bwd(const void* q, const void* k, const void* v, const void* b1, con
                 const void* o, const float* lse, const void* dout, void* dq, void* dk, void* dv,
                 void* db2, float* delta, int n_rows, int s, int heads, hipStream_t stream);
 
+// Streams `bytes` (a multiple of 16) from src to dst; src null: write-only, dst null: read-only.
+int hbm_stream(const void* src, void* dst, int64_t bytes, int nontemporal, hipStream_t stream);
+
 }  // namespace ptx

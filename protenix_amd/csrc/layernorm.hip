@@ -34,7 +34,13 @@ __device__ __forceinline__ float group_sum(float v) {
   return v;
 }
 
-template <typename T, int VEC, int G, int NCHUNK, int UNROLL>
+// HOIST: gamma and beta of the lane's columns are read once, before the rows (short rows: a
+// load per row and vector otherwise, more load instructions than the rows themselves need).
+// NT: rows are read and written with non-temporal accesses (tensors that do not fit the
+// memory-side cache anyway).  Waves walk over row batches with a grid stride and request the
+// next batch before they work on the current one; with one batch per wave that is a plain
+// one-shot kernel.
+template <typename T, int VEC, int G, int NCHUNK, int UNROLL, bool HOIST, bool NT>
 __global__ __launch_bounds__(256) void layernorm_fwd_kernel(
     const T* __restrict__ x, const T* __restrict__ gamma, const T* __restrict__ beta,
     T* __restrict__ y, float* __restrict__ mean_out, float* __restrict__ rstd_out, int64_t rows,
@@ -46,72 +52,121 @@ __global__ __launch_bounds__(256) void layernorm_fwd_kernel(
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int sub = lane % G;   // lane within the row group
   const int grp = lane / G;   // which row of the wave's batch
-  const int64_t row0 = ((int64_t)blockIdx.x * (blockDim.x >> 6) + wave) * ROWS_PER_WAVE;
   const float inv_n = 1.0f / (float)cols;
+  const int64_t n_batches = (rows + ROWS_PER_WAVE - 1) / ROWS_PER_WAVE;
+  const int64_t stride = (int64_t)gridDim.x * (blockDim.x >> 6);
+  int64_t batch = (int64_t)blockIdx.x * (blockDim.x >> 6) + wave;
+  if (batch >= n_batches) return;
 
-  F v[UNROLL][NCHUNK];
-#pragma unroll
-  for (int u = 0; u < UNROLL; ++u) {
-    const int64_t row = row0 + (int64_t)u * (kWave / G) + grp;
+  F gm[HOIST ? NCHUNK : 1], bt[HOIST ? NCHUNK : 1];
+  if (HOIST) {
 #pragma unroll
     for (int c = 0; c < NCHUNK; ++c) {
       const int col = (c * G + sub) * VEC;
-      if (row < rows && col < cols) {
-        v[u][c] = __builtin_convertvector(*reinterpret_cast<const V*>(x + row * cols + col), F);
-      } else {
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) v[u][c][e] = 0.0f;
+      for (int e = 0; e < VEC; ++e) {
+        gm[c][e] = 1.0f;
+        bt[c][e] = 0.0f;
+      }
+      if (col < cols) {
+        if (gamma) gm[c] = __builtin_convertvector(*reinterpret_cast<const V*>(gamma + col), F);
+        if (beta) bt[c] = __builtin_convertvector(*reinterpret_cast<const V*>(beta + col), F);
       }
     }
   }
+
+  // raw rows of one batch: rows and columns beyond the end repeat the last valid ones (their
+  // values are masked where they are used), so the loads themselves are unconditional
+  auto load = [&](V (&r)[UNROLL][NCHUNK], int64_t b) {
 #pragma unroll
-  for (int u = 0; u < UNROLL; ++u) {
-    const int64_t row = row0 + (int64_t)u * (kWave / G) + grp;
-    float s = 0.0f;
+    for (int u = 0; u < UNROLL; ++u) {
+      int64_t row = b * ROWS_PER_WAVE + (int64_t)u * (kWave / G) + grp;
+      row = row < rows ? row : rows - 1;
 #pragma unroll
-    for (int c = 0; c < NCHUNK; ++c)
+      for (int c = 0; c < NCHUNK; ++c) {
+        int col = (c * G + sub) * VEC;
+        col = col < cols ? col : 0;
+        const V* p = reinterpret_cast<const V*>(x + row * cols + col);
+        r[u][c] = NT ? __builtin_nontemporal_load(p) : *p;
+      }
+    }
+  };
+  auto work = [&](const V (&r)[UNROLL][NCHUNK], int64_t b) {
 #pragma unroll
-      for (int e = 0; e < VEC; ++e) s += v[u][c][e];
-    const float mean = group_sum<G>(s) * inv_n;
-    float q = 0.0f;
+    for (int u = 0; u < UNROLL; ++u) {
+      const int64_t row = b * ROWS_PER_WAVE + (int64_t)u * (kWave / G) + grp;
+      F v[NCHUNK];
+      float s = 0.0f;
 #pragma unroll
-    for (int c = 0; c < NCHUNK; ++c) {
-      const int col = (c * G + sub) * VEC;
-      if (col < cols) {
+      for (int c = 0; c < NCHUNK; ++c) {
+        v[c] = __builtin_convertvector(r[u][c], F);
+        if ((c * G + sub) * VEC < cols) {
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) {
-          const float d = v[u][c][e] - mean;
-          q += d * d;
+          for (int e = 0; e < VEC; ++e) s += v[c][e];
+        }
+      }
+      const float mean = group_sum<G>(s) * inv_n;
+      float q = 0.0f;
+#pragma unroll
+      for (int c = 0; c < NCHUNK; ++c) {
+        if ((c * G + sub) * VEC < cols) {
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) {
+            const float d = v[c][e] - mean;
+            q += d * d;
+          }
+        }
+      }
+      const float var = group_sum<G>(q) * inv_n;
+      const float rstd = rsqrtf(fmaxf(var, 0.0f) + eps);
+      if (row < rows) {
+        if (sub == 0) {
+          if (mean_out) mean_out[row] = mean;
+          if (rstd_out) rstd_out[row] = rstd;
+        }
+#pragma unroll
+        for (int c = 0; c < NCHUNK; ++c) {
+          const int col = (c * G + sub) * VEC;
+          if (col < cols) {
+            F o;
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) o[e] = (v[c][e] - mean) * rstd;
+            if (HOIST) {
+#pragma unroll
+              for (int e = 0; e < VEC; ++e) o[e] = o[e] * gm[c][e] + bt[c][e];
+            } else {
+              if (gamma) {
+                F g1 = __builtin_convertvector(*reinterpret_cast<const V*>(gamma + col), F);
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) o[e] *= g1[e];
+              }
+              if (beta) {
+                F b1 = __builtin_convertvector(*reinterpret_cast<const V*>(beta + col), F);
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) o[e] += b1[e];
+              }
+            }
+            V* p = reinterpret_cast<V*>(y + row * cols + col);
+            const V ov = __builtin_convertvector(o, V);
+            if (NT) __builtin_nontemporal_store(ov, p); else *p = ov;
+          }
         }
       }
     }
-    const float var = group_sum<G>(q) * inv_n;
-    const float rstd = rsqrtf(fmaxf(var, 0.0f) + eps);
-    if (row < rows) {
-      if (sub == 0) {
-        if (mean_out) mean_out[row] = mean;
-        if (rstd_out) rstd_out[row] = rstd;
-      }
+  };
+
+  V cur[UNROLL][NCHUNK];
+  load(cur, batch);
+  for (; batch < n_batches; batch += stride) {
+    const bool more = batch + stride < n_batches;
+    V nxt[UNROLL][NCHUNK];
+    if (more) load(nxt, batch + stride);
+    work(cur, batch);
+    if (more) {
 #pragma unroll
-      for (int c = 0; c < NCHUNK; ++c) {
-        const int col = (c * G + sub) * VEC;
-        if (col < cols) {
-          F o;
+      for (int u = 0; u < UNROLL; ++u)
 #pragma unroll
-          for (int e = 0; e < VEC; ++e) o[e] = (v[u][c][e] - mean) * rstd;
-          if (gamma) {
-            F gm = __builtin_convertvector(*reinterpret_cast<const V*>(gamma + col), F);
-#pragma unroll
-            for (int e = 0; e < VEC; ++e) o[e] *= gm[e];
-          }
-          if (beta) {
-            F bt = __builtin_convertvector(*reinterpret_cast<const V*>(beta + col), F);
-#pragma unroll
-            for (int e = 0; e < VEC; ++e) o[e] += bt[e];
-          }
-          *reinterpret_cast<V*>(y + row * cols + col) = __builtin_convertvector(o, V);
-        }
-      }
+        for (int c = 0; c < NCHUNK; ++c) cur[u][c] = nxt[u][c];
     }
   }
 }
@@ -148,16 +203,33 @@ __global__ __launch_bounds__(256) void layernorm_fwd_long_kernel(
   }
 }
 
+// Tensors whose read + write traffic exceeds this are streamed with non-temporal accesses:
+// measured on [768^2, 128], fp32 rows (604 MB of traffic, more than the 256 MB memory-side
+// cache holds) 0.101 -> 0.095 ms, bf16 rows (302 MB) no gain.
+constexpr int64_t kLnNonTemporalBytes = (int64_t)384 << 20;
+
 template <typename T, int VEC, int G, int NCHUNK>
 static void launch_ln(const T* x, const T* gamma, const T* beta, T* y, float* mean, float* rstd,
                       int64_t rows, int cols, float eps, hipStream_t stream) {
-  // (rows in flight per lane group; measured: 16-bit rows of one vector per lane run 30 %
-  // faster with 2 than with 4, 32-bit rows the other way round)
-  constexpr int UNROLL = (NCHUNK * VEC * (int)sizeof(T) <= 16) ? (sizeof(T) == 2 ? 2 : 4) : (NCHUNK <= 2 ? 2 : 1);
+  // Row groups in flight per lane group, and how the grid is formed.  Measured on [768^2, 128]:
+  // 16-bit rows of one vector per lane are fastest as 16 workgroups per compute unit whose waves
+  // walk over batches of 2 row groups with the next batch requested ahead (0.047 ms against
+  // 0.050 one-shot with 4 row groups, 0.051 with 2); 32-bit rows as a one-shot grid with 4 row
+  // groups per wave (persistent: 0.101 against 0.095 ms).
+  constexpr bool SHORT = NCHUNK * VEC * (int)sizeof(T) <= 16;
+  constexpr int UNROLL = SHORT ? (sizeof(T) == 2 ? 2 : 4) : (NCHUNK <= 2 ? 2 : 1);
+  constexpr bool HOIST = NCHUNK * VEC <= 16;
   constexpr int ROWS_PER_BLOCK = 4 * (kWave / G) * UNROLL;
-  const int64_t blocks = (rows + ROWS_PER_BLOCK - 1) / ROWS_PER_BLOCK;
-  layernorm_fwd_kernel<T, VEC, G, NCHUNK, UNROLL>
-      <<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(x, gamma, beta, y, mean, rstd, rows, cols, eps);
+  int64_t blocks = (rows + ROWS_PER_BLOCK - 1) / ROWS_PER_BLOCK;
+  if (sizeof(T) == 2 && SHORT) blocks = std::min<int64_t>(blocks, 16 * 256);
+  blocks = std::min<int64_t>(blocks, 0x7fffffff);
+  const bool nt = 2 * rows * (int64_t)cols * (int64_t)sizeof(T) > kLnNonTemporalBytes;
+  if (nt)
+    layernorm_fwd_kernel<T, VEC, G, NCHUNK, UNROLL, HOIST, true>
+        <<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(x, gamma, beta, y, mean, rstd, rows, cols, eps);
+  else
+    layernorm_fwd_kernel<T, VEC, G, NCHUNK, UNROLL, HOIST, false>
+        <<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(x, gamma, beta, y, mean, rstd, rows, cols, eps);
 }
 
 template <typename T, int VEC>
@@ -170,7 +242,7 @@ static bool dispatch_ln_vec(const T* x, const T* gamma, const T* beta, T* y, flo
     return true;                                                                            \
   }
   PTX_LN_CASE(1, 1) PTX_LN_CASE(2, 1) PTX_LN_CASE(4, 1) PTX_LN_CASE(8, 1) PTX_LN_CASE(16, 1)
-  PTX_LN_CASE(16, 2) PTX_LN_CASE(16, 3) PTX_LN_CASE(64, 1) PTX_LN_CASE(64, 2) PTX_LN_CASE(64, 4)
+  PTX_LN_CASE(32, 1) PTX_LN_CASE(16, 2) PTX_LN_CASE(16, 3) PTX_LN_CASE(64, 1) PTX_LN_CASE(64, 2) PTX_LN_CASE(64, 4)
   PTX_LN_CASE(64, 8)
 #undef PTX_LN_CASE
   return false;

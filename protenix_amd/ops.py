@@ -351,8 +351,9 @@ def triangle_attention(z: torch.Tensor, mask: Optional[torch.Tensor], w: dict, h
             # mask = m (x) m, padding at the end: the valid rows attend the valid keys with no
             # mask at all (a masked key of such a row has weight exactly zero in the reference);
             # the padded rows, all of whose keys are masked, go through the masked path
-            for rows, mk, nk in (((0, n_valid), None, n_valid), ((n_valid, n - n_valid), mask, n)):
-                _call("triattn_fwd", lib.ptx_triattn_fwd_rows, _ptr(q), _ptr(k), _ptr(vt),
+            for name, rows, mk, nk in (("triattn_fwd", (0, n_valid), None, n_valid),
+                                       ("triattn_fwd_padded_rows", (n_valid, n - n_valid), mask, n)):
+                _call(name, lib.ptx_triattn_fwd_rows, _ptr(q), _ptr(k), _ptr(vt),
                       None if late_gate else _ptr(g), _ptr(tb), _ptr(mk), _ptr(g), n, heads, d, pitch,
                       0, float(inf), rows[0], rows[1], nk, dt, st)
         else:
@@ -508,3 +509,19 @@ def single_attention(qkg: torch.Tensor, vt: torch.Tensor, bias: Optional[torch.T
               int(bias is not None and bias.dtype == torch.float32),
               _ptr(out), n, heads, d, qkg.shape[1], vt.shape[1], hd, float(scale), _dt(qkg), _stream())
     return out
+
+
+# ---------------------------------------------------------------- measurement aid
+def hbm_stream(src: Optional[torch.Tensor], dst: Optional[torch.Tensor], nontemporal: bool = False) -> None:
+    """One streaming pass with plain 16-byte accesses: copy src -> dst, read src only (dst None) or
+    write dst only (src None); the rate of such a pass is the ceiling an HBM-bound kernel of the
+    same size is reported against."""
+    t = src if src is not None else dst
+    _dev(t, "src" if src is not None else "dst")
+    if src is not None and dst is not None and src.numel() * src.element_size() != dst.numel() * dst.element_size():
+        raise RuntimeError("hbm_stream: src and dst differ in size")
+    if not all(x is None or x.is_contiguous() for x in (src, dst)):
+        raise RuntimeError("hbm_stream: tensors must be contiguous")
+    with torch.cuda.device(t.device):
+        _call("hbm_stream", _lib.load().ptx_hbm_stream, _ptr(src), _ptr(dst), t.numel() * t.element_size(),
+              int(nontemporal), _stream())
