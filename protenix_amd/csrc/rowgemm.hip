@@ -260,7 +260,8 @@ rowgemm_in_kernel(RowGemmInParams p) {
     }
   };
   // (the first tile's rows go first: their LayerNorm then runs while the weights arrive)
-  if (kPrefetch && tile < n_tiles) issue_rows(tile);
+  if (kPrefetch) issue_rows(tile < n_tiles ? tile : n_tiles - 1);
+  RowFrags<T, RB, KS> xf;   // the tile's normalised rows (kPrefetch: carried from tile to tile)
   // (A wait for the resident weights deferred to the first tile's first chunk, so that they
   // would travel under that tile's row loads, was tried: the conditional barrier inside the
   // tile loop cost the triangle-multiplication output 848 bytes of spills per lane.)
@@ -272,6 +273,22 @@ rowgemm_in_kernel(RowGemmInParams p) {
     for (int j = 0; j < FPW; ++j) dma_frag(wave * FPW + j, wave * FPW + j);
     ring_barrier<0>();
   }
+
+  // kPrefetch: a tile's rows are normalised at the END of the tile before it, in the iteration
+  // that requested them.  The wait for them then stands in straight-line code (the chunk loop
+  // of this instantiation is unrolled) behind a number of stores the compiler can count, and
+  // leaves those in flight: memory operations of a wave complete in order, and for a wait at the
+  // head of the next iteration the compiler has to assume that nothing was issued behind the
+  // loads, which drained every store of the tile there (181 -> 170 us per launch at N = 768).
+  auto normalize_prefetched = [&]() {
+    if constexpr (kPrefetch) {
+      f32x8 v[KS];
+#pragma unroll
+      for (int kk = 0; kk < KS; ++kk) v[kk] = to_f32(raw[kk]);
+      normalize_row<T, KS, float, false>(v, lds_affine[0], lds_affine[1], p.eps, lane >> 5, xf.f[0]);
+    }
+  };
+  normalize_prefetched();
 
   // Staged path (fp32; bf16 rows of 256 channels): the next chunk's fragments are prefetched
   // into registers and stored to LDS
@@ -330,7 +347,6 @@ rowgemm_in_kernel(RowGemmInParams p) {
     const T* beta2 = (const T*)p.beta2;
     if constexpr (RES) asm volatile("" : "+s"(gamma), "+s"(beta), "+s"(gamma2), "+s"(beta2));
 
-  RowFrags<T, RB, KS> xf;
   // (the raw rows in their storage type: fp32 rows as fp32, bf16 rows as bf16 - half the registers)
   typename Vec8<TZ>::type zres[kRegRes ? RB : 1][kRegRes ? KS : 1];
   if constexpr (MODE == kTriMulIn) {
@@ -359,10 +375,7 @@ rowgemm_in_kernel(RowGemmInParams p) {
     }
   } else {
     if constexpr (kPrefetch) {
-      f32x8 v[KS];
-#pragma unroll
-      for (int kk = 0; kk < KS; ++kk) v[kk] = to_f32(raw[kk]);
-      normalize_row<T, KS, float, false>(v, lds_affine[0], lds_affine[1], p.eps, g, xf.f[0]);
+      // the next tile's rows, normalised at the end of this iteration
       // (no branch around the loads: with one, this instantiation spills.  A wave past its
       // last tile reads the rows every such wave reads, out of the L2.)
       const int64_t nt = tile + tile_step;
@@ -890,9 +903,17 @@ rowgemm_in_kernel(RowGemmInParams p) {
       __syncthreads();
     }
   };
+  if constexpr (kPrefetch) {
+    // (unrolled: the stores between the request for the next rows and the wait for them are
+    // then a count the compiler knows)
+#pragma unroll
+    for (int ch = 0; ch < nch; ++ch) chunk_body(ch);
+  } else {
 #pragma clang loop unroll(disable)
-  for (int ch = 0; ch < nch; ++ch) chunk_body(ch);
+    for (int ch = 0; ch < nch; ++ch) chunk_body(ch);
+  }
     if (!RES) break;
+    normalize_prefetched();
     tile += tile_step;
   }
 }

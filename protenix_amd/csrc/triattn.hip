@@ -72,7 +72,7 @@ struct AttnAux {
 // n_keys set to -inf (kMaskTail; kMaskNone where the keys fill whole tiles).
 enum { kMaskNone = 0, kMaskTail = 1, kMaskGiven = 2 };
 template <typename T, int R, int NWQ, int MK>
-__global__ __launch_bounds__((NWQ * 64), (sizeof(T) == 2 ? (R == 1 ? 16 / NWQ : (NWQ == 8 ? 2 : 3)) : 2)) void triattn_fwd_kernel(
+__global__ __launch_bounds__((NWQ * 64), (sizeof(T) == 2 ? (R == 1 ? 16 / NWQ : (NWQ == 8 ? (MK == kMaskTail ? 4 : 2) : 3)) : 2)) void triattn_fwd_kernel(
     const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ vt,
     const T* gate, const T* __restrict__ bias, const T* __restrict__ mask,
     T* o, int n, int heads, int key_pitch, int mask_transposed, float inf,
@@ -480,16 +480,16 @@ int triattn_fwd_ex(const T* q, const T* k, const T* vt, const T* g, const T* tri
   // -2.2 % at 2048), where their 256 queries divide n or n is large enough for the idle waves
   // of the last one not to matter
   const bool wide = sizeof(T) == 2 && ((n % 256 == 0 && n >= 1536) || n >= 2048);
-  // Two rows per wave, in 8-wave workgroups (16-bit, whole key tiles, no mask): the two rows
+  // Two rows per wave, in 8-wave workgroups (16-bit, no mask): the two rows
   // share the query block and with it the bias tile - one load and one conversion per logit for
   // both, half the bias stream from the L2 - at 123 registers, so that four waves still share a
-  // SIMD (with a mask or a partial tile the kernel needs 131 to 160 and loses a wave; with four
-  // waves per workgroup the K / V tiles of two rows leave room for three workgroups only: no
-  // gain).  Per launch: 395 -> 356 us at n = 768 in the trunk; in a loop of attention updates
+  // SIMD (with a partial last key tile the register allocator is held to 128 by the kernel's
+  // launch bounds and gets there without spills; with a mask the kernel needs 160 and loses a
+  // wave; with four waves per workgroup the K / V tiles of two rows leave room for three
+  // workgroups only: no gain).  Per launch: 395 -> 356 us at n = 768 in the trunk; in a loop of attention updates
   // -7 % at n = 512, -3 % at 768, -11 % at 1536, -13 % at 2048, but +10 to +25 % where 256
   // queries do not divide n (256, 384, 640) and waves of the last workgroup idle.
-  const bool r2 = sizeof(T) == 2 && !mask && n_keys % kKeyTile == 0 && n % 256 == 0 && n >= 512 &&
-                  row_count >= 2;
+  const bool r2 = sizeof(T) == 2 && !mask && n % 256 == 0 && n >= 512 && row_count >= 2;
   const int n_qtiles = (wide || r2) ? (n + 255) / 256 : (n + 127) / 128;
   const int R = r2 ? 2 : 1;
   const int n_rowgroups = (row_count + R - 1) / R;
@@ -503,7 +503,8 @@ int triattn_fwd_ex(const T* q, const T* k, const T* vt, const T* g, const T* tri
 #define PTX_ATTN_LAUNCH(NWQ, MK) PTX_ATTN_LAUNCH_R(1, NWQ, MK)
   if (r2) {
     if constexpr (sizeof(T) == 2) {
-      PTX_ATTN_LAUNCH_R(2, 8, kMaskNone);
+      if (mk == kMaskTail) PTX_ATTN_LAUNCH_R(2, 8, kMaskTail);
+      else PTX_ATTN_LAUNCH_R(2, 8, kMaskNone);
     }
     return 0;
   }

@@ -51,7 +51,7 @@ def test_short_rows_keep_one_launch():
 @pytest.mark.parametrize("mode", ["bf16", "mixed", "fp32"])
 @pytest.mark.parametrize("starting", [True, False])
 @pytest.mark.parametrize("n,n_pad", [(2, 1), (33, 1), (37, 5), (64, 63), (100, 36), (128, 64), (130, 2),
-                                     (256, 32), (300, 45), (512, 40), (512, 64)])
+                                     (256, 32), (300, 45), (512, 40), (512, 64), (768, 48)])
 def test_padded_tail_equals_given_mask_and_oracle(mode, starting, n, n_pad):
     mixed = mode == "mixed"
     dt = torch.bfloat16 if mode == "bf16" else torch.float32
