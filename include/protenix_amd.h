@@ -48,7 +48,9 @@ extern "C" {
  * ptx_triattn_fwd, ptx_transition_pack) treat it as PTX_BF16, so one code serves a whole
  * update; the LayerNorm entry points refuse it.
  */
-enum ptx_dtype { PTX_F32 = 0, PTX_BF16 = 1, PTX_MIXED = 2 };
+enum ptx_dtype { PTX_F32 = 0, PTX_BF16 = 1, PTX_MIXED = 2, PTX_F16 = 3 };
+/* PTX_F16 (IEEE half) is taken by the LayerNorm entry points only, which dispatch on float /
+ * Half / BFloat16 like the reference's kernel (layer_norm_cuda_kernel.cu:304-330). */
 
 enum ptx_status {
   PTX_OK = 0,
@@ -174,6 +176,27 @@ PTX_API int ptx_trimul_output(const void* x, const void* z, const void* ln_in_w,
                       const void* ln_out_w, const void* ln_out_b, const void* w_z,
                       const void* w_g, void* out, int n, int c_z, int c_hidden,
                       int add_residual, float eps, int dtype, void* stream);
+
+/*
+ * The whole triangle multiplication in one call, with the argument list of the reference's
+ * fused operator (triangular.py:26-90, kernel_triangular_mult -> triangle_multiplicative_update;
+ * call site triangular.py:497-514): stacked input weights
+ *   p_in_weight = [linear_a_p.weight ; linear_b_p.weight]   [2 * c_hidden][c_z]
+ *   g_in_weight = [linear_a_g.weight ; linear_b_g.weight]   [2 * c_hidden][c_z]
+ *   p_out_weight = linear_z.weight [c_z][c_hidden],  g_out_weight = linear_g.weight [c_z][c_z]
+ * x, out [n][n][c_z] (out may alias x);  mask [n][n] or NULL;  incoming = 0: 'outgoing'.
+ * out = update, or x + update with add_residual.  Runs ptx_trimul_project,
+ * ptx_trimul_contract and ptx_trimul_output on `stream` with their intermediates in
+ * `workspace`: ptx_triangle_multiplicative_update_workspace_elems(n, c_hidden) elements of the
+ * arithmetic type (bf16 for PTX_MIXED), 16-byte aligned, uninitialised.
+ */
+PTX_API int64_t ptx_triangle_multiplicative_update_workspace_elems(int n, int c_hidden);
+PTX_API int ptx_triangle_multiplicative_update(
+    const void* x, int incoming, const void* mask, const void* norm_in_weight,
+    const void* norm_in_bias, const void* p_in_weight, const void* g_in_weight,
+    const void* norm_out_weight, const void* norm_out_bias, const void* p_out_weight,
+    const void* g_out_weight, void* out, void* workspace, int n, int c_z, int c_hidden,
+    int add_residual, float eps, int dtype, void* stream);
 
 /*
  * Triangle attention, stage 1 (triangular.py:683-692, layers.py:361-382, 386):

@@ -16,6 +16,8 @@ from .triangular import (
     TriangleMultiplicationIncoming,
     TriangleMultiplicationOutgoing,
     TriangleMultiplicativeUpdate,
+    kernel_triangular_mult,
+    triangle_multiplicative_update,
 )
 
 __all__ = [
@@ -24,5 +26,6 @@ __all__ = [
     "PairformerBlock", "PairformerStack", "Transition", "TriangleAttention",
     "TriangleAttentionEndingNode", "TriangleAttentionStartingNode",
     "TriangleMultiplicationIncoming", "TriangleMultiplicationOutgoing",
-    "TriangleMultiplicativeUpdate", "TriAttentionFunction", "tri_attention", "tri_attention_forward",
+    "TriangleMultiplicativeUpdate", "kernel_triangular_mult", "triangle_multiplicative_update",
+    "TriAttentionFunction", "tri_attention", "tri_attention_forward",
 ]

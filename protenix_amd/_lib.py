@@ -13,7 +13,7 @@ import threading
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libprotenix_amd.so")
 
-PTX_F32, PTX_BF16, PTX_MIXED = 0, 1, 2
+PTX_F32, PTX_BF16, PTX_MIXED, PTX_F16 = 0, 1, 2, 3
 ABI_VERSION = 2
 
 _p = ctypes.c_void_p
@@ -36,6 +36,8 @@ SIGNATURES = {
     "ptx_trimul_project": (_i, [_p] * 10 + [_i, _i, _i, _i, _i, _f, _i, _p]),
     "ptx_trimul_contract": (_i, [_p, _p, _p, _i, _i, _i, _i, _p]),
     "ptx_trimul_output": (_i, [_p] * 9 + [_i, _i, _i, _i, _f, _i, _p]),
+    "ptx_triangle_multiplicative_update_workspace_elems": (_l, [_i, _i]),
+    "ptx_triangle_multiplicative_update": (_i, [_p, _i] + [_p] * 11 + [_i, _i, _i, _i, _f, _i, _p]),
     "ptx_triattn_project": (_i, [_p] * 13 + [_i, _i, _i, _i, _i, _i, _f, _i, _p]),
     "ptx_triattn_fwd": (_i, [_p] * 7 + [_i, _i, _i, _i, _i, _f, _i, _p]),
     "ptx_triattn_fwd_rows": (_i, [_p] * 7 + [_i, _i, _i, _i, _i, _f, _i, _i, _i, _i, _p]),

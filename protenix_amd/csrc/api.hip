@@ -29,6 +29,8 @@ int after_launch(const char* what) {
 }
 
 bool dtype_ok(int dtype) { return dtype == PTX_F32 || dtype == PTX_BF16; }
+// the stand-alone LayerNorm also takes IEEE half, like the reference's kernel
+bool dtype_ok_ln(int dtype) { return dtype_ok(dtype) || dtype == PTX_F16; }
 // entry points that read or write the residual stream also take PTX_MIXED
 bool dtype_ok_z(int dtype) { return dtype_ok(dtype) || dtype == PTX_MIXED; }
 
@@ -39,6 +41,20 @@ bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
 #define PTX_REQUIRE(cond, code, ...) \
   do {                               \
     if (!(cond)) return fail(code, __VA_ARGS__); \
+  } while (0)
+
+#define PTX_DISPATCH_LN(dtype, CALL)     \
+  do {                                   \
+    if ((dtype) == PTX_F16) {            \
+      typedef ptx::f16_t T;              \
+      CALL;                              \
+    } else if ((dtype) == PTX_BF16) {    \
+      typedef ptx::bf16_t T;             \
+      CALL;                              \
+    } else {                             \
+      typedef float T;                   \
+      CALL;                              \
+    }                                    \
   } while (0)
 
 #define PTX_DISPATCH(dtype, CALL)        \
@@ -127,15 +143,15 @@ PTX_API int64_t ptx_triattn_bias_elems(int n, int heads) {
 
 PTX_API int ptx_layernorm_fwd(const void* x, const void* gamma, const void* beta, void* y, float* mean,
                       float* rstd, int64_t rows, int cols, float eps, int dtype, void* stream) {
-  PTX_REQUIRE(dtype_ok(dtype), PTX_ERR_BAD_ARG, "layernorm: unknown dtype %d", dtype);
+  PTX_REQUIRE(dtype_ok_ln(dtype), PTX_ERR_BAD_ARG, "layernorm: unknown dtype %d", dtype);
   PTX_REQUIRE(rows >= 0 && cols > 0, PTX_ERR_BAD_ARG, "layernorm: rows=%lld cols=%d",
               (long long)rows, cols);
   if (rows == 0) return PTX_OK;
   PTX_REQUIRE(x && y, PTX_ERR_BAD_ARG, "layernorm: null x or y");
   PTX_REQUIRE(rows < ((int64_t)1 << 31), PTX_ERR_UNSUPPORTED, "layernorm: rows=%lld too large",
               (long long)rows);
-  PTX_DISPATCH(dtype, ptx::layernorm_fwd<T>((const T*)x, (const T*)gamma, (const T*)beta, (T*)y,
-                                            mean, rstd, rows, cols, eps, (hipStream_t)stream));
+  PTX_DISPATCH_LN(dtype, ptx::layernorm_fwd<T>((const T*)x, (const T*)gamma, (const T*)beta, (T*)y,
+                                               mean, rstd, rows, cols, eps, (hipStream_t)stream));
   return after_launch("layernorm");
 }
 
@@ -146,7 +162,7 @@ PTX_API int64_t ptx_layernorm_bwd_workspace_elems(int64_t rows, int cols) {
 PTX_API int ptx_layernorm_bwd(const void* dout, const void* x, const float* mean, const float* rstd,
                       const void* gamma, void* dx, void* dgamma, void* dbeta, float* workspace,
                       int64_t rows, int cols, int dtype, void* stream) {
-  PTX_REQUIRE(dtype_ok(dtype), PTX_ERR_BAD_ARG, "layernorm_bwd: unknown dtype %d", dtype);
+  PTX_REQUIRE(dtype_ok_ln(dtype), PTX_ERR_BAD_ARG, "layernorm_bwd: unknown dtype %d", dtype);
   PTX_REQUIRE(rows >= 0 && cols > 0, PTX_ERR_BAD_ARG, "layernorm_bwd: rows=%lld cols=%d",
               (long long)rows, cols);
   PTX_REQUIRE(rows < ((int64_t)1 << 31), PTX_ERR_UNSUPPORTED,
@@ -156,9 +172,9 @@ PTX_API int ptx_layernorm_bwd(const void* dout, const void* x, const float* mean
   if (rows == 0 && !dgamma && !dbeta) return PTX_OK;
   if (rows > 0)
     PTX_REQUIRE(dout && x && mean && rstd && dx, PTX_ERR_BAD_ARG, "layernorm_bwd: null pointer");
-  PTX_DISPATCH(dtype, ptx::layernorm_bwd<T>((const T*)dout, (const T*)x, mean, rstd,
-                                            (const T*)gamma, (T*)dx, (T*)dgamma, (T*)dbeta,
-                                            workspace, rows, cols, (hipStream_t)stream));
+  PTX_DISPATCH_LN(dtype, ptx::layernorm_bwd<T>((const T*)dout, (const T*)x, mean, rstd,
+                                               (const T*)gamma, (T*)dx, (T*)dgamma, (T*)dbeta,
+                                               workspace, rows, cols, (hipStream_t)stream));
   return after_launch("layernorm_bwd");
 }
 
@@ -251,6 +267,47 @@ PTX_API int ptx_trimul_output(const void* x, const void* z, const void* ln_in_w,
   PTX_DISPATCH_Z(dtype, (ptx::trimul_output<T, TZ>)(x, z, ln_in_w, ln_in_b, ln_out_w, ln_out_b, w_z, w_g,
                                             out, n, c_z, add_residual, eps, (hipStream_t)stream));
   return after_launch("trimul_output");
+}
+
+PTX_API int64_t ptx_triangle_multiplicative_update_workspace_elems(int n, int c_hidden) {
+  if (n <= 0 || c_hidden <= 0) return 0;
+  // a, b (fragment order) and the channel-major product x
+  return 2 * ptx_trimul_operand_elems(n, c_hidden) + (int64_t)c_hidden * n * n;
+}
+
+PTX_API int ptx_triangle_multiplicative_update(
+    const void* x, int incoming, const void* mask, const void* norm_in_weight,
+    const void* norm_in_bias, const void* p_in_weight, const void* g_in_weight,
+    const void* norm_out_weight, const void* norm_out_bias, const void* p_out_weight,
+    const void* g_out_weight, void* out, void* workspace, int n, int c_z, int c_hidden,
+    int add_residual, float eps, int dtype, void* stream) {
+  PTX_REQUIRE(dtype_ok_z(dtype), PTX_ERR_BAD_ARG, "triangle_multiplicative_update: unknown dtype %d", dtype);
+  PTX_REQUIRE(n >= 0, PTX_ERR_BAD_ARG, "triangle_multiplicative_update: n=%d", n);
+  PTX_REQUIRE(pair_width_ok(c_z, c_hidden, dtype), PTX_ERR_UNSUPPORTED,
+              "triangle_multiplicative_update: %s (got c_z=%d c_hidden=%d)", kWidthMsg, c_z, c_hidden);
+  if (n == 0) return PTX_OK;
+  PTX_REQUIRE(x && p_in_weight && g_in_weight && p_out_weight && g_out_weight && out && workspace,
+              PTX_ERR_BAD_ARG, "triangle_multiplicative_update: null pointer");
+  PTX_REQUIRE(aligned16(workspace), PTX_ERR_BAD_ARG,
+              "triangle_multiplicative_update: workspace must be 16-byte aligned");
+  // p_in_weight = [W_a_p ; W_b_p], g_in_weight = [W_a_g ; W_b_g], each [2 * c_hidden][c_z]
+  const size_t es = esize(dtype == PTX_MIXED ? PTX_BF16 : dtype);
+  const size_t half = (size_t)c_hidden * c_z * es;
+  const char* w_p = (const char*)p_in_weight;
+  const char* w_g = (const char*)g_in_weight;
+  const int64_t n_op = ptx_trimul_operand_elems(n, c_hidden);
+  char* a = (char*)workspace;
+  char* b = a + n_op * es;
+  char* xc = b + n_op * es;
+  const int pitch = ptx_key_pitch(n);
+  int rc = ptx_trimul_project(x, mask, norm_in_weight, norm_in_bias, w_p, w_g, w_p + half, w_g + half, a,
+                              b, n, c_z, c_hidden, pitch, incoming, eps, dtype, stream);
+  if (rc != PTX_OK) return rc;
+  rc = ptx_trimul_contract(a, b, xc, n, c_hidden, pitch, dtype, stream);
+  if (rc != PTX_OK) return rc;
+  return ptx_trimul_output(xc, x, norm_in_weight, norm_in_bias, norm_out_weight, norm_out_bias,
+                           p_out_weight, g_out_weight, out, n, c_z, c_hidden, add_residual, eps, dtype,
+                           stream);
 }
 
 PTX_API int ptx_triattn_project(const void* z, const void* ln_w, const void* ln_b, const void* w_q,

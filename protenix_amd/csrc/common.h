@@ -18,6 +18,7 @@
 namespace ptx {
 
 typedef __bf16 bf16_t;
+typedef _Float16 f16_t;   // IEEE half: the stand-alone LayerNorm only
 typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
 typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
@@ -40,6 +41,7 @@ __device__ __forceinline__ f32x8 to_f32(f32x8 v) { return v; }
 __device__ __forceinline__ f32x4 to_f32(bf16x4 v) { return __builtin_convertvector(v, f32x4); }
 __device__ __forceinline__ f32x4 to_f32(f32x4 v) { return v; }
 __device__ __forceinline__ float to_f32(bf16_t v) { return (float)v; }
+__device__ __forceinline__ float to_f32(f16_t v) { return (float)v; }
 __device__ __forceinline__ float to_f32(float v) { return v; }
 
 template <typename T> __device__ __forceinline__ typename Vec8<T>::type from_f32(f32x8 v);
@@ -50,6 +52,7 @@ template <> __device__ __forceinline__ bf16x4 from_f32<bf16_t>(f32x4 v) { return
 template <> __device__ __forceinline__ f32x4 from_f32<float>(f32x4 v) { return v; }
 template <typename T> __device__ __forceinline__ T from_f32(float v);
 template <> __device__ __forceinline__ bf16_t from_f32<bf16_t>(float v) { return (bf16_t)v; }
+template <> __device__ __forceinline__ f16_t from_f32<f16_t>(float v) { return (f16_t)v; }
 template <> __device__ __forceinline__ float from_f32<float>(float v) { return v; }
 
 // acc += A * B for one 16-deep K step (see the convention above).

@@ -20,12 +20,20 @@ template <typename T, int VEC> struct VecN;
 template <> struct VecN<bf16_t, 8> { typedef bf16x8 type; typedef f32x8 ftype; };
 template <> struct VecN<bf16_t, 4> { typedef bf16x4 type; typedef f32x4 ftype; };
 template <> struct VecN<bf16_t, 2> { typedef bf16x2 type; typedef f32x2 ftype; };
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
+typedef __attribute__((ext_vector_type(4))) _Float16 f16x4;
+typedef __attribute__((ext_vector_type(2))) _Float16 f16x2;
+typedef __attribute__((ext_vector_type(1))) _Float16 f16x1;
+template <> struct VecN<f16_t, 8> { typedef f16x8 type; typedef f32x8 ftype; };
+template <> struct VecN<f16_t, 4> { typedef f16x4 type; typedef f32x4 ftype; };
+template <> struct VecN<f16_t, 2> { typedef f16x2 type; typedef f32x2 ftype; };
 template <> struct VecN<float, 4> { typedef f32x4 type; typedef f32x4 ftype; };
 template <> struct VecN<float, 2> { typedef f32x2 type; typedef f32x2 ftype; };
 typedef __attribute__((ext_vector_type(1))) float f32x1;
 typedef __attribute__((ext_vector_type(1))) __bf16 bf16x1;
 template <> struct VecN<bf16_t, 1> { typedef bf16x1 type; typedef f32x1 ftype; };
 template <> struct VecN<float, 1> { typedef f32x1 type; typedef f32x1 ftype; };
+template <> struct VecN<f16_t, 1> { typedef f16x1 type; typedef f32x1 ftype; };
 
 template <int G>
 __device__ __forceinline__ float group_sum(float v) {
@@ -278,6 +286,8 @@ template int layernorm_fwd<float>(const float*, const float*, const float*, floa
                                   int64_t, int, float, hipStream_t);
 template int layernorm_fwd<bf16_t>(const bf16_t*, const bf16_t*, const bf16_t*, bf16_t*, float*,
                                    float*, int64_t, int, float, hipStream_t);
+template int layernorm_fwd<f16_t>(const f16_t*, const f16_t*, const f16_t*, f16_t*, float*, float*,
+                                  int64_t, int, float, hipStream_t);
 
 // ---------------------------------------------------------------------------
 // Backward.  With xc = x - mean, gd = gamma * dout (gamma = 1 when absent), all in fp32:
@@ -558,5 +568,8 @@ template int layernorm_bwd<float>(const float*, const float*, const float*, cons
 template int layernorm_bwd<bf16_t>(const bf16_t*, const bf16_t*, const float*, const float*,
                                    const bf16_t*, bf16_t*, bf16_t*, bf16_t*, float*, int64_t, int,
                                    hipStream_t);
+template int layernorm_bwd<f16_t>(const f16_t*, const f16_t*, const float*, const float*,
+                                  const f16_t*, f16_t*, f16_t*, f16_t*, float*, int64_t, int,
+                                  hipStream_t);
 
 }  // namespace ptx

@@ -109,6 +109,18 @@ def key_pitch(n: int) -> int:
     return _lib.load().ptx_key_pitch(n)
 
 
+_LN_DTYPES = dict(_DTYPES)
+_LN_DTYPES[torch.float16] = _lib.PTX_F16
+
+
+def _dt_ln(t: torch.Tensor) -> int:
+    """dtype code of the stand-alone LayerNorm, which also takes float16."""
+    try:
+        return _LN_DTYPES[t.dtype]
+    except KeyError:
+        raise RuntimeError(f"protenix_amd LayerNorm takes float32, bfloat16 or float16 tensors, got {t.dtype}")
+
+
 def layer_norm(x: torch.Tensor, weight: Optional[torch.Tensor], bias: Optional[torch.Tensor],
                eps: float = 1e-5, return_stats: bool = False):
     """LayerNorm over the last dim (reference: layer_norm.py:70-112)."""
@@ -126,7 +138,7 @@ def layer_norm(x: torch.Tensor, weight: Optional[torch.Tensor], bias: Optional[t
         rstd = torch.empty(rows, dtype=torch.float32, device=x.device)
     with torch.cuda.device(x.device):
         _call("layernorm", lib.ptx_layernorm_fwd, _ptr(x), _ptr(w), _ptr(b), _ptr(y), _ptr(mean), _ptr(rstd),
-                                         rows, cols, eps, _dt(x), _stream())
+                                         rows, cols, eps, _dt_ln(x), _stream())
     return (y, mean, rstd) if return_stats else y
 
 
@@ -151,7 +163,7 @@ def layer_norm_backward(dout: torch.Tensor, x: torch.Tensor, mean: torch.Tensor,
                         x.device)
     with torch.cuda.device(x.device):
         _call("layernorm_bwd", lib.ptx_layernorm_bwd, _ptr(dout), _ptr(x), _ptr(mean), _ptr(rstd),
-              _ptr(w), _ptr(dx), _ptr(dw), _ptr(db), _ptr(ws), rows, cols, _dt(x), _stream())
+              _ptr(w), _ptr(dx), _ptr(dw), _ptr(db), _ptr(ws), rows, cols, _dt_ln(x), _stream())
     return dx, dw, db
 
 
@@ -305,6 +317,30 @@ def triangle_multiplication(z: torch.Tensor, mask: Optional[torch.Tensor], w: di
         _call("trimul_output", lib.ptx_trimul_output, _ptr(x), _ptr(z), _ptr(w["ln_in_w"]), _ptr(w["ln_in_b"]), _ptr(w["ln_out_w"]),
             _ptr(w["ln_out_b"]), _ptr(w["w_z"]), _ptr(w["w_g"]), _ptr(out), n, c_z, c_h,
             int(add_residual), eps, dt, st)
+    return out
+
+
+def triangle_multiplicative_update(x: torch.Tensor, incoming: bool, mask: Optional[torch.Tensor],
+                                   norm_in_weight, norm_in_bias, p_in_weight: torch.Tensor,
+                                   g_in_weight: torch.Tensor, norm_out_weight, norm_out_bias,
+                                   p_out_weight: torch.Tensor, g_out_weight: torch.Tensor,
+                                   eps: float = 1e-5) -> torch.Tensor:
+    """One [N, N, c_z] pair tensor through the one-call operator of the C ABI
+    (ptx_triangle_multiplicative_update: stacked input weights, one workspace); returns the
+    update.  Parameters in x's dtype, or bfloat16 beside float32 rows (PTX_MIXED)."""
+    _dev(x, "x")
+    lib = _lib.load()
+    n, c_z = x.shape[0], x.shape[-1]
+    c_h = p_in_weight.shape[0] // 2
+    cd = p_in_weight.dtype
+    mask = _mask_for(mask, x, cd)
+    ws = _workspace((lib.ptx_triangle_multiplicative_update_workspace_elems(n, c_h),), cd, x.device)
+    out = torch.empty_like(x)
+    with torch.cuda.device(x.device):
+        _call("triangle_multiplicative_update", lib.ptx_triangle_multiplicative_update, _ptr(x),
+              int(incoming), _ptr(mask), _ptr(norm_in_weight), _ptr(norm_in_bias), _ptr(p_in_weight),
+              _ptr(g_in_weight), _ptr(norm_out_weight), _ptr(norm_out_bias), _ptr(p_out_weight),
+              _ptr(g_out_weight), _ptr(out), _ptr(ws), n, c_z, c_h, 0, eps, _dt_stream(x, cd), _stream())
     return out
 
 

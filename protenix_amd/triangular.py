@@ -59,6 +59,34 @@ def _per_batch(z: torch.Tensor, mask: Optional[torch.Tensor]):
     return zb, mb
 
 
+def kernel_triangular_mult(x: torch.Tensor, direction: str, mask: Optional[torch.Tensor],
+                           norm_in_weight: Optional[torch.Tensor], norm_in_bias: Optional[torch.Tensor],
+                           p_in_weight: torch.Tensor, g_in_weight: torch.Tensor,
+                           norm_out_weight: Optional[torch.Tensor], norm_out_bias: Optional[torch.Tensor],
+                           p_out_weight: torch.Tensor, g_out_weight: torch.Tensor,
+                           eps: float = 1e-5) -> torch.Tensor:
+    """The reference's fused triangle-multiplication operator (triangular.py:26-90 and its
+    call site :497-514) on the HIP kernels: x [*, N, N, c_z], mask [*, N, N] or None,
+    p_in_weight / g_in_weight the stacked a / b projections and gates [2 * c_hidden, c_z],
+    p_out_weight = linear_z.weight, g_out_weight = linear_g.weight.  Returns the update."""
+    if direction not in ("outgoing", "incoming"):
+        raise ValueError(f"direction must be 'outgoing' or 'incoming', but got {direction}")
+    _forward_only(x, p_in_weight, g_in_weight, p_out_weight, g_out_weight, norm_in_weight, norm_in_bias,
+                  norm_out_weight, norm_out_bias)
+    z, cd, cast_back = _stream_and_compute_dtype(x, x.shape[-1])
+    ps = [_cv(p, cd, z.device) for p in (norm_in_weight, norm_in_bias, p_in_weight, g_in_weight,
+                                         norm_out_weight, norm_out_bias, p_out_weight, g_out_weight)]
+    src = z if z.is_contiguous() else z.contiguous()
+    zb, mb = _per_batch(src, mask)
+    out = torch.stack([ops.triangle_multiplicative_update(
+        zb[i], direction == "incoming", None if mb is None else mb[i], *ps, eps=eps)
+        for i in range(zb.shape[0])]).view(src.shape)
+    return out.to(cast_back) if cast_back is not None else out
+
+
+triangle_multiplicative_update = kernel_triangular_mult
+
+
 class TriangleMultiplicativeUpdate(nn.Module):
     """Algorithms 11 and 12 of AF3 (triangular.py:172-570)."""
 

@@ -45,6 +45,38 @@ def test_layernorm(dtype, rows, cols, affine):
     assert rel_err(y, ref) <= (1e-5 if dtype == torch.float32 else 2 ** -7)
 
 
+@pytest.mark.parametrize("rows,cols", [(1000, 128), (4099, 128), (70001, 128), (77, 384), (19, 100), (5, 7),
+                                       (3, 4096), (2, 5000), (0, 128)])
+@pytest.mark.parametrize("affine", ["both", "none"])
+def test_layernorm_float16(rows, cols, affine):
+    """IEEE half, the third dtype the reference's kernel dispatches on
+    (layer_norm_cuda_kernel.cu:304-330): forward and backward against the oracle."""
+    dtype = torch.float16
+    g = torch.Generator().manual_seed(rows * 17 + cols)
+    x = (torch.randn(rows, cols, generator=g) * 3 + 1.5).to(dtype)
+    dout = torch.randn(rows, cols, generator=g).to(dtype)
+    ln = P.LayerNorm(cols, create_scale=affine == "both", create_offset=affine == "both")
+    with torch.no_grad():
+        if ln.weight is not None:
+            ln.weight.copy_(1 + 0.1 * torch.randn(cols, generator=g))
+            ln.bias.copy_(0.1 * torch.randn(cols, generator=g))
+    ln = ln.to("cuda", dtype)
+    xg = x.cuda().requires_grad_(True)
+    y = ln(xg)
+    assert y.dtype == dtype and y.shape == x.shape
+    y.backward(dout.cuda())
+    assert xg.grad.dtype == dtype and xg.grad.shape == x.shape
+    if rows == 0:
+        return
+    w = ln.weight.detach().float().cpu() if ln.weight is not None else None
+    b = ln.bias.detach().float().cpu() if ln.bias is not None else None
+    assert rel_err(y, O.layer_norm(x.float(), w, b)) <= 2 ** -10      # half: 11 significant bits
+    dx, dg, db = O.layer_norm_backward(dout.float(), x.float(), w)
+    assert rel_err(xg.grad, dx) <= 2e-3
+    if w is not None:
+        assert rel_err(ln.weight.grad, dg) <= 2e-3 and rel_err(ln.bias.grad, db) <= 2e-3
+
+
 def test_layernorm_stats_and_closed_forms():
     from protenix_amd import ops
     x = torch.randn(513, 128, device="cuda") * 2 + 3
@@ -120,6 +152,37 @@ def test_layernorm_backward_c_abi_options_and_determinism():
 
 
 # ------------------------------------------------------------------ TriMul
+@pytest.mark.parametrize("mode", ["fp32", "bf16", "mixed"])
+@pytest.mark.parametrize("direction", ["outgoing", "incoming"])
+@pytest.mark.parametrize("n,n_pad,batch", [(64, 0, 1), (100, 7, 2), (37, 0, 1)])
+def test_fused_trimul_operator(mode, direction, n, n_pad, batch):
+    """The reference's one-call operator (triangular.py:26-90, call site :497-514): stacked
+    input weights, one call; against the oracle module and, bit for bit, the three-stage module."""
+    dtype = torch.float32 if mode == "fp32" else torch.bfloat16
+    cls = "TriangleMultiplicationOutgoing" if direction == "outgoing" else "TriangleMultiplicationIncoming"
+    ref, prod = oracle_and_product(getattr(O, cls), getattr(P, cls), 128, 128, dtype=dtype)
+    g = torch.Generator().manual_seed(n + batch)
+    z = torch.randn(batch, n, n, 128, generator=g).to(dtype)
+    mask = pad_mask(n, n_pad).expand(batch, n, n).contiguous() if n_pad else None
+    with torch.no_grad():
+        want = ref(z.float(), None if mask is None else mask.float())
+    m = prod if mode != "mixed" else prod.float()
+    zd = z.cuda() if mode != "mixed" else z.float().cuda()
+    md = None if mask is None else mask.to(zd.dtype).cuda()
+    args = (m.layer_norm_in.weight, m.layer_norm_in.bias,
+            torch.cat([m.linear_a_p.weight, m.linear_b_p.weight], 0),
+            torch.cat([m.linear_a_g.weight, m.linear_b_g.weight], 0),
+            m.layer_norm_out.weight, m.layer_norm_out.bias, m.linear_z.weight, m.linear_g.weight)
+    with torch.no_grad(), torch.autocast("cuda", dtype=torch.bfloat16, enabled=mode == "mixed"):
+        got = P.kernel_triangular_mult(zd, direction, md, *args, eps=1e-5)
+        staged = m(zd, mask=md)
+    assert got.shape == z.shape and got.dtype == staged.dtype
+    assert torch.equal(got, staged)
+    assert rel_err(got, want) <= tol(dtype)
+    with pytest.raises(ValueError):
+        P.kernel_triangular_mult(zd, "sideways", md, *args)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("cls", ["TriangleMultiplicationOutgoing", "TriangleMultiplicationIncoming"])
 @pytest.mark.parametrize("n,n_pad", [(64, 0), (100, 7), (37, 0), (200, 16)])
