@@ -446,6 +446,31 @@ def main() -> int:
                     "workload": "TriAttentionFunction.apply + backward (dQ, dK, dV, dBias2); fwd_ms includes "
                                 "the scaling of Q and the repack of the operands into the core's tile order"}
                 del qkv, qo, ko, vo, do, b1o, b2o, oo
+            # the scaled-up model's block (c_z = 256, 8 pair heads, c_hidden_mul = 256), fp32 rows
+            # under bf16 autocast: the fused fp32-row kernels of that width
+            del stack
+            torch.cuda.empty_cache()
+            ref256 = O.seed_parameters_(O.PairformerStack(n_blocks=2, c_z=256, hidden_scale_up=True))
+            st256 = P.PairformerStack(n_blocks=2, c_z=256, hidden_scale_up=True)
+            st256.load_state_dict(ref256.state_dict())
+            st256 = st256.to(dev).eval()
+            del ref256
+            s6, z6, pm6 = (t.to(dev) for t in O.make_inputs(n, c_z=256))
+            zw6 = torch.empty_like(z6)
+
+            def step256():
+                zw6.copy_(z6)
+                with amp(True):
+                    return st256(s6, zw6, pm6, inplace_safe=True)
+            _, per256, _ = timed(step256, 2, 5)
+            shapes["scaled_up_cz256_2_blocks_n768"] = {
+                "ms": round(statistics.median(per256), 3),
+                "ms_per_block": round(statistics.median(per256) / 2, 3),
+                "workload": f"PairformerStack 2 blocks, c_z=256, hidden_scale_up (8 pair heads, c_hidden_mul=256), "
+                            f"N_token={n}, fp32 tensors and parameters under torch.autocast(bfloat16)"}
+            del st256, s6, z6, pm6, zw6, step256
+            torch.cuda.empty_cache()
+            stack = None
             # stand-alone LayerNorm over c_z = 128 on the pair tensor's rows
             for dt, name, ckey in ((BF16, "bf16", "151MB"), (torch.float32, "fp32", "302MB")):
                 x = torch.randn(768 * 768, 128, device=dev, dtype=dt)
@@ -512,7 +537,7 @@ def main() -> int:
         "shapes": shapes,
     }
     if not args.no_cpu_baseline:
-        del stack
+        stack = None
         torch.cuda.empty_cache()
         out["cpu_baseline"] = _cpu_baseline(n, 2)
     print(json.dumps(out))

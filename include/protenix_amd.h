@@ -44,7 +44,7 @@ extern "C" {
  * the `out` it adds its update to are fp32; weights, masks, workspaces and every other tensor
  * are bf16.  Rows are normalised in fp32 and rounded to bf16 for the matrix products; the
  * update is rounded to bf16 and added to the fp32 row.  Accepted by the entry points that
- * touch the residual stream (rows of 64 or 128 channels); the others (ptx_trimul_contract,
+ * touch the residual stream (rows of 64, 128 or 256 channels); the others (ptx_trimul_contract,
  * ptx_triattn_fwd, ptx_transition_pack) treat it as PTX_BF16, so one code serves a whole
  * update; the LayerNorm entry points refuse it.
  */
@@ -148,7 +148,7 @@ PTX_API int ptx_layernorm_bwd_static(const void* dout, const void* x, const floa
  *   elements each, written in the contraction's operand order (K between n and
  *   k_pitch is written as zeros, rows beyond n stay unwritten);
  *   k_pitch = ptx_key_pitch(n).  Widths: c_z = 64 or 128 with c_hidden = 128, or
- *   (bf16 only) c_z = c_hidden = 256.
+ *   (PTX_BF16, PTX_MIXED) c_z = c_hidden = 256.
  */
 PTX_API int ptx_trimul_project(const void* z, const void* mask, const void* ln_w, const void* ln_b,
                        const void* w_ap, const void* w_ag, const void* w_bp, const void* w_bg,
@@ -207,7 +207,7 @@ PTX_API int ptx_triangle_multiplicative_update(
  *   q, g [heads][n][n][d] (logical row p = i*n + j);  k, vt: workspaces of
  *   ptx_triattn_kv_elems(n, heads) elements;  tri_bias: ptx_triattn_bias_elems(n, heads)
  *   elements;  key_pitch = ptx_key_pitch(n).   d = 32;  c_in = 64 or 128 with 4 heads,
- *   or (bf16 only) c_in = 256 with 8 heads  (w_q, w_k, w_v, w_g [heads*d][c_in],
+ *   or (PTX_BF16, PTX_MIXED) c_in = 256 with 8 heads  (w_q, w_k, w_v, w_g [heads*d][c_in],
  *   w_b [heads][c_in]).
  * g = NULL (c_in = 128, 4 heads, PTX_BF16 / PTX_MIXED): no gate is written; stage 2 is then
  * called without one and ptx_triattn_gate_output forms it in stage 3.
@@ -299,7 +299,7 @@ PTX_API int ptx_triattn_core_bwd(const void* q, const void* k, const void* v, co
  * pairformer.py:189-213):  out(p) = [z(p) +] W_o o[p], where logical row p maps
  * to z[i][j] or, transposed = 1, z[j][i].  o [heads][n][n][d] as written by
  * stage 2; w_o [c_in][heads*d]; out may alias z.  c_in = 64 or 128 (heads*d = 128), or
- * (bf16 only) c_in = heads*d = 256.
+ * (PTX_BF16, PTX_MIXED) c_in = heads*d = 256.
  */
 PTX_API int ptx_triattn_output(const void* o, const void* w_o, const void* z, void* out, int n,
                        int c_in, int transposed, int add_residual, int dtype, void* stream);
@@ -327,7 +327,7 @@ PTX_API int ptx_triattn_gate_output(const void* o, const void* z, const void* ln
  *     packed, ptx_transition_packed_elems(c, n_factor) = 3*n_factor*c*c elements.
  *   ptx_transition_fwd:   x, out [rows][c] (out may alias x), ln_w / ln_b may be NULL.
  * a and b stay in fp32 through the activation (the reference rounds them to the
- * storage dtype first); the product is rounded once.   c = 64, 128 or (bf16 only) 256;
+ * storage dtype first); the product is rounded once.   c = 64, 128 or (PTX_BF16, PTX_MIXED) 256;
  * n_factor*c a multiple of 64.
  */
 PTX_API int64_t ptx_transition_packed_elems(int c, int n_factor);
@@ -355,7 +355,7 @@ PTX_API int ptx_transition_pair_bias_fwd(const void* x, const void* ln_w, const 
 /*
  * Pair bias of the single-representation attention (transformer.py:191-194):
  *   bias[h][i][j] = (W LN(z[i][j]))[h],  W [heads][c_z], heads <= 32, c_z = 128 or
- * (bf16 only) 256.
+ * (PTX_BF16, PTX_MIXED) 256.
  * ln_b may be NULL.  bias is fp32 when out_f32 = 1, else `dtype`.
  */
 PTX_API int ptx_pair_bias_fwd(const void* z, const void* ln_w, const void* ln_b, const void* w,

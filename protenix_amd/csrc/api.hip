@@ -198,13 +198,13 @@ PTX_API int ptx_layernorm_bwd_static(const void* dout, const void* x, const floa
 }
 
 // Pair-row widths the kernels are built for: c_z = 64 or 128 with hidden widths (c_hidden,
-// heads * 32) of 128, or c_z = 256 in bf16 with hidden widths of 256.
+// heads * 32) of 128, or c_z = 256 in bf16 arithmetic with hidden widths of 256.
 static bool pair_width_ok(int c_z, int hidden, int dtype) {
   if (c_z == 64 || c_z == 128) return hidden == 128;
-  return c_z == 256 && hidden == 256 && dtype == PTX_BF16;   // (not PTX_MIXED)
+  return c_z == 256 && hidden == 256 && dtype != PTX_F32;   // (bf16 arithmetic: PTX_BF16, PTX_MIXED)
 }
 static const char* const kWidthMsg =
-    "only c_z = 64 / 128 with hidden width 128, or c_z = 256 with hidden width 256 in bf16, is built";
+    "only c_z = 64 / 128 with hidden width 128, or c_z = 256 with hidden width 256 in bf16 arithmetic, is built";
 
 PTX_API int ptx_trimul_project(const void* z, const void* mask, const void* ln_w, const void* ln_b,
                        const void* w_ap, const void* w_ag, const void* w_bp, const void* w_bg,
@@ -542,8 +542,8 @@ PTX_API int ptx_transition_fwd(const void* x, const void* ln_w, const void* ln_b
   PTX_REQUIRE(dtype_ok_z(dtype), PTX_ERR_BAD_ARG, "transition: unknown dtype %d", dtype);
   PTX_REQUIRE(rows >= 0 && n_factor > 0, PTX_ERR_BAD_ARG, "transition: rows=%lld n_factor=%d",
               (long long)rows, n_factor);
-  PTX_REQUIRE(c == 128 || c == 64 || (c == 256 && dtype == PTX_BF16), PTX_ERR_UNSUPPORTED,
-              "transition: only c = 64, 128, or 256 in bf16 (not mixed), is built (got %d)", c);
+  PTX_REQUIRE(c == 128 || c == 64 || (c == 256 && dtype != PTX_F32), PTX_ERR_UNSUPPORTED,
+              "transition: only c = 64, 128, or 256 in bf16 arithmetic, is built (got %d)", c);
   PTX_REQUIRE((n_factor * c) % 64 == 0, PTX_ERR_UNSUPPORTED,
               "transition: the hidden width %d is not a multiple of 64", n_factor * c);
   PTX_REQUIRE(n_factor <= 64, PTX_ERR_UNSUPPORTED, "transition: n_factor=%d too large", n_factor);
@@ -666,8 +666,8 @@ PTX_API int ptx_pair_bias_fwd(const void* z, const void* ln_w, const void* ln_b,
                       void* stream) {
   PTX_REQUIRE(dtype_ok_z(dtype), PTX_ERR_BAD_ARG, "pair_bias: unknown dtype %d", dtype);
   PTX_REQUIRE(n >= 0, PTX_ERR_BAD_ARG, "pair_bias: n=%d", n);
-  PTX_REQUIRE(c_z == 128 || (c_z == 256 && dtype == PTX_BF16), PTX_ERR_UNSUPPORTED,
-              "pair_bias: only c_z = 128, or 256 in bf16, is built (got %d)", c_z);
+  PTX_REQUIRE(c_z == 128 || (c_z == 256 && dtype != PTX_F32), PTX_ERR_UNSUPPORTED,
+              "pair_bias: only c_z = 128, or 256 in bf16 arithmetic, is built (got %d)", c_z);
   PTX_REQUIRE(heads >= 1 && heads <= 32, PTX_ERR_UNSUPPORTED,
               "pair_bias: heads=%d outside 1..32", heads);
   PTX_REQUIRE(n < 32768, PTX_ERR_UNSUPPORTED, "pair_bias: n=%d too large", n);

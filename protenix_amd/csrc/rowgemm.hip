@@ -147,8 +147,8 @@ rowgemm_in_kernel(RowGemmInParams p) {
   typedef Cfg<TZ> CZ;
   typedef InCfg<T, MODE, KS> IC;
   constexpr bool MIXED = !std::is_same<T, TZ>::value;
-  static_assert(!MIXED || (sizeof(T) == 2 && sizeof(TZ) == 4 && KS <= 8),
-                "mixed storage: bf16 arithmetic on fp32 rows of at most 128 channels");
+  static_assert(!MIXED || (sizeof(T) == 2 && sizeof(TZ) == 4),
+                "mixed storage: bf16 arithmetic on fp32 rows");
   // kTriMulOut with bf16 arithmetic on rows of at most 128 channels keeps the raw rows (as
   // fp32) in registers for the residual add instead of a copy in LDS (see below)
   constexpr bool kRegRes = MODE == kTriMulOut && sizeof(T) == 2 && KS <= 8;
@@ -163,7 +163,11 @@ rowgemm_in_kernel(RowGemmInParams p) {
   // HBM at the end costs a full extra pass: by then they have left the L2)
   constexpr int kCz = 16 * KS;   // channels of a pair-tensor row
   constexpr int kResPitch = kCz + 16 / (int)sizeof(T);
-  constexpr bool kLdsRes = MODE == kTriMulOut && !kRegRes;
+  // kGlobRes (fp32 rows of 256 channels): no copy of the raw rows is kept - an fp32 copy in LDS
+  // would take 133 KB next to the weight ring, in registers 128 of them; each chunk reads the
+  // residual of its own 32 columns from memory again before it stores them
+  constexpr bool kGlobRes = MODE == kTriMulOut && !kRegRes && MIXED;
+  constexpr bool kLdsRes = MODE == kTriMulOut && !kRegRes && !MIXED;
   __shared__ __attribute__((aligned(16))) T lds_res[kLdsRes ? NW : 1][kLdsRes ? RB * 32 : 1][kLdsRes ? kResPitch : 8];
   // kRegRes: staging tile of the fp32 output rows (one 32 x 32 tile per wave)
   __shared__ __attribute__((aligned(16))) TZ lds_stage_z[kRegRes ? NW : 1][kRegRes ? 32 * CZ::PITCH : 4];
@@ -361,6 +365,8 @@ rowgemm_in_kernel(RowGemmInParams p) {
     // (the fp32 rows are requested further down, once the triangle product's rows are on
     // their way through the staging tile: both sets of raw rows at once do not fit the
     // registers)
+  } else if constexpr (kGlobRes) {
+    load_rows<T, RB, true>(xf, (const TZ*)p.x, p.xmap, row0, p.n_rows, gamma, beta, p.eps, lane);
   } else if constexpr (MODE == kTriMulOut) {
     RowFrags<T, RB, KS> zraw;
     load_rows<T, RB, false>(zraw, (const T*)p.x, p.xmap, row0, p.n_rows, (const T*)nullptr,
@@ -608,6 +614,23 @@ rowgemm_in_kernel(RowGemmInParams p) {
           int mj, m0;
           stage_coord<T>(ps, lane, mj, m0);
           resv[rb][ps] = *reinterpret_cast<const VE_t*>(&lds_res[wave][rb * 32 + mj][ch * 32 + m0]);
+        }
+    }
+    // kGlobRes: the fp32 residual of this chunk's columns, read back from the pair tensor (the
+    // same addresses this lane stores to below; other chunks touch other columns, so the values
+    // are the kernel's input also where out aliases z)
+    f32x4 resz[kGlobRes ? RB : 1][kGlobRes ? C::NPASS : 1][2];
+    if constexpr (kGlobRes) {
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+        for (int ps = 0; ps < C::NPASS; ++ps) {
+          int mj, m0;
+          stage_coord<T>(ps, lane, mj, m0);
+          const int64_t pr = rrow[rb][ps] >= 0 ? rrow[rb][ps] : 0;
+          const TZ* src = (const TZ*)p.x + p.xmap(pr) + ch * 32 + m0;
+          resz[rb][ps][0] = *reinterpret_cast<const f32x4*>(src);
+          resz[rb][ps][1] = *reinterpret_cast<const f32x4*>(src + 4);
         }
     }
     // Orientation: channel-major outputs want lane <-> channel (x as A operand).
@@ -874,6 +897,32 @@ rowgemm_in_kernel(RowGemmInParams p) {
                 rrow_z[rb][ps] >= 0 ? dstp : reinterpret_cast<TZ*>(g_store_sink) + lane * CZ::VE) = v;
           }
         }
+      } else if constexpr (kGlobRes) {
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) {
+          float vals[16];
+#pragma unroll
+          for (int r = 0; r < 16; ++r)
+            vals[r] = to_f32(from_f32<T>(acc[rb][0][r])) * sigmoidf_fast(acc[rb][1][r]);
+          wave_lds_sync();
+          stage_put<T>(st, vals, lane);   // (rounds the update to T)
+          wave_lds_sync();
+#pragma unroll
+          for (int ps = 0; ps < C::NPASS; ++ps) {
+            int mj, m0;
+            stage_coord<T>(ps, lane, mj, m0);
+            const f32x8 u = to_f32(stage_get_vec<T>(st, mj, m0));
+            f32x4 o0 = {u[0], u[1], u[2], u[3]}, o1 = {u[4], u[5], u[6], u[7]};
+            if (p.add_residual) {
+              o0 += resz[rb][ps][0];
+              o1 += resz[rb][ps][1];
+            }
+            TZ* dst = rrow[rb][ps] >= 0 ? (TZ*)p.out[0] + rrow[rb][ps] * kCz + ch * 32 + m0
+                                        : reinterpret_cast<TZ*>(g_store_sink) + lane * 4;
+            *reinterpret_cast<f32x4*>(dst) = o0;
+            *reinterpret_cast<f32x4*>(rrow[rb][ps] >= 0 ? dst + 4 : dst) = o1;
+          }
+        }
       } else {
 #pragma unroll
       for (int rb = 0; rb < RB; ++rb) {
@@ -1065,12 +1114,14 @@ __global__ __launch_bounds__(256, 2) void rowgemm_out_kernel(RowGemmOutParams p)
   }
 
   // out may alias res: a lane reads the residual vectors it is about to overwrite.  They
-  // are all requested up front: next to their stores each would cost a serialised memory
-  // round trip, since no load can move above the previous (possibly aliasing) store.
+  // are requested up front, a group of output column blocks at a time: next to their stores
+  // each would cost a serialised memory round trip, since no load can move above the previous
+  // (possibly aliasing) store.  One group, except for fp32 rows of 256 channels, whose 32
+  // residual vectors per lane do not fit beside the accumulators: two groups of four blocks.
+  constexpr int GOB = (MIXED && NOB > 4) ? 4 : NOB;
   TZ* outp = (TZ*)p.out;
   const TZ* resp = (const TZ*)p.res;
   int64_t obase[RB][C::NPASS];
-  VE_t resv[RB][NOB][C::NPASS];
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
@@ -1080,35 +1131,39 @@ __global__ __launch_bounds__(256, 2) void rowgemm_out_kernel(RowGemmOutParams p)
       const int64_t pr = row0 + rb * 32 + mj;
       obase[rb][ps] = pr < p.n_rows ? p.omap(pr) + m0 : -1;
     }
-  if (resp) {
 #pragma unroll
-    for (int rb = 0; rb < RB; ++rb)
+  for (int t0 = 0; t0 < NOB; t0 += GOB) {
+    VE_t resv[RB][GOB][C::NPASS];
+    if (resp) {
 #pragma unroll
-      for (int t = 0; t < NOB; ++t)
+      for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
-        for (int ps = 0; ps < C::NPASS; ++ps)
-          if (obase[rb][ps] >= 0)
-            resv[rb][t][ps] = *reinterpret_cast<const VE_t*>(resp + obase[rb][ps] + t * 32);
-  }
+        for (int t = 0; t < GOB; ++t)
 #pragma unroll
-  for (int rb = 0; rb < RB; ++rb) {
+          for (int ps = 0; ps < C::NPASS; ++ps)
+            if (obase[rb][ps] >= 0)
+              resv[rb][t][ps] = *reinterpret_cast<const VE_t*>(resp + obase[rb][ps] + (t0 + t) * 32);
+    }
 #pragma unroll
-    for (int t = 0; t < NOB; ++t) {
-      float vals[16];
+    for (int rb = 0; rb < RB; ++rb) {
 #pragma unroll
-      for (int r = 0; r < 16; ++r)   // (mixed: the product is rounded to T before it is added)
-        vals[r] = MIXED ? to_f32(from_f32<T>(acc[rb][t][r])) : acc[rb][t][r];
-      wave_lds_sync();
-      stage_put<TZ>(st, vals, lane);
-      wave_lds_sync();
+      for (int t = 0; t < GOB; ++t) {
+        float vals[16];
 #pragma unroll
-      for (int ps = 0; ps < C::NPASS; ++ps) {
-        int mj, m0;
-        stage_coord<TZ>(ps, lane, mj, m0);
-        if (obase[rb][ps] >= 0) {
-          VE_t v = stage_get_vec<TZ>(st, mj, m0);
-          if (resp) v = add_vec<TZ>(v, resv[rb][t][ps]);
-          *reinterpret_cast<VE_t*>(outp + obase[rb][ps] + t * 32) = v;
+        for (int r = 0; r < 16; ++r)   // (mixed: the product is rounded to T before it is added)
+          vals[r] = MIXED ? to_f32(from_f32<T>(acc[rb][t0 + t][r])) : acc[rb][t0 + t][r];
+        wave_lds_sync();
+        stage_put<TZ>(st, vals, lane);
+        wave_lds_sync();
+#pragma unroll
+        for (int ps = 0; ps < C::NPASS; ++ps) {
+          int mj, m0;
+          stage_coord<TZ>(ps, lane, mj, m0);
+          if (obase[rb][ps] >= 0) {
+            VE_t v = stage_get_vec<TZ>(st, mj, m0);
+            if (resp) v = add_vec<TZ>(v, resv[rb][t][ps]);
+            *reinterpret_cast<VE_t*>(outp + obase[rb][ps] + (t0 + t) * 32) = v;
+          }
         }
       }
     }
@@ -1158,8 +1213,8 @@ int trimul_project(const void* z, const void* mask, const void* ln_w, const void
   p.aux = incoming != 0;   // walk direction (see the kernel)
   if (c_z == 64) return launch_rowgemm_in<T, kTriMulIn, 4, TZ>(p, stream);
   if (c_z == 256) {
-    if constexpr (sizeof(T) == 2 && sizeof(TZ) == 2) return launch_rowgemm_in<T, kTriMulIn, 16>(p, stream);
-    else return -1;   // 256-channel rows are built for bf16 only (refused by the caller)
+    if constexpr (sizeof(T) == 2) return launch_rowgemm_in<T, kTriMulIn, 16, TZ>(p, stream);
+    else return -1;   // 256-channel rows are built for 16-bit arithmetic only (refused by the caller)
   }
   return launch_rowgemm_in<T, kTriMulIn, 8, TZ>(p, stream);
 }
@@ -1184,8 +1239,8 @@ int trimul_output(const void* x, const void* z, const void* ln_in_w, const void*
   p.add_residual = add_residual;
   if (c_z == 64) return launch_rowgemm_in<T, kTriMulOut, 4, TZ>(p, stream);
   if (c_z == 256) {
-    if constexpr (sizeof(T) == 2 && sizeof(TZ) == 2) return launch_rowgemm_in<T, kTriMulOut, 16>(p, stream);
-    else return -1;   // 256-channel rows are built for bf16 only (refused by the caller)
+    if constexpr (sizeof(T) == 2) return launch_rowgemm_in<T, kTriMulOut, 16, TZ>(p, stream);
+    else return -1;   // 256-channel rows are built for 16-bit arithmetic only (refused by the caller)
   }
   return launch_rowgemm_in<T, kTriMulOut, 8, TZ>(p, stream);
 }
@@ -1210,8 +1265,8 @@ int triattn_project(const void* z, const void* ln_w, const void* ln_b, const voi
   p.q_scale = 1.4426950408889634f / sqrtf((float)d);   // log2(e) / sqrt(d), see triattn.hip
   if (c_z == 64) return launch_rowgemm_in<T, kTriAttnIn, 4, TZ>(p, stream);
   if (c_z == 256) {
-    if constexpr (sizeof(T) == 2 && sizeof(TZ) == 2) return launch_rowgemm_in<T, kTriAttnIn, 16>(p, stream);
-    else return -1;   // 256-channel rows are built for bf16 only (refused by the caller)
+    if constexpr (sizeof(T) == 2) return launch_rowgemm_in<T, kTriAttnIn, 16, TZ>(p, stream);
+    else return -1;   // 256-channel rows are built for 16-bit arithmetic only (refused by the caller)
   }
   return launch_rowgemm_in<T, kTriAttnIn, 8, TZ>(p, stream);
 }
@@ -1230,7 +1285,7 @@ int triattn_output(const void* o, const void* w_o, const void* z, void* out, int
   p.n_rows = (int64_t)n * n;
   if (c_z == 64) return launch_rowgemm_out<T, 2, TZ>(p, stream);
   if (c_z == 256) {
-    if constexpr (sizeof(T) == 2 && sizeof(TZ) == 2) return launch_rowgemm_out<T, 8>(p, stream);
+    if constexpr (sizeof(T) == 2) return launch_rowgemm_out<T, 8, TZ>(p, stream);
     else return -1;
   }
   return launch_rowgemm_out<T, 4, TZ>(p, stream);
@@ -1251,7 +1306,7 @@ int pair_bias_fwd(const void* z, const void* ln_w, const void* ln_b, const void*
   p.n = n;
   p.aux = heads | (out_f32 ? 0x100 : 0);
   if (c_z == 256) {
-    if constexpr (sizeof(T) == 2 && sizeof(TZ) == 2) return launch_rowgemm_in<T, kPairBias, 16>(p, stream);
+    if constexpr (sizeof(T) == 2) return launch_rowgemm_in<T, kPairBias, 16, TZ>(p, stream);
     else return -1;
   }
   return launch_rowgemm_in<T, kPairBias, 8, TZ>(p, stream);

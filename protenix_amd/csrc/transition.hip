@@ -1,4 +1,4 @@
-// Transition (SwiGLU feed-forward) on rows of c = 128 (or 64; 256 in bf16) channels, one kernel:
+// Transition (SwiGLU feed-forward) on rows of c = 128 (or 64; 256 in 16-bit arithmetic) channels, one kernel:
 //   out = [x +] W_o ( silu(W_a LN(x)) * (W_b LN(x)) ),   W_a, W_b [c*n_factor][c]
 // (the comments below give the sizes for c = 128).
 // The hidden activations (n_factor * c per row) never leave the chip: a wave
@@ -282,8 +282,12 @@ __global__ __launch_bounds__((TrCfg<T, KS>::NW * 64), 2) void transition_fused_k
   // latency passes under the drain (loading each one next to its store would serialise a
   // full memory round trip per tile: out may alias x, so no load could move above the
   // previous store).  Each lane reads exactly the vectors it later overwrites.
+  // (fp32 rows of 256 channels: 32 residual vectors per lane do not fit beside the output
+  // accumulators; the second half of the column blocks is requested after the first half's
+  // stores, one serialised round trip per wave)
+  constexpr int GOB = (MIXED && NOB > 4) ? 4 : NOB;
   int64_t obase[RB][C::NPASS];
-  VE_t resv[RB][NOB][C::NPASS];
+  VE_t resv[RB][GOB][C::NPASS];
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
@@ -293,16 +297,19 @@ __global__ __launch_bounds__((TrCfg<T, KS>::NW * 64), 2) void transition_fused_k
       const int64_t pr = row0 + rb * 32 + mj;
       obase[rb][ps] = pr < n_rows ? pr * kCx + m0 : -1;
     }
-  if (add_residual) {
+  auto load_residual = [&](int ob0) {
+    if (add_residual) {
 #pragma unroll
-    for (int rb = 0; rb < RB; ++rb)
+      for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
-      for (int ob = 0; ob < NOB; ++ob)
+        for (int ob = 0; ob < GOB; ++ob)
 #pragma unroll
-        for (int ps = 0; ps < C::NPASS; ++ps)
-          if (obase[rb][ps] >= 0)
-            resv[rb][ob][ps] = *reinterpret_cast<const VE_t*>(x + obase[rb][ps] + ob * 32);
-  }
+          for (int ps = 0; ps < C::NPASS; ++ps)
+            if (obase[rb][ps] >= 0)
+              resv[rb][ob][ps] = *reinterpret_cast<const VE_t*>(x + obase[rb][ps] + (ob0 + ob) * 32);
+    }
+  };
+  load_residual(0);
   // drain: activation and GEMM2 of the last chunk
 #pragma unroll
   for (int kk = 0; kk < KS; ++kk) act_part(kk, ab1);
@@ -334,6 +341,10 @@ __global__ __launch_bounds__((TrCfg<T, KS>::NW * 64), 2) void transition_fused_k
   for (int rb = 0; rb < RB; ++rb) {
 #pragma unroll
     for (int ob = 0; ob < NOB; ++ob) {
+      if (GOB < NOB && ob > 0 && ob % GOB == 0) {
+        static_assert(GOB == NOB || RB == 1, "column groups: one row block");
+        load_residual(ob);
+      }
       float vals[16];
 #pragma unroll
       for (int r = 0; r < 16; ++r)   // (mixed: the update is rounded to T before it is added)
@@ -347,7 +358,7 @@ __global__ __launch_bounds__((TrCfg<T, KS>::NW * 64), 2) void transition_fused_k
         stage_coord<TZ>(ps, lane, mj, m0);
         VE_t v = stage_get_vec<TZ>(st, mj, m0);
         if (obase[rb][ps] >= 0) {
-          if (add_residual) v = add_vec<TZ>(v, resv[rb][ob][ps]);
+          if (add_residual) v = add_vec<TZ>(v, resv[rb][ob % GOB][ps]);
           *reinterpret_cast<VE_t*>(out + obase[rb][ps] + ob * 32) = v;
         }
         if constexpr (PB) done[rb][ob][ps] = v;
@@ -499,8 +510,8 @@ int transition_fwd(const void* x, const void* ln_w, const void* ln_b, const void
     return transition_fwd_ks<T, 4, TZ>(x, ln_w, ln_b, packed, out, rows, n_factor, add_residual, eps,
                                    stream);
   if (c == 256) {
-    // bf16 only: an fp32 chunk of weights (96 KB) leaves no room for a ring in LDS
-    if constexpr (sizeof(T) == 2 && sizeof(TZ) == 2)
+    // 16-bit arithmetic only: an fp32 chunk of weights (96 KB) leaves no room for a ring in LDS
+    if constexpr (sizeof(T) == 2)
       return transition_fwd_ks<T, 16, TZ>(x, ln_w, ln_b, packed, out, rows, n_factor, add_residual,
                                       eps, stream);
     else

@@ -79,10 +79,10 @@ def _same(t: Optional[torch.Tensor], like: torch.Tensor, name: str) -> Optional[
 
 def compute_dtype(x: torch.Tensor) -> torch.dtype:
     """dtype the kernels' arithmetic, weights and workspaces take for rows `x`: x's own, or
-    bfloat16 for float32 rows of at most 128 channels under torch.autocast(bfloat16) - the
+    bfloat16 for float32 rows of 64, 128 or 256 channels under torch.autocast(bfloat16) - the
     fused fp32-residual-stream mode (PTX_MIXED of the C ABI)."""
     ac = autocast_compute_dtype(x)
-    if ac == torch.bfloat16 and x.shape[-1] in (64, 128):
+    if ac == torch.bfloat16 and x.shape[-1] in (64, 128, 256):
         return ac
     return x.dtype
 

@@ -102,10 +102,12 @@ class PairformerBlock(nn.Module):
     def _forward_autocast_unfused(self, s: Optional[torch.Tensor], z: torch.Tensor,
                                   pair_mask: Optional[torch.Tensor], ac: torch.dtype
                                   ) -> Tuple[Optional[torch.Tensor], torch.Tensor]:
-        """fp32 residual stream under torch.autocast for the widths without a fused fp32-row
-        kernel (c_z = 256): every update is computed by the kernels in the autocast dtype from
-        a rounded copy of z and added to the fp32 z (in place; z is private here).  Costs a
-        cast and an add pass per update on top of the fused path."""
+        """fp32 residual stream under torch.autocast where no fused fp32-row kernel applies (an
+        autocast dtype other than bfloat16 - the kernels' 16-bit arithmetic is bf16 - or a row
+        width outside 64 / 128 / 256): every update is computed by the kernels in the autocast
+        dtype from a rounded copy of z and added to the fp32 z (in place; z is private here).
+        Costs a cast and an add pass per update on top of the fused path; widths and dtypes the
+        kernels do not take at all are refused by them."""
         m = None if pair_mask is None else pair_mask.to(ac)
         z.add_(self.tri_mul_out(z.to(ac), mask=m))
         z.add_(self.tri_mul_in(z.to(ac), mask=m))

@@ -139,12 +139,11 @@ class Transition(nn.Module):
             assert _residual_out is not None and self.fuses_pair_bias(x, _pair_bias_w[2].shape[0])
             return ops.transition(x, self._weights(torch.bfloat16, x.device), self.n, add_residual=True,
                                   out=_residual_out, pair_bias_w=_pair_bias_w)
-        if _residual_new and _residual_out is None and (
-                self.c_in in (64, 128) or (self.c_in == 256 and x.dtype == torch.bfloat16)):
+        cd = ops.compute_dtype(x)     # bf16 for fp32 rows of 64 / 128 / 256 channels under bf16 autocast
+        fused = self.c_in in (64, 128) or (self.c_in == 256 and cd == torch.bfloat16)
+        if _residual_new and _residual_out is None and fused:
             _residual_out = torch.empty_like(x)
         add = _residual_out is not None or _residual_new
-        cd = ops.compute_dtype(x)     # bf16 for fp32 rows of <= 128 channels under bf16 autocast
-        fused = self.c_in in (64, 128) or (self.c_in == 256 and x.dtype == torch.bfloat16)
         if fused and (self.n * self.c_in) % 64 == 0:
             out = ops.transition(x, self._weights(cd, x.device), self.n, add_residual=add,
                                  out=_residual_out)

@@ -79,6 +79,30 @@ def test_stack_48_blocks_against_oracle(n):
     print("; ".join(report))
 
 
+def test_scaled_up_stack_cz256_at_depth():
+    """The scaled-up model's pair stack (c_z = 256, hidden_scale_up: 8 pair heads, c_hidden_mul =
+    256; configs_model_type.py:52-85, pairformer.py:76-78 of the reference) through 24 blocks
+    at N_token = 96: bf16 arithmetic on the fp32 residual stream (the fused fp32-row kernels
+    of this width) against the fp32 oracle."""
+    kw = dict(n_blocks=24, c_z=256, hidden_scale_up=True)
+    ref = O.seed_parameters_(O.PairformerStack(**kw)).eval()
+    with torch.no_grad():
+        for p in ref.parameters():
+            p.copy_(p.to(BF16).float())
+    st = P.PairformerStack(**kw)
+    st.load_state_dict(ref.state_dict())
+    st = st.to("cuda").eval()
+    s, z, pm = O.make_inputs(96, c_z=256, n_pad=6, dtype=BF16)
+    s, z, pm = s.float(), z.float(), pm.float()
+    with torch.no_grad():
+        want_s, want_z = ref(s, z, pm)
+        with torch.autocast("cuda", dtype=BF16):
+            got_s, got_z = st(s.cuda(), z.cuda(), pm.cuda())
+    ez, es = rel_err(got_z, want_z), rel_err(got_s, want_s)
+    print(f"c_z = 256, 24 blocks, N = 96, fp32 residual stream: z {ez:.2e} s {es:.2e}")
+    assert got_z.dtype == torch.float32 and ez <= TOL_BF16 and es <= TOL_BF16
+
+
 def test_block_n768_against_oracle():
     """One full PairformerBlock at the benchmark's N_token = 768 with 48 padded tokens, bf16
     throughout and bf16 on fp32 rows, against the fp32 oracle."""

@@ -145,10 +145,92 @@ def test_c_abi_refuses_mixed_where_no_kernel_is_built():
     # LayerNorm has no residual stream
     assert lib.ptx_layernorm_fwd(x.data_ptr(), None, None, y.data_ptr(), None, None, 8, 128, 1e-5,
                                  _lib.PTX_MIXED, st) == 1
-    # rows of 256 channels: bf16 throughout only
+    # rows of 256 channels: bf16 arithmetic only (PTX_BF16, PTX_MIXED), not fp32
     z = torch.randn(8, 8, 256, device="cuda")
-    w = torch.randn(16, 256, device="cuda", dtype=BF16)
+    w = torch.randn(16, 256, device="cuda")
     out = torch.empty(16, 8, 8, device="cuda")
     assert lib.ptx_pair_bias_fwd(z.data_ptr(), None, None, w.data_ptr(), out.data_ptr(), 8, 256, 16,
-                                 1, 1e-5, _lib.PTX_MIXED, st) == 2
+                                 1, 1e-5, _lib.PTX_F32, st) == 2
     assert b"256" in lib.ptx_last_error_string()
+    assert lib.ptx_pair_bias_fwd(z.data_ptr(), None, None, w.to(BF16).data_ptr(), out.data_ptr(), 8, 256, 16,
+                                 1, 1e-5, _lib.PTX_MIXED, st) == 0
+
+
+# ------------------------------------------------------------------ rows of 256 channels (hidden_scale_up)
+@pytest.mark.parametrize("cls", ["TriangleMultiplicationOutgoing", "TriangleMultiplicationIncoming"])
+@pytest.mark.parametrize("n,n_pad", [(64, 0), (100, 7), (37, 0)])
+def test_trimul_cz256(cls, n, n_pad):
+    ref, prod = _pair(getattr(O, cls), getattr(P, cls), 256, 256)
+    z = _z(n, 256)
+    mask = pad_mask(n, n_pad) if n_pad else None
+    mc = None if mask is None else mask.cuda()
+    with torch.no_grad():
+        want = ref(z, mask)
+        with _amp():
+            got = prod(z.cuda(), mc)
+            zc = z.cuda().clone()
+            got2 = prod(zc, mc, inplace_safe=True, _add_with_inplace=True)
+    assert got.dtype == BF16 and rel_err(got, want) <= TOL_BF16
+    assert got2.data_ptr() == zc.data_ptr() and got2.dtype == torch.float32
+    assert torch.equal(got2, z.cuda() + got.float())      # z + bf16(update), exactly
+
+
+@pytest.mark.parametrize("starting", [True, False])
+@pytest.mark.parametrize("n,n_pad", [(64, 0), (100, 7), (37, 5)])
+def test_triattn_cz256(starting, n, n_pad):
+    ref, prod = _pair(O.TriangleAttention, P.TriangleAttention, 256, 32, 8, starting=starting)
+    z = _z(n, 256)
+    mask = pad_mask(n, n_pad) if n_pad else None
+    mc = None if mask is None else mask.cuda()
+    with torch.no_grad():
+        want = ref(z, mask, chunk_size=64)
+        with _amp():
+            got = prod(z.cuda(), mc)
+            zc = z.cuda().clone()
+            got2 = prod._run(zc, mc, transposed=not starting, residual_inplace=True)
+    assert got.dtype == BF16 and rel_err(got, want) <= TOL_BF16
+    assert got2.dtype == torch.float32 and torch.equal(got2, z.cuda() + got.float())
+
+
+@pytest.mark.parametrize("shape,factor", [((1, 50, 50, 256), 4), ((3001, 256), 2)])
+def test_transition_cz256(shape, factor):
+    ref, prod = _pair(O.Transition, P.Transition, 256, factor)
+    x = torch.randn(*shape, generator=torch.Generator().manual_seed(11))
+    with torch.no_grad():
+        want = ref(x)
+        with _amp():
+            got = prod(x.cuda())
+            xc = x.cuda().clone()
+            got2 = prod(xc, _residual_out=xc)
+    assert got.dtype == BF16 and rel_err(got, want) <= TOL_BF16
+    assert got2.dtype == torch.float32 and torch.equal(got2, x.cuda() + got.float())
+
+
+@pytest.mark.parametrize("n_blocks", [1, 4])
+def test_stack_cz256_scaled_up_runs_on_the_fused_fp32_row_kernels(n_blocks):
+    """The scaled-up model (c_z = 256, hidden_scale_up: 8 pair heads, c_hidden_mul = 256;
+    configs_model_type.py:52-85, pairformer.py:76-78) with fp32 tensors and parameters under
+    bf16 autocast: against the oracle, with the kernel timer and a look at the allocator as
+    witnesses that no rounded copy of z and no separate add pass exist any more."""
+    kw = dict(n_blocks=n_blocks, c_z=256, hidden_scale_up=True)
+    ref, prod = _pair(O.PairformerStack, P.PairformerStack, **kw)
+    s, z, pm = O.make_inputs(72, c_z=256, n_pad=5)
+    with torch.no_grad():
+        want_s, want_z = ref(s, z, pm)
+        sc, zc, pc = s.cuda(), z.cuda(), pm.cuda()
+        ops.kernel_timer = {}
+        try:
+            with _amp():
+                got_s, got_z = prod(sc, zc, pc)
+            seen = {k: len(v) for k, v in ops.kernel_timer.items()}
+        finally:
+            ops.kernel_timer = None
+    assert got_z.dtype == torch.float32 and got_s.dtype == torch.float32
+    assert torch.equal(zc.cpu(), z)
+    assert rel_err(got_z, want_z) <= TOL_BF16 and rel_err(got_s, want_s) <= TOL_BF16
+    assert seen["trimul_project"] == 2 * n_blocks and seen["transition"] == n_blocks
+    # the fused path hands the fp32 rows themselves to the kernels
+    blk = prod.blocks[0]
+    assert ops.compute_dtype(zc) == zc.dtype      # (outside autocast: fp32 arithmetic, refused for this width)
+    with _amp():
+        assert ops.compute_dtype(zc) == BF16

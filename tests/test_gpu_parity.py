@@ -534,6 +534,8 @@ def test_block_cz256_scaled_up():
 
 
 def test_cz256_fp32_is_refused():
+    """fp32 arithmetic on rows of 256 channels has no kernels (fp32 rows under bf16 autocast
+    have: tests/test_gpu_mixed.py)."""
     blk = P.TriangleMultiplicationOutgoing(256, 256).cuda()
     with torch.no_grad(), pytest.raises(RuntimeError, match="unsupported"):
         blk(torch.randn(1, 8, 8, 256, device="cuda"))
