@@ -154,6 +154,11 @@ rowgemm_in_kernel(RowGemmInParams p) {
   constexpr bool kRegRes = MODE == kTriMulOut && sizeof(T) == 2 && KS <= 8;
   constexpr bool RES = IC::RES;
   constexpr int NW = IC::NW, SL = IC::SL, FPW = IC::FPW;
+  // K steps by which the weight fragments' LDS reads run ahead of their products (see the chunk
+  // body): one in the attention projection on rows of 128 channels, which has the registers
+  // (168 -> 164 us per launch; in the triangle-multiplication kernels, at the register limit,
+  // the ring's eight registers turn into spills: 161 -> 164 us)
+  constexpr int kWeightPrefetch = (RES && MODE == kTriAttnIn && RB == 1) ? 1 : 0;
   __shared__ V8 lds_w[IC::NFRAG][kWave];
   // Staging tiles per wave.  Resident: one (LDS is full of weights).  Otherwise one per
   // 32 x 32 result tile of a chunk: all tiles of a chunk are written, then all are read back
@@ -647,40 +652,45 @@ rowgemm_in_kernel(RowGemmInParams p) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[rb][t][r] = 0.0f;
 
-    if (chan_on_lanes) {
+    // Weight fragments are read from LDS PF K steps ahead of the products that use them (a
+    // ring of PF + 1 fragment pairs; PF = 0: each K step reads its own).  Left to the compiler,
+    // every K step is "read two fragments, wait for them, two products" on one pair of
+    // fragment registers.
+    constexpr int PF = kWeightPrefetch;
+    constexpr int NK0 = MODE == kTriMulOut ? SL : KS;   // K steps of tile 0; tile 1 has KS
+    V8 wr0[PF + 1], wr1[PF + 1];
 #pragma unroll
-      for (int kk = 0; kk < KS; ++kk) {
-        const V8 w0 = lds_w[wf0 + kk][lane];
-        const V8 w1 = lds_w[wf1 + kk][lane];
+    for (int d = 0; d < PF; ++d) {
+      wr0[d] = lds_w[wf0 + d][lane];
+      if (d < KS) wr1[d] = lds_w[wf1 + d][lane];
+    }
+#pragma unroll
+    for (int kk = 0; kk < NK0; ++kk) {
+      if (kk + PF < NK0) wr0[(kk + PF) % (PF + 1)] = lds_w[wf0 + kk + PF][lane];
+      if (kk + PF < KS) wr1[(kk + PF) % (PF + 1)] = lds_w[wf1 + kk + PF][lane];
+      if constexpr (PF > 0) __builtin_amdgcn_sched_barrier(0);
+      const V8 w0 = wr0[kk % (PF + 1)], w1 = wr1[kk % (PF + 1)];
+      if (chan_on_lanes) {
 #pragma unroll
         for (int rb = 0; rb < RB; ++rb) {
           mma32(acc[rb][0], xf.f[rb][kk], w0);
           mma32(acc[rb][1], xf.f[rb][kk], w1);
         }
-      }
-    } else if constexpr (MODE == kTriMulOut) {
-#pragma unroll
-      for (int kk = 0; kk < SL; ++kk) {
-        const V8 w0 = lds_w[wf0 + kk][lane];
+      } else if constexpr (MODE == kTriMulOut) {
 #pragma unroll
         for (int rb = 0; rb < RB; ++rb) mma32(acc[rb][0], w0, xf2.f[rb][kk]);   // W_z LN_out(x)
         if (kk < KS) {
-          const V8 w1 = lds_w[wf1 + kk][lane];
 #pragma unroll
           for (int rb = 0; rb < RB; ++rb) mma32(acc[rb][1], w1, xf.f[rb][kk]);  // W_g LN_in(z)
         }
-      }
-    } else {
-#pragma unroll
-      for (int kk = 0; kk < KS; ++kk) {
-        const V8 w0 = lds_w[wf0 + kk][lane];
-        const V8 w1 = lds_w[wf1 + kk][lane];
+      } else {
 #pragma unroll
         for (int rb = 0; rb < RB; ++rb) {
           mma32(acc[rb][0], w0, xf.f[rb][kk]);
           mma32(acc[rb][1], w1, xf.f[rb][kk]);
         }
       }
+      if constexpr (PF > 0) __builtin_amdgcn_sched_barrier(0);
     }
 
     // fp32: the next chunk's weights go to LDS now, before this chunk's stores are issued:
