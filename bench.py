@@ -40,8 +40,8 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 # HBM bytes per launch of the triangle-attention core at N_token = 768, bf16: a constant taken
 # from profiles/trunk_n768_fp32_residual_hbm_traffic.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # on this benchmark, calibrated against a plain elementwise kernel of known size), not measured
-# in this run.  Algorithmic: 594432 + 147456 KiB.
-TRIATTN_FWD_TRAFFIC_BYTES_N768 = (533719 + 147459) * 1024
+# in this run.  Algorithmic: 446976 + 147456 KiB.
+TRIATTN_FWD_TRAFFIC_BYTES_N768 = (521001 + 147459) * 1024
 TRAFFIC_SOURCE = "profiles/trunk_n768_fp32_residual_hbm_traffic.txt (rocprofv3 --pmc, not measured in this run)"
 
 
