@@ -73,7 +73,8 @@ def test_stack_48_blocks_against_oracle(n):
         got = _run(_product_stack(ref, mode), mode, s, z, pm, upto=(2, 48))
         for d in (2, 48):
             es, ez = rel_err(got[d][0], want[d][0]), rel_err(got[d][1], want[d][1])
-            report.append(f"{mode}@{d}: z {ez:.2e} s {es:.2e}")
+            known = "" if d in depths else " (KNOWN OUT OF TOLERANCE, not asserted: bf16 storage of the residual stream drifts)"
+            report.append(f"{mode}@{d}: z {ez:.2e} s {es:.2e}{known}")
             if d in depths:
                 assert ez <= tol and es <= tol, report
     print("; ".join(report))
