@@ -55,6 +55,7 @@ struct AttnAux {
   int64_t lh, li, lj;     // element strides of lse: head, row, query
   int row0, row_end;      // rows row0 .. row_end-1 are this launch's (a launch may cover a range)
   int n_keys;             // keys 0 .. n_keys-1 take part (n_keys <= n; the rest count as masked)
+  int q_begin, q_end;     // queries q_begin .. q_end-1 of every row are this launch's (q_begin % 32 == 0)
 };
 
 // Rows of the pair tensor handled by one wave: R = 1 or 2, chosen per launch (triattn_fwd_ex).
@@ -95,7 +96,7 @@ __global__ __launch_bounds__((NWQ * 64), (sizeof(T) == 2 ? (R == 1 ? 16 / NWQ : 
   const int i0 = ax.row0 + (int)((item / n_qtiles) % n_rowgroups) * R;   // first of this workgroup's R rows
   const int h = (int)(item / ((int64_t)n_qtiles * n_rowgroups));
 
-  const int q0 = (qt * NWQ + wave) * 32;   // first query of this wave
+  const int q0 = ax.q_begin + (qt * NWQ + wave) * 32;   // first query of this wave
   const int key_tiles = key_pitch >> 6;
   const int q_blocks = (n + 31) >> 5;
   const int nk = ax.n_keys;
@@ -110,7 +111,7 @@ __global__ __launch_bounds__((NWQ * 64), (sizeof(T) == 2 ? (R == 1 ? 16 / NWQ : 
   // Lanes whose query lies beyond n compute on whatever the bias workspace holds there; they
   // store nothing, and they are kept out of the wave-wide decisions below so that the path a
   // wave takes (and with it the rounding of its valid queries) never depends on that content.
-  const bool q_ok = q0 + ln < n;
+  const bool q_ok = q0 + ln < ax.q_end;
   // (as a lane mask: wave-wide decisions are ballots of the condition alone, combined with this
   // mask on the scalar unit)
   const uint64_t q_ok_mask = __builtin_amdgcn_ballot_w64(q_ok);
@@ -436,10 +437,10 @@ __global__ __launch_bounds__((NWQ * 64), (sizeof(T) == 2 ? (R == 1 ? 16 / NWQ : 
   for (int r = 0; r < R; ++r) {
     const float l_tot = l_run[r] + swap32(l_run[r]);
     const float inv = fast_rcp(l_tot);
-    if (ax.lse && g == 0 && q0 + ln < n && i0 + r < ax.row_end)
+    if (ax.lse && g == 0 && q0 + ln < ax.q_end && i0 + r < ax.row_end)
       ax.lse[h * ax.lh + (int64_t)(i0 + r) * ax.li + (int64_t)qi_again * ax.lj] =
           m_run[r] * kLog2e + __builtin_amdgcn_logf(l_tot);   // v_log_f32 is log2
-    if (q0 + ln < n && i0 + r < ax.row_end) {
+    if (q0 + ln < ax.q_end && i0 + r < ax.row_end) {
 #pragma unroll
       for (int c = 0; c < 4; ++c) {
         f32x4 ov;
@@ -475,7 +476,7 @@ int triattn_fwd_ex(const T* q, const T* k, const T* vt, const T* g, const T* tri
                    int64_t sj, float* lse, int64_t lh, int64_t li, int64_t lj, int row_begin,
                    int row_count, int n_keys, hipStream_t stream) {
   if (n == 0 || n_rows == 0 || row_count == 0) return 0;
-  AttnAux ax = {sh, si, sj, n_rows, mask_is_bias, lse, lh, li, lj, row_begin, row_begin + row_count, n_keys};
+  AttnAux ax = {sh, si, sj, n_rows, mask_is_bias, lse, lh, li, lj, row_begin, row_begin + row_count, n_keys, 0, n};
   // 8-wave workgroups for long rows (measured: +2 % at n = 768, even at 1024, -2.6 % at 1536,
   // -2.2 % at 2048), where their 256 queries divide n or n is large enough for the idle waves
   // of the last one not to matter
@@ -487,38 +488,56 @@ int triattn_fwd_ex(const T* q, const T* k, const T* vt, const T* g, const T* tri
   // launch bounds and gets there without spills; with a mask the kernel needs 160 and loses a
   // wave; with four waves per workgroup the K / V tiles of two rows leave room for three
   // workgroups only: no gain).  Per launch: 395 -> 356 us at n = 768 in the trunk; in a loop of attention updates
-  // -7 % at n = 512, -3 % at 768, -11 % at 1536, -13 % at 2048, but +10 to +25 % where 256
-  // queries do not divide n (256, 384, 640) and waves of the last workgroup idle.
-  const bool r2 = sizeof(T) == 2 && !mask && n % 256 == 0 && n >= 512 && row_count >= 2;
-  const int n_qtiles = (wide || r2) ? (n + 255) / 256 : (n + 127) / 128;
-  const int R = r2 ? 2 : 1;
-  const int n_rowgroups = (row_count + R - 1) / R;
-  const int64_t total = (int64_t)heads * n_rowgroups * n_qtiles;
-  const int64_t per_xcd = (total + 7) / 8;
+  // -7 % at n = 512, -3 % at 768, -11 % at 1536, -13 % at 2048.  Where 256 queries do not divide
+  // n the idle waves of a last workgroup would cost more than the rows save (+10 to +25 % at
+  // 256, 384, 640): those launches cover the whole blocks of 256 queries only, and a second
+  // launch with one row per wave takes the remaining queries of every row (per update at
+  // n = 640: 269 -> 266 us, 1000: 1017 -> 987, 1100: 1328 -> 1241; a remainder of a few queries
+  // costs a launch that stages every row's keys for them: 211 -> 222 us at n = 520, so short
+  // remainders of short rows stay with one row per wave throughout).
+  const int q_rest = n % 256;
+  const bool r2 = sizeof(T) == 2 && !mask && n >= 512 && row_count >= 2 &&
+                  (q_rest == 0 || (n >= 640 && (q_rest >= 64 || n >= 1024)));
   const int mk = mask ? kMaskGiven : n_keys % kKeyTile ? kMaskTail : kMaskNone;
+  // one launch over the queries q_begin .. q_end-1 of the launch's rows
+  auto launch = [&](int q_begin, int q_end, bool two_rows, bool wide8) {
+    ax.q_begin = q_begin;
+    ax.q_end = q_end;
+    const int nq = q_end - q_begin;
+    const int n_qtiles = (two_rows || wide8) ? (nq + 255) / 256 : (nq + 127) / 128;
+    const int R = two_rows ? 2 : 1;
+    const int n_rowgroups = (row_count + R - 1) / R;
+    const int64_t total = (int64_t)heads * n_rowgroups * n_qtiles;
+    const int64_t per_xcd = (total + 7) / 8;
 #define PTX_ATTN_LAUNCH_R(RR, NWQ, MK)                                                            \
   triattn_fwd_kernel<T, RR, NWQ, MK><<<dim3((unsigned)(per_xcd * 8)), dim3(NWQ * 64), 0, stream>>>( \
       q, k, vt, g, tri_bias, mask, o, n, heads, key_pitch, mask_transposed, inf, n_qtiles,        \
       n_rowgroups, total, ax)
 #define PTX_ATTN_LAUNCH(NWQ, MK) PTX_ATTN_LAUNCH_R(1, NWQ, MK)
-  if (r2) {
-    if constexpr (sizeof(T) == 2) {
-      if (mk == kMaskTail) PTX_ATTN_LAUNCH_R(2, 8, kMaskTail);
-      else PTX_ATTN_LAUNCH_R(2, 8, kMaskNone);
+    if (two_rows) {
+      if constexpr (sizeof(T) == 2) {
+        if (mk == kMaskTail) PTX_ATTN_LAUNCH_R(2, 8, kMaskTail);
+        else PTX_ATTN_LAUNCH_R(2, 8, kMaskNone);
+      }
+    } else if (wide8) {
+      if (mk == kMaskGiven) PTX_ATTN_LAUNCH(8, kMaskGiven);
+      else if (mk == kMaskTail) PTX_ATTN_LAUNCH(8, kMaskTail);
+      else PTX_ATTN_LAUNCH(8, kMaskNone);
+    } else {
+      if (mk == kMaskGiven) PTX_ATTN_LAUNCH(4, kMaskGiven);
+      else if (mk == kMaskTail) PTX_ATTN_LAUNCH(4, kMaskTail);
+      else PTX_ATTN_LAUNCH(4, kMaskNone);
     }
-    return 0;
-  }
-  if (wide) {
-    if (mk == kMaskGiven) PTX_ATTN_LAUNCH(8, kMaskGiven);
-    else if (mk == kMaskTail) PTX_ATTN_LAUNCH(8, kMaskTail);
-    else PTX_ATTN_LAUNCH(8, kMaskNone);
-  } else {
-    if (mk == kMaskGiven) PTX_ATTN_LAUNCH(4, kMaskGiven);
-    else if (mk == kMaskTail) PTX_ATTN_LAUNCH(4, kMaskTail);
-    else PTX_ATTN_LAUNCH(4, kMaskNone);
-  }
 #undef PTX_ATTN_LAUNCH
 #undef PTX_ATTN_LAUNCH_R
+  };
+  if (r2) {
+    const int q_main = (n / 256) * 256;
+    launch(0, q_main, true, false);
+    if (q_main < n) launch(q_main, n, false, false);
+  } else {
+    launch(0, n, false, wide);
+  }
   return 0;
 }
 

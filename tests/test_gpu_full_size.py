@@ -29,6 +29,58 @@ def test_config2_triattn_start_n384_pad32():
     assert rel_err(got, want) <= TOL_BF16
 
 
+@pytest.mark.parametrize("mixed", [False, True])
+@pytest.mark.parametrize("starting", [True, False])
+@pytest.mark.parametrize("n,n_pad", [(520, 0), (600, 0), (640, 24), (777, 0), (777, 50)])
+def test_triattn_two_rows_per_wave_at_sizes_256_does_not_divide(mixed, starting, n, n_pad):
+    """From 512 tokens on, launches without a mask take two rows per wave in workgroups of 256
+    queries; where 256 does not divide N those cover the whole blocks of 256 queries and a
+    second launch (one row per wave) takes the remaining queries of every row.  Against the
+    oracle, with and without a padded tail (whose valid rows run over a prefix of the keys), and
+    against the same module with the mask handed to the kernels as it is (one row per wave)."""
+    from protenix_amd import ops
+    ref, prod = oracle_and_product(O.TriangleAttention, P.TriangleAttention, 128, 32, 4,
+                                   starting=starting, dtype=BF16)
+    z = _z(n, seed=n)
+    mask = pad_mask(n, n_pad, BF16) if n_pad else None
+    with torch.no_grad():
+        want = ref(z.float(), None if mask is None else mask.float(), chunk_size=64)
+    if mixed:
+        prod = prod.float()
+    zd = z.float().cuda() if mixed else z.cuda()
+    md = None if mask is None else mask.to(zd.dtype).cuda()
+
+    def run():
+        with torch.no_grad(), torch.autocast("cuda", dtype=BF16, enabled=mixed):
+            return prod(zd, md)
+    got = run()
+    assert rel_err(got, want) <= TOL_BF16
+    if mask is not None:
+        keep = ops.prefix_mask_enabled
+        ops.prefix_mask_enabled = False
+        ops._mask_cache.clear()
+        try:
+            plain = run()
+        finally:
+            ops.prefix_mask_enabled = keep
+            ops._mask_cache.clear()
+        assert rel_err(got, plain) <= 1e-2
+    else:
+        # the same rows through the masked kernels (an explicit mask of ones that is not
+        # recognised as such: one row per wave) give the same bits
+        keep = ops.mask_class
+        ones = torch.ones(1, n, n, dtype=zd.dtype, device="cuda")
+        ops.mask_class = lambda m: (False, None)
+        ops._mask_cache.clear()
+        try:
+            with torch.no_grad(), torch.autocast("cuda", dtype=BF16, enabled=mixed):
+                plain = prod(zd, ones)
+        finally:
+            ops.mask_class = keep
+            ops._mask_cache.clear()
+        assert torch.equal(got, plain)
+
+
 def test_triattn_n1536_pad40_wide_workgroups():
     """From 1536 tokens on the attention core runs 8-wave workgroups (256 queries share the
     staged key tiles): oracle parity at the smallest such size, ending node, padded."""
