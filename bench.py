@@ -55,6 +55,8 @@ def _work(n: int, z_bytes: int) -> dict:
         "triattn_fwd":     ("mfma", 512.0 * n ** 3),              # QK^T + PV, 4*N^3*H*D
         "trimul_contract": ("mfma", 256.0 * n ** 3),              # 2*N^3*c
         "transition":      ("mfma", 393216.0 * n * n),            # 3 GEMMs 128<->512, fused
+        # ending node's last stage (gate and output projection, 2 GEMMs 128x128) + transition, one launch
+        "triattn_output_transition": ("mfma", (393216.0 + 65536.0) * n * n),
         "trimul_project":  ("hbm", ez + 2.0 * e),                 # read z, write a and b
         "trimul_output":   ("hbm", e + 2.0 * ez),                 # read x and z, write z
         "triattn_project": ("hbm", ez + 3.0 * e),                 # read z, write q k v (+ bias); no gate tensor

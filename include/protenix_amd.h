@@ -353,6 +353,35 @@ PTX_API int ptx_transition_pair_bias_fwd(const void* x, const void* ln_w, const 
                                  int bias_f32, float pb_eps, int dtype, void* stream);
 
 /*
+ * The last stage of the ending-node triangle attention and the pair transition that follows
+ * it in a Pairformer block (pairformer.py:201-217: z = z + tri_att_end(z); z = z +
+ * pair_transition(z)), in one launch: what ptx_triattn_gate_output (add_residual = 1) followed
+ * by ptx_transition_fwd / ptx_transition_pair_bias_fwd (add_residual = 1) compute, bit for bit,
+ * without the pair tensor between the two travelling through memory (both stages are local to
+ * a pair position, and nothing else reads that tensor):
+ *   z' = z + W_o (sigmoid(W_g LN_att(z)) * o),   out = z' + transition(z')   [, bias from out]
+ * o: the attention core's output, head-major [4][n*n][32] (rows in the attention's logical
+ * order: with transposed = 1 row (i, j) belongs to z[j][i]); z, out [n][n][128] (out may be z).
+ * The weights of both stages are packed once per weight set:
+ *   ptx_triattn_output_transition_pack: w_g, w_o [128][128] of the attention, w_a, w_b
+ *     [n_factor*128][128], w_to [128][n_factor*128] of the transition -> packed,
+ *     ptx_triattn_output_transition_packed_elems(n_factor) elements.
+ * pb_w = NULL: no pair bias (bias, pb_* unused).  c_in = 128, heads = 4 (of 32); dtype
+ * PTX_BF16 or PTX_MIXED.
+ */
+PTX_API int64_t ptx_triattn_output_transition_packed_elems(int n_factor);
+PTX_API int ptx_triattn_output_transition_pack(const void* w_g, const void* w_o, const void* w_a,
+                                       const void* w_b, const void* w_to, void* packed,
+                                       int n_factor, int dtype, void* stream);
+PTX_API int ptx_triattn_output_transition_fwd(const void* o, const void* z, const void* att_ln_w,
+                                      const void* att_ln_b, const void* packed, const void* ln_w,
+                                      const void* ln_b, void* out, int n, int c_in, int heads,
+                                      int transposed, int n_factor, float att_eps, float eps,
+                                      const void* pb_ln_w, const void* pb_ln_b, const void* pb_w,
+                                      void* bias, int pb_heads, int bias_f32, float pb_eps,
+                                      int dtype, void* stream);
+
+/*
  * Pair bias of the single-representation attention (transformer.py:191-194):
  *   bias[h][i][j] = (W LN(z[i][j]))[h],  W [heads][c_z], heads <= 32, c_z = 128 or
  * (PTX_BF16, PTX_MIXED) 256.

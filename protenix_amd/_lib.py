@@ -49,6 +49,10 @@ SIGNATURES = {
     "ptx_transition_packed_elems": (_l, [_i, _i]),
     "ptx_transition_pack": (_i, [_p, _p, _p, _p, _i, _i, _i, _p]),
     "ptx_transition_fwd": (_i, [_p] * 5 + [_l, _i, _i, _i, _f, _i, _p]),
+    "ptx_triattn_output_transition_packed_elems": (_l, [_i]),
+    "ptx_triattn_output_transition_pack": (_i, [_p] * 6 + [_i, _i, _p]),
+    "ptx_triattn_output_transition_fwd": (_i, [_p] * 8 + [_i, _i, _i, _i, _i, _f, _f, _p, _p, _p, _p, _i, _i,
+                                               _f, _i, _p]),
     "ptx_transition_pair_bias_fwd": (_i, [_p] * 5 + [_l, _i, _i, _i, _f, _p, _p, _p, _p, _i, _i, _f, _i, _p]),
     "ptx_linear_fwd": (_i, [_p, _p, _p, _i, _p, _p, _p, _i, _l, _i, _i, _i, _i, _p]),
     "ptx_swiglu_fwd": (_i, [_p, _p, _p, _p, _i, _i, _i, _i, _p]),

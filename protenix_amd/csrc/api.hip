@@ -596,6 +596,68 @@ PTX_API int ptx_transition_pair_bias_fwd(const void* x, const void* ln_w, const 
   return after_launch("transition_pair_bias");
 }
 
+PTX_API int64_t ptx_triattn_output_transition_packed_elems(int n_factor) {
+  return n_factor > 0 ? ptx::triattn_output_transition_packed_elems(n_factor) : 0;
+}
+
+PTX_API int ptx_triattn_output_transition_pack(const void* w_g, const void* w_o, const void* w_a,
+                                               const void* w_b, const void* w_to, void* packed,
+                                               int n_factor, int dtype, void* stream) {
+  PTX_REQUIRE(dtype == PTX_BF16 || dtype == PTX_MIXED, PTX_ERR_UNSUPPORTED,
+              "triattn_output_transition_pack: built for PTX_BF16 and PTX_MIXED only (got dtype %d)", dtype);
+  PTX_REQUIRE(n_factor > 0 && n_factor <= 64 && (n_factor * 128) % 64 == 0, PTX_ERR_UNSUPPORTED,
+              "triattn_output_transition_pack: n_factor=%d", n_factor);
+  PTX_REQUIRE(w_g && w_o && w_a && w_b && w_to && packed, PTX_ERR_BAD_ARG,
+              "triattn_output_transition_pack: null pointer");
+  PTX_REQUIRE(aligned16(w_g) && aligned16(w_o) && aligned16(packed), PTX_ERR_BAD_ARG,
+              "triattn_output_transition_pack: w_g, w_o and packed must be 16-byte aligned");
+  const int rc = ptx::triattn_output_transition_pack<ptx::bf16_t>(w_g, w_o, w_a, w_b, w_to, packed, n_factor,
+                                                                (hipStream_t)stream);
+  PTX_REQUIRE(rc == 0, PTX_ERR_UNSUPPORTED, "triattn_output_transition_pack: not built for this type");
+  return after_launch("triattn_output_transition_pack");
+}
+
+PTX_API int ptx_triattn_output_transition_fwd(const void* o, const void* z, const void* att_ln_w,
+                                              const void* att_ln_b, const void* packed,
+                                              const void* ln_w, const void* ln_b, void* out, int n,
+                                              int c_in, int heads, int transposed, int n_factor,
+                                              float att_eps, float eps, const void* pb_ln_w,
+                                              const void* pb_ln_b, const void* pb_w, void* bias,
+                                              int pb_heads, int bias_f32, float pb_eps, int dtype,
+                                              void* stream) {
+  PTX_REQUIRE(dtype == PTX_BF16 || dtype == PTX_MIXED, PTX_ERR_UNSUPPORTED,
+              "triattn_output_transition: built for PTX_BF16 and PTX_MIXED only (got dtype %d)", dtype);
+  PTX_REQUIRE(n >= 0, PTX_ERR_BAD_ARG, "triattn_output_transition: n=%d", n);
+  PTX_REQUIRE(c_in == 128 && heads == 4, PTX_ERR_UNSUPPORTED,
+              "triattn_output_transition: only c_in = 128 with 4 heads of 32 is built (got c_in=%d heads=%d)",
+              c_in, heads);
+  PTX_REQUIRE(n_factor > 0 && n_factor <= 64 && (n_factor * 128) % 64 == 0, PTX_ERR_UNSUPPORTED,
+              "triattn_output_transition: n_factor=%d", n_factor);
+  PTX_REQUIRE(n < 32768, PTX_ERR_UNSUPPORTED, "triattn_output_transition: n=%d too large", n);
+  PTX_REQUIRE(!pb_w || (pb_heads >= 1 && pb_heads <= 32), PTX_ERR_UNSUPPORTED,
+              "triattn_output_transition: pair-bias heads=%d (1..32)", pb_heads);
+  if (n == 0) return PTX_OK;
+  PTX_REQUIRE(o && z && packed && out && (!pb_w || bias), PTX_ERR_BAD_ARG,
+              "triattn_output_transition: null pointer");
+  PTX_REQUIRE(aligned16(o) && aligned16(z) && aligned16(packed) && aligned16(out) &&
+                  (!att_ln_w || aligned16(att_ln_w)) && (!att_ln_b || aligned16(att_ln_b)) &&
+                  (!ln_w || aligned16(ln_w)) && (!ln_b || aligned16(ln_b)) &&
+                  (!pb_w || (aligned16(pb_w) && aligned16(bias))) &&
+                  (!pb_ln_w || aligned16(pb_ln_w)) && (!pb_ln_b || aligned16(pb_ln_b)),
+              PTX_ERR_BAD_ARG, "triattn_output_transition: pointers must be 16-byte aligned");
+  int rc;
+  if (dtype == PTX_MIXED)
+    rc = ptx::triattn_output_transition_fwd<ptx::bf16_t, float>(
+        o, z, att_ln_w, att_ln_b, packed, ln_w, ln_b, out, n, transposed, n_factor, att_eps, eps, pb_ln_w,
+        pb_ln_b, pb_w, bias, pb_heads, bias_f32, pb_eps, (hipStream_t)stream);
+  else
+    rc = ptx::triattn_output_transition_fwd<ptx::bf16_t, ptx::bf16_t>(
+        o, z, att_ln_w, att_ln_b, packed, ln_w, ln_b, out, n, transposed, n_factor, att_eps, eps, pb_ln_w,
+        pb_ln_b, pb_w, bias, pb_heads, bias_f32, pb_eps, (hipStream_t)stream);
+  PTX_REQUIRE(rc == 0, PTX_ERR_UNSUPPORTED, "triattn_output_transition: not built for this type");
+  return after_launch("triattn_output_transition");
+}
+
 PTX_API int ptx_linear_fwd(const void* x, const void* w, const void* bias, int bias_cols,
                            const void* res, void* out, void* out_t, int split_col, int64_t ldt,
                            int rows, int k, int n_out, int dtype, void* stream) {

@@ -60,6 +60,23 @@ int transition_pair_bias_fwd(const void* x, const void* ln_w, const void* ln_b, 
                              const void* pb_ln_w, const void* pb_ln_b, const void* pb_w,
                              void* bias, int heads, int bias_f32, float pb_eps,
                              hipStream_t stream);
+// The last stage of a triangle attention (as triattn_gate_output, residual added) and the pair
+// transition that follows it (as transition_fwd / transition_pair_bias_fwd, residual added) in
+// one launch on rows of 128 channels, 16-bit arithmetic: out = z' + transition(z'),
+// z' = z + W_o (sigmoid(W_g LN_att(z)) * o).  `packed` holds both stages' weights
+// (triattn_output_transition_pack); pb_w null: no pair bias.
+int64_t triattn_output_transition_packed_elems(int n_factor);
+template <typename T>
+int triattn_output_transition_pack(const void* w_g, const void* w_o, const void* w_a,
+                                   const void* w_b, const void* w_to, void* packed, int n_factor,
+                                   hipStream_t stream);
+template <typename T, typename TZ = T>
+int triattn_output_transition_fwd(const void* o, const void* z, const void* att_ln_w,
+                                  const void* att_ln_b, const void* packed, const void* ln_w,
+                                  const void* ln_b, void* out, int n, int transposed, int n_factor,
+                                  float att_eps, float eps, const void* pb_ln_w, const void* pb_ln_b,
+                                  const void* pb_w, void* bias, int heads, int bias_f32, float pb_eps,
+                                  hipStream_t stream);
 template <typename T, typename TZ = T>
 int pair_bias_fwd(const void* z, const void* ln_w, const void* ln_b, const void* w, void* bias,
                   int n, int c_z, int heads, int out_f32, float eps, hipStream_t stream);

@@ -109,11 +109,34 @@ struct PairBiasArgs {
   float eps;
 };
 
-template <typename T, int KS, typename TZ = T, bool PB = false>
+// AO: the last stage of a triangle attention in front of the transition,
+//   x' = x + W_o (sigmoid(W_g LN_att(x)) * o)                      (layers.py:380-396)
+//   out = x' + transition(x'),
+// on rows of 128 channels, 4 heads of 32, 16-bit arithmetic: the attention's update never
+// travels through memory as a pair tensor of its own (one write and one read of the residual
+// stream less than the two kernels one after the other).  The rows are addressed through a
+// RowMap (the ending node's output belongs at z[j][i]); x' exists in registers only, for the
+// LayerNorm of the transition, and is formed again in the epilogue from x and the attention's
+// update (kept in registers, rounded to T as the module's output is), with the roundings of
+// the two separate kernels.  The two weight matrices of the attention stage travel through
+// the chunk ring ahead of the transition's chunks, as three chunks of 24 fragments:
+//   fragments 0 .. 31: W_g, (head c, K step kk) at 8 c + kk; 32 .. 63: W_o, (block ob, kk);
+//   rows of a 32-row block permuted as in triattn_gate_out_kernel, so that accumulator
+//   registers 8 u .. 8 u + 7 of half-wave g are the channels 16 u + 8 g .. + 7 of the block:
+//   a lane's own fragment of K step 2 c + u.
+struct AttnOutArgs {
+  const void* o;             // attention output, head-major [4][n_rows][32], T, rows in logical order
+  const void *gamma, *beta;  // the attention's LayerNorm (either may be null)
+  RowMap zmap;               // logical row -> element offset of its row in x / out
+  float eps;
+};
+constexpr int kAoChunks = 3;   // chunks of 24 fragments that hold the 64 fragments of W_g and W_o
+
+template <typename T, int KS, typename TZ = T, bool PB = false, bool AO = false>
 __global__ __launch_bounds__((TrCfg<T, KS>::NW * 64), 2) void transition_fused_kernel(
     const TZ* x, const T* __restrict__ gamma, const T* __restrict__ beta,
     const T* __restrict__ packed, TZ* out, int64_t n_rows, int n_chunks, int add_residual,
-    float eps, PairBiasArgs pb) {
+    float eps, PairBiasArgs pb, AttnOutArgs ao) {
   typedef typename Vec8<T>::type V8;
   typedef typename VecE<TZ>::type VE_t;
   typedef TrCfg<T, KS> G;
@@ -121,6 +144,10 @@ __global__ __launch_bounds__((TrCfg<T, KS>::NW * 64), 2) void transition_fused_k
   constexpr bool MIXED = !std::is_same<T, TZ>::value;
   constexpr int RB = G::RB, NBUF = G::NBUF, D = G::D, PIECES = G::PIECES, FPW = G::FPW, NW = G::NW;
   constexpr int NOB = G::NOB, kTrFrags = G::FRAGS, kCx = 16 * KS;
+  static_assert(!AO || (KS == 8 && sizeof(T) == 2 && RB == 1 && D == 1),
+                "attention-output prologue: rows of 128 channels, 16-bit arithmetic");
+  constexpr int PRO = AO ? kAoChunks : 0;   // ring positions ahead of the transition's chunk 0
+  const int n_ring = n_chunks + PRO;
   __shared__ u32x4_t lds_w[NBUF][kTrFrags][PIECES][kWave];
   static_assert(sizeof(TZ) * NW * 32 * C::PITCH <= sizeof(u32x4_t) * (NBUF - 1) * kTrFrags * PIECES * kWave,
                 "the staging tiles reuse the chunk buffers");
@@ -146,8 +173,8 @@ __global__ __launch_bounds__((TrCfg<T, KS>::NW * 64), 2) void transition_fused_k
   // (address = wave-uniform base in scalar registers + this lane's offset inside a fragment:
   // no vector ALU work per load)
   const uint32_t lane_off = lane * 8 * (uint32_t)sizeof(T);
-  auto dma_chunk = [&](int j) {
-    const int jc = min(j, n_chunks - 1);
+  auto dma_chunk = [&](int j) {   // j: position in the ring (AO: the attention stage's chunks first)
+    const int jc = min(j, n_ring - 1);
     const int buf = j % NBUF;
     const uint64_t base = uniform64(
         (uint64_t)(packed + ((int64_t)jc * kTrFrags + wave * FPW) * kFragElems));
@@ -180,10 +207,98 @@ __global__ __launch_bounds__((TrCfg<T, KS>::NW * 64), 2) void transition_fused_k
   };
 
   // start the weight ring, then fetch and normalise this wave's rows
+  // (AO: the three chunks of the attention stage at once, into the three empty buffers - the
+  // prologue's steps are far shorter than a chunk's way from the L2, one chunk ahead would not do)
 #pragma unroll
-  for (int j = 0; j < D; ++j) dma_chunk(j);
+  for (int j = 0; j < (AO ? PRO : D); ++j) dma_chunk(j);
   RowFrags<T, RB, KS> xf;
-  load_rows<T, RB, true>(xf, x, RowMap{kCx, 0, 1}, row0, n_rows, gamma, beta, eps, lane);
+  V8 upd[AO ? KS : 1];   // AO: the attention's update of this lane's row, rounded to T
+  if constexpr (!AO) {
+    load_rows<T, RB, true>(xf, x, RowMap{kCx, 0, 1}, row0, n_rows, gamma, beta, eps, lane);
+  } else {
+    typedef typename Vec8<TZ>::type VZ;
+    const int n = lane & 31, g = lane >> 5;
+    const int64_t pr = row0 + n;
+    const int64_t prc = pr < n_rows ? pr : n_rows - 1;
+    const TZ* zp = x + ao.zmap(prc) + 8 * g;
+    f32x8 zr[KS];   // the raw row, then x'
+    V8 of[KS];      // the attention output of the row, then gated
+#pragma unroll
+    for (int kk = 0; kk < KS; ++kk) zr[kk] = to_f32(load8<TZ>(zp + 16 * kk));
+#pragma unroll
+    for (int kk = 0; kk < KS; ++kk)
+      of[kk] = load8<T>((const T*)ao.o + ((int64_t)(kk >> 1) * n_rows + prc) * 32 + 16 * (kk & 1) + 8 * g);
+    V8 xg[KS];
+    {
+      f32x8 v[KS];
+#pragma unroll
+      for (int kk = 0; kk < KS; ++kk) v[kk] = zr[kk];
+      normalize_row<T, KS>(v, (const T*)ao.gamma, (const T*)ao.beta, ao.eps, g, xg);
+    }
+    // gate of head c from the fragments at `f0` of a chunk buffer, applied to the attention
+    // output in place (both rounded to T like the reference's sigmoid(linear_g(x)) and o * g)
+    auto gate_head = [&](BufPtr b, int f0, int c) {
+      f32x16 accg;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) accg[r] = 0.0f;
+#pragma unroll
+      for (int kk = 0; kk < KS; ++kk) mma32(accg, read_frag(b, f0 + kk), xg[kk]);
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        const f32x8 ov = to_f32(of[2 * c + u]);
+        f32x8 gated;
+#pragma unroll
+        for (int t = 0; t < 8; ++t)
+          gated[t] = ov[t] * to_f32(from_f32<T>(sigmoidf_fast(accg[8 * u + t])));
+        of[2 * c + u] = from_f32<T>(gated);
+      }
+    };
+    // output block ob of the attention: the update rounded to T, then x' = x + update as stored
+    auto out_block = [&](BufPtr b, int f0, int ob) {
+      f32x16 acc;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
+#pragma unroll
+      for (int kk = 0; kk < KS; ++kk) mma32(acc, read_frag(b, f0 + kk), of[kk]);
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        f32x8 a8;
+#pragma unroll
+        for (int t = 0; t < 8; ++t) a8[t] = acc[8 * u + t];
+        upd[2 * ob + u] = from_f32<T>(a8);
+        const f32x8 uf = to_f32(upd[2 * ob + u]);
+        f32x8 v;
+#pragma unroll
+        for (int t = 0; t < 8; ++t) v[t] = zr[2 * ob + u][t] + uf[t];
+        zr[2 * ob + u] = to_f32(from_f32<TZ>(v));
+      }
+    };
+    // ring positions 0 .. 2 sit in buffers 0 .. 2; the transition's first chunk follows into
+    // buffer 0 once every wave is done with position 0, its second one (into buffer 1) is
+    // requested by the main loop's first step, behind a barrier that every wave reaches after
+    // its last read of positions 1 and 2
+    static_assert(!AO || (NBUF == 3 && PRO == 3), "one buffer per prologue chunk");
+    ring_barrier<0>();
+    {
+      const BufPtr b = buf_ptr(0);
+#pragma unroll
+      for (int c = 0; c < 3; ++c) gate_head(b, 8 * c, c);
+    }
+    ring_barrier<0>();
+    dma_chunk(PRO);
+    {
+      const BufPtr b = buf_ptr(1);
+      gate_head(b, 0, 3);
+      out_block(b, 8, 0);
+      out_block(b, 16, 1);
+    }
+    {
+      const BufPtr b = buf_ptr(2);
+      out_block(b, 0, 2);
+      out_block(b, 8, 3);
+    }
+    normalize_row<T, KS>(zr, gamma, beta, eps, g, xf.f[0]);
+  }
 
   f32x16 acc_o[RB][NOB];   // [row block][output column block]: lane <-> row, register <-> column
 #pragma unroll
@@ -256,7 +371,7 @@ __global__ __launch_bounds__((TrCfg<T, KS>::NW * 64), 2) void transition_fused_k
   // pass the barrier (loads complete in issue order; the only younger ones are chunks
   // j+1 .. j+D-1), and every wave has finished reading buffer (j-2) % NBUF, which the loads
   // of chunk j + D now refill.
-  auto iteration = [&](int j, f32x16 (&cur)[RB][2], f32x16 (&prev)[RB][2]) {
+  auto iteration = [&](int j, f32x16 (&cur)[RB][2], f32x16 (&prev)[RB][2]) {   // j: ring position
     ring_barrier<(D - 1) * G::DMA_PER_CHUNK>();
     dma_chunk(j + D);
     const BufPtr cbuf = buf_ptr(j % NBUF), pbuf = buf_ptr((j + NBUF - 1) % NBUF);
@@ -266,18 +381,18 @@ __global__ __launch_bounds__((TrCfg<T, KS>::NW * 64), 2) void transition_fused_k
 
   // chunk 0: GEMM1 only
   ring_barrier<(D - 1) * G::DMA_PER_CHUNK>();
-  dma_chunk(D);
+  dma_chunk(PRO + D);
   {
-    const BufPtr b0 = buf_ptr(0);
+    const BufPtr b0 = buf_ptr(PRO % NBUF);
     gemm1(std::false_type{}, b0, ab0, ab1, b0);
   }
   // chunks 1 .. n_chunks-1 (n_chunks is even): GEMM1(j), activation and GEMM2 of j-1
   int j = 1;
   for (; j + 1 < n_chunks; j += 2) {
-    iteration(j, ab1, ab0);
-    iteration(j + 1, ab0, ab1);
+    iteration(PRO + j, ab1, ab0);
+    iteration(PRO + j + 1, ab0, ab1);
   }
-  iteration(j, ab1, ab0);
+  iteration(PRO + j, ab1, ab0);
   // The residual vectors this lane will add in the epilogue, requested now so that their
   // latency passes under the drain (loading each one next to its store would serialise a
   // full memory round trip per tile: out may alias x, so no load could move above the
@@ -295,7 +410,8 @@ __global__ __launch_bounds__((TrCfg<T, KS>::NW * 64), 2) void transition_fused_k
       int mj, m0;
       stage_coord<TZ>(ps, lane, mj, m0);
       const int64_t pr = row0 + rb * 32 + mj;
-      obase[rb][ps] = pr < n_rows ? pr * kCx + m0 : -1;
+      if constexpr (AO) obase[rb][ps] = pr < n_rows ? ao.zmap(pr) + m0 : -1;
+      else obase[rb][ps] = pr < n_rows ? pr * kCx + m0 : -1;
     }
   auto load_residual = [&](int ob0) {
     if (add_residual) {
@@ -314,7 +430,7 @@ __global__ __launch_bounds__((TrCfg<T, KS>::NW * 64), 2) void transition_fused_k
 #pragma unroll
   for (int kk = 0; kk < KS; ++kk) act_part(kk, ab1);
   {
-    const BufPtr lbuf = buf_ptr((n_chunks - 1) % NBUF);
+    const BufPtr lbuf = buf_ptr((PRO + n_chunks - 1) % NBUF);
     gemm2(lbuf, read_frag(lbuf, 2 * KS));
   }
 
@@ -349,6 +465,29 @@ __global__ __launch_bounds__((TrCfg<T, KS>::NW * 64), 2) void transition_fused_k
 #pragma unroll
       for (int r = 0; r < 16; ++r)   // (mixed: the update is rounded to T before it is added)
         vals[r] = MIXED ? to_f32(from_f32<T>(acc_o[rb][ob][r])) : acc_o[rb][ob][r];
+      if constexpr (AO) {
+        // x' of the block's columns, as the attention stage would have stored it: its update
+        // goes from the fragment layout (lane <-> row, channels 16 u + 8 g .. + 7) through the
+        // staging tile to the layout of the stores and meets the raw row there
+        typedef typename Vec8<TZ>::type VZ;
+        const int n = lane & 31, g = lane >> 5;
+        wave_lds_sync();
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+          const VZ pk = from_f32<TZ>(to_f32(upd[2 * ob + u]));
+          u32x2* d2 = reinterpret_cast<u32x2*>(st + n * C::PITCH + 16 * u + 8 * g);
+          const u32x2* s2 = reinterpret_cast<const u32x2*>(&pk);
+#pragma unroll
+          for (int w8 = 0; w8 < (int)sizeof(VZ) / 8; ++w8) d2[w8] = s2[w8];
+        }
+        wave_lds_sync();
+#pragma unroll
+        for (int ps = 0; ps < C::NPASS; ++ps) {
+          int mj, m0;
+          stage_coord<TZ>(ps, lane, mj, m0);
+          resv[rb][ob % GOB][ps] = add_vec<TZ>(stage_get_vec<TZ>(st, mj, m0), resv[rb][ob % GOB][ps]);
+        }
+      }
       wave_lds_sync();
       stage_put<TZ>(st, vals, lane);
       wave_lds_sync();
@@ -436,12 +575,14 @@ __global__ __launch_bounds__((TrCfg<T, KS>::NW * 64), 2) void transition_fused_k
     }
     const int64_t pr = row0 + n;
     if (pr < n_rows) {
+      // (AO: the bias is indexed like the tensor's rows in memory)
+      const int64_t prm = AO ? ao.zmap(pr) / kCx : pr;
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int head = acc_row(r, g);
         if (head < pb.heads) {
-          if (pb.out_f32) ((float*)pb.out)[(int64_t)head * n_rows + pr] = accb[r];
-          else ((T*)pb.out)[(int64_t)head * n_rows + pr] = from_f32<T>(accb[r]);
+          if (pb.out_f32) ((float*)pb.out)[(int64_t)head * n_rows + prm] = accb[r];
+          else ((T*)pb.out)[(int64_t)head * n_rows + prm] = from_f32<T>(accb[r]);
         }
       }
     }
@@ -475,7 +616,7 @@ static int transition_fwd_ks(const void* x, const void* ln_w, const void* ln_b, 
   const int64_t blocks = (rows + rows_per_block - 1) / rows_per_block;
   transition_fused_kernel<T, KS, TZ, false><<<dim3((unsigned)blocks), dim3(TrCfg<T, KS>::NW * 64), 0, stream>>>(
       (const TZ*)x, (const T*)ln_w, (const T*)ln_b, (const T*)packed, (TZ*)out, rows,
-      16 * KS * n_factor / 32, add_residual, eps, PairBiasArgs{});
+      16 * KS * n_factor / 32, add_residual, eps, PairBiasArgs{}, AttnOutArgs{});
   return 0;
 }
 
@@ -494,10 +635,89 @@ int transition_pair_bias_fwd(const void* x, const void* ln_w, const void* ln_b, 
     const PairBiasArgs pb = {pb_ln_w, pb_ln_b, pb_w, bias, heads, bias_f32, pb_eps};
     transition_fused_kernel<T, KS, TZ, true><<<dim3((unsigned)blocks), dim3(TrCfg<T, KS>::NW * 64), 0, stream>>>(
         (const TZ*)x, (const T*)ln_w, (const T*)ln_b, (const T*)packed, (TZ*)out, rows,
-        16 * KS * n_factor / 32, add_residual, eps, pb);
+        16 * KS * n_factor / 32, add_residual, eps, pb, AttnOutArgs{});
     return 0;
   } else {
     return 1;   // 16-bit arithmetic only (the caller checks)
+  }
+}
+
+// The 64 fragments of the attention stage's W_g and W_o, in the order the prologue reads them
+// (see AttnOutArgs), padded to kAoChunks whole chunks.
+template <typename T>
+__global__ void attn_out_pack_kernel(const T* __restrict__ w_g, const T* __restrict__ w_o,
+                                     T* __restrict__ packed) {
+  constexpr int kFrags = kAoChunks * TrCfg<T, 8>::FRAGS;
+  const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= kFrags * kWave) return;
+  const int lane = idx & 63, f = idx >> 6;
+  const int m = lane & 31, g = lane >> 5;
+  typename Vec8<T>::type v;
+#pragma unroll
+  for (int t = 0; t < 8; ++t) v[t] = (T)0.0f;
+  if (f < 64) {
+    const T* w = f < 32 ? w_g : w_o;
+    const int cb = (f & 31) >> 3, kk = f & 7;
+    const int row = 32 * cb + 16 * (m >> 4) + 8 * ((m >> 2) & 1) + 4 * ((m >> 3) & 1) + (m & 3);
+    v = load8<T>(w + (int64_t)row * 128 + 16 * kk + 8 * g);
+  }
+  store8<T>(packed + (int64_t)idx * 8, v);
+}
+
+int64_t triattn_output_transition_packed_elems(int n_factor) {
+  return (int64_t)kAoChunks * 24 * kFragElems + (int64_t)3 * n_factor * 128 * 128;
+}
+
+template <typename T>
+int triattn_output_transition_pack(const void* w_g, const void* w_o, const void* w_a,
+                                   const void* w_b, const void* w_to, void* packed, int n_factor,
+                                   hipStream_t stream) {
+  if constexpr (sizeof(T) == 2) {
+    constexpr int total = kAoChunks * TrCfg<T, 8>::FRAGS * kWave;
+    attn_out_pack_kernel<T><<<dim3((total + 255) / 256), dim3(256), 0, stream>>>(
+        (const T*)w_g, (const T*)w_o, (T*)packed);
+    return transition_pack_ks<T, 8>(w_a, w_b, w_to, (T*)packed + (int64_t)kAoChunks * 24 * kFragElems,
+                                    n_factor, stream);
+  } else {
+    return 1;
+  }
+}
+
+template <typename T, typename TZ>
+int triattn_output_transition_fwd(const void* o, const void* z, const void* att_ln_w,
+                                  const void* att_ln_b, const void* packed, const void* ln_w,
+                                  const void* ln_b, void* out, int n, int transposed, int n_factor,
+                                  float att_eps, float eps, const void* pb_ln_w, const void* pb_ln_b,
+                                  const void* pb_w, void* bias, int heads, int bias_f32, float pb_eps,
+                                  hipStream_t stream) {
+  if (n == 0) return 0;
+  if constexpr (sizeof(T) == 2) {
+    constexpr int KS = 8;
+    const int64_t rows = (int64_t)n * n;
+    const int64_t rows_per_block = TrCfg<T, KS>::NW * 32;
+    const int64_t blocks = (rows + rows_per_block - 1) / rows_per_block;
+    AttnOutArgs ao = {};
+    ao.o = o;
+    ao.gamma = att_ln_w;
+    ao.beta = att_ln_b;
+    ao.zmap.n_inner = n;
+    ao.zmap.stride_outer = transposed ? 128 : (int64_t)n * 128;
+    ao.zmap.stride_inner = transposed ? (int64_t)n * 128 : 128;
+    ao.eps = att_eps;
+    const int n_chunks = 16 * KS * n_factor / 32;
+    if (pb_w) {
+      const PairBiasArgs pb = {pb_ln_w, pb_ln_b, pb_w, bias, heads, bias_f32, pb_eps};
+      transition_fused_kernel<T, KS, TZ, true, true><<<dim3((unsigned)blocks), dim3(TrCfg<T, KS>::NW * 64), 0, stream>>>(
+          (const TZ*)z, (const T*)ln_w, (const T*)ln_b, (const T*)packed, (TZ*)out, rows, n_chunks, 1, eps,
+          pb, ao);
+    } else {
+      transition_fused_kernel<T, KS, TZ, false, true><<<dim3((unsigned)blocks), dim3(TrCfg<T, KS>::NW * 64), 0, stream>>>(
+          (const TZ*)z, (const T*)ln_w, (const T*)ln_b, (const T*)packed, (TZ*)out, rows, n_chunks, 1, eps,
+          PairBiasArgs{}, ao);
+    }
+    return 0;
+  } else {
+    return 1;
   }
 }
 
@@ -521,6 +741,17 @@ int transition_fwd(const void* x, const void* ln_w, const void* ln_b, const void
                                  stream);
 }
 
+template int triattn_output_transition_pack<bf16_t>(const void*, const void*, const void*,
+                                                    const void*, const void*, void*, int,
+                                                    hipStream_t);
+#define PTX_INSTANTIATE_AOT(TZ)                                                                    \
+  template int triattn_output_transition_fwd<bf16_t, TZ>(                                          \
+      const void*, const void*, const void*, const void*, const void*, const void*, const void*,   \
+      void*, int, int, int, float, float, const void*, const void*, const void*, void*, int, int,  \
+      float, hipStream_t);
+PTX_INSTANTIATE_AOT(bf16_t)
+PTX_INSTANTIATE_AOT(float)
+#undef PTX_INSTANTIATE_AOT
 template int transition_pack<float>(const void*, const void*, const void*, void*, int, int,
                                     hipStream_t);
 template int transition_pack<bf16_t>(const void*, const void*, const void*, void*, int, int,

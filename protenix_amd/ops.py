@@ -350,13 +350,48 @@ def triangle_multiplicative_update(x: torch.Tensor, incoming: bool, mask: Option
 late_gate_enabled = True
 
 
+# The ending node's last stage and the pair transition behind it as one launch where the
+# late-gate kernels apply (see triangle_attention(then_transition=...)).  False: two launches
+# (tests compare the two, bit for bit).
+fuse_attention_transition = True
+
+
+def attention_transition_pack(w_g: torch.Tensor, w_o: torch.Tensor, w_a: torch.Tensor,
+                              w_b: torch.Tensor, w_to: torch.Tensor) -> torch.Tensor:
+    """Packs the attention's gate and output weights [128, 128] and the three Transition weights
+    (c = 128, bf16) into the streaming order of the fused launch."""
+    _dev(w_g, "w_g")
+    lib = _lib.load()
+    n_factor = w_a.shape[0] // w_a.shape[1]
+    packed = torch.empty((lib.ptx_triattn_output_transition_packed_elems(n_factor),), dtype=w_g.dtype,
+                         device=w_g.device)
+    with torch.cuda.device(w_g.device):
+        _call("transition_pack", lib.ptx_triattn_output_transition_pack, _ptr(w_g.contiguous()),
+              _ptr(w_o.contiguous()), _ptr(w_a.contiguous()), _ptr(w_b.contiguous()),
+              _ptr(w_to.contiguous()), _ptr(packed), n_factor, _dt(w_g), _stream())
+    return packed
+
+
+def fuses_attention_transition(z: torch.Tensor, heads: int, d: int, n_factor: int) -> bool:
+    """Whether triangle_attention(then_transition=...) is available for rows `z`."""
+    return (fuse_attention_transition and late_gate_enabled and z.is_cuda and z.shape[-1] == 128
+            and heads == 4 and d == 32 and compute_dtype(z) == torch.bfloat16
+            and (n_factor * 128) % 64 == 0 and n_factor <= 64)
+
+
 def triangle_attention(z: torch.Tensor, mask: Optional[torch.Tensor], w: dict, heads: int, d: int,
                        inf: float, transposed: bool, add_residual: bool,
-                       out: Optional[torch.Tensor] = None, eps: float = 1e-5) -> torch.Tensor:
+                       out: Optional[torch.Tensor] = None, eps: float = 1e-5,
+                       then_transition: Optional[dict] = None):
     """Starting-node attention over z (transposed=False) or over z^T with the
     result written back transposed (transposed=True), i.e. the ending node as
     the Pairformer block uses it, without materialising z^T.  `mask` is indexed
-    like z: the key mask of logical row i is mask[i, :] (or mask[:, i])."""
+    like z: the key mask of logical row i is mask[i, :] (or mask[:, i]).
+    `then_transition` (with add_residual, where fuses_attention_transition() holds): the pair
+    transition that follows, {"packed": attention_transition_pack(...), "ln_w", "ln_b",
+    "n_factor", "pair_bias_w": (ln_w, ln_b, w [heads, 128]) or None}; the result is then
+    out = z' + transition(z') with z' = z + attention(z), from the launch that forms z', and
+    the return value (out, fp32 pair bias [heads, n*n] of out or None)."""
     _dev(z, "z")
     lib = _lib.load()
     n, c = z.shape[0], z.shape[-1]
@@ -399,6 +434,20 @@ def triangle_attention(z: torch.Tensor, mask: Optional[torch.Tensor], w: dict, h
         del q, k, vt, tb
         if out is None:
             out = torch.empty_like(z)
+        if then_transition is not None:
+            assert late_gate and add_residual
+            tt = then_transition
+            pbw = tt.get("pair_bias_w")
+            bias = None
+            if pbw is not None:
+                bias = torch.empty((pbw[2].shape[0], n * n), dtype=torch.float32, device=dev)
+            _call("triattn_output_transition", lib.ptx_triattn_output_transition_fwd, _ptr(g), _ptr(z),
+                  _ptr(w["ln_w"]), _ptr(w["ln_b"]), _ptr(tt["packed"]), _ptr(tt["ln_w"]), _ptr(tt["ln_b"]),
+                  _ptr(out), n, c, heads, int(transposed), tt["n_factor"], eps, eps,
+                  _ptr(pbw[0]) if pbw else None, _ptr(pbw[1]) if pbw else None,
+                  _ptr(pbw[2].contiguous()) if pbw else None, _ptr(bias), 0 if pbw is None else pbw[2].shape[0],
+                  1, eps, dt, st)
+            return out, bias
         if late_gate:
             _call("triattn_output", lib.ptx_triattn_gate_output, _ptr(g), _ptr(z), _ptr(w["ln_w"]),
                   _ptr(w["ln_b"]), _ptr(w["w_g"]), _ptr(w["w_o"]), _ptr(out), n, c, heads,

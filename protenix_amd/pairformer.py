@@ -16,7 +16,7 @@ import torch
 import torch.nn as nn
 
 from . import ops
-from .primitives import Transition
+from .primitives import Transition, _WeightCache, _cv
 from .transformer import AttentionPairBias
 from .triangular import (TriangleAttention, TriangleMultiplicationIncoming,
                          TriangleMultiplicationOutgoing)
@@ -40,6 +40,7 @@ class PairformerBlock(nn.Module):
                                              no_heads=no_heads_pair)
         self.p_drop = dropout
         self.pair_transition = Transition(c_in=c_z, n=num_intermediate_factor)
+        self._fused_cache = _WeightCache()
         self.c_s = c_s
         if self.c_s > 0:
             self.attention_pair_bias = AttentionPairBias(has_s=False, create_offset_ln_z=True,
@@ -83,6 +84,31 @@ class PairformerBlock(nn.Module):
         self.tri_att_start._run(z, pair_mask, transposed=False, residual_inplace=True)
         # ending node: the starting-node module of the reference applied to z^T with
         # mask^T, expressed through transposed addressing of z and mask
+        apb = self.attention_pair_bias if want_bias else None
+        att, tr = self.tri_att_end, self.pair_transition
+        if (z.is_contiguous() and tr.c_in == att.c_in
+                and ops.fuses_attention_transition(z, att.no_heads, att.c_hidden, tr.n)
+                and (apb is None or apb.n_heads <= 32)):
+            # the ending node's last stage and the transition (and the pair bias) in one launch:
+            # the tensor between the two never travels through memory
+            def fused_weights(cd, device):
+                ps = (att.mha.linear_g.weight, att.mha.linear_o.weight, tr.layernorm1.weight,
+                      tr.layernorm1.bias, tr.linear_no_bias_a.weight, tr.linear_no_bias_b.weight,
+                      tr.linear_no_bias.weight)
+                def make():
+                    w_g, w_o, ln_w, ln_b, w_a, w_b, w_to = (_cv(p, cd, device) for p in ps)
+                    return {"packed": ops.attention_transition_pack(w_g, w_o, w_a, w_b, w_to),
+                            "ln_w": ln_w, "ln_b": ln_b, "n_factor": tr.n}
+                tt = dict(self._fused_cache.get(ps, cd, device, make))
+                tt["pair_bias_w"] = None if apb is None else apb.pair_bias_weights(z)
+                return tt
+            _, biases = att._run(z, pair_mask, transposed=True, residual_inplace=True,
+                                 then_transition=fused_weights)
+            if apb is None:
+                return None
+            n = z.shape[-2]
+            bias = biases[0] if len(biases) == 1 else torch.stack(biases)
+            return bias.view(*z.shape[:-3], apb.n_heads, n, n)
         self.tri_att_end._run(z, pair_mask, transposed=True, residual_inplace=True)
         if not want_bias:
             self.pair_transition(z, _residual_out=z)

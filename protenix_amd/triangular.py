@@ -216,10 +216,24 @@ class TriangleAttention(nn.Module):
                                lambda: dict(zip(names, (_cv(p, dtype, device) for p in ps))))
 
     def _run(self, x: torch.Tensor, mask: Optional[torch.Tensor], transposed: bool,
-             residual_inplace: bool) -> torch.Tensor:
+             residual_inplace: bool, then_transition=None):
+        """`then_transition`: a callable (arithmetic dtype, device) -> the dict of
+        ops.triangle_attention(then_transition=...), for a contiguous x updated in place where
+        ops.fuses_attention_transition() holds; the result is then (x, list of pair biases or
+        Nones, one per pair tensor of the batch)."""
         _forward_only(x, module=self)
         x_in = x
         x, cd, cast_back = _stream_and_compute_dtype(x, self.c_in)
+        if then_transition is not None:
+            assert residual_inplace and x is x_in and x.is_contiguous()
+            w = self._weights(cd, x.device)
+            tt = then_transition(cd, x.device)
+            xb, mb = _per_batch(x, mask)
+            biases = [ops.triangle_attention(xb[bi], None if mb is None else mb[bi], w, self.no_heads,
+                                             self.c_hidden, self.inf, transposed=transposed,
+                                             add_residual=True, out=xb[bi], then_transition=tt)[1]
+                      for bi in range(xb.shape[0])]
+            return x, biases
         if residual_inplace and x is not x_in:
             # rows rounded for the kernels: the update is added to the caller's own rows
             return x_in.add_(self._run(x_in, mask, transposed, residual_inplace=False))
