@@ -114,8 +114,11 @@ struct PairBiasArgs {
 //   out = x' + transition(x'),
 // on rows of 128 channels, 4 heads of 32, 16-bit arithmetic: the attention's update never
 // travels through memory as a pair tensor of its own (one write and one read of the residual
-// stream less than the two kernels one after the other).  The rows are addressed through a
-// RowMap (the ending node's output belongs at z[j][i]); x' exists in registers only, for the
+// stream less than the two kernels one after the other).  The kernel walks the rows of x in
+// memory order, like the transition alone, and finds a row's attention output through a RowMap
+// (the ending node's output for z[a][b] is row (b, a) of o: 64-byte pieces per head, where
+// walking o's order instead would scatter the rows of x and, four bytes at a time, the pair
+// bias: measured as 1.6 times the bytes written); x' exists in registers only, for the
 // LayerNorm of the transition, and is formed again in the epilogue from x and the attention's
 // update (kept in registers, rounded to T as the module's output is), with the roundings of
 // the two separate kernels.  The two weight matrices of the attention stage travel through
@@ -125,9 +128,9 @@ struct PairBiasArgs {
 //   registers 8 u .. 8 u + 7 of half-wave g are the channels 16 u + 8 g .. + 7 of the block:
 //   a lane's own fragment of K step 2 c + u.
 struct AttnOutArgs {
-  const void* o;             // attention output, head-major [4][n_rows][32], T, rows in logical order
+  const void* o;             // attention output, head-major [4][n_rows][32], T, rows in the attention's order
   const void *gamma, *beta;  // the attention's LayerNorm (either may be null)
-  RowMap zmap;               // logical row -> element offset of its row in x / out
+  RowMap omap;               // row of x -> element offset of its 32 channels inside a head's plane of o
   float eps;
 };
 constexpr int kAoChunks = 3;   // chunks of 24 fragments that hold the 64 fragments of W_g and W_o
@@ -156,6 +159,15 @@ __global__ __launch_bounds__((TrCfg<T, KS>::NW * 64), 2) void transition_fused_k
   // Workgroups take the rows back to front: the kernel before this one wrote the pair tensor
   // front to back, and its tail is what the memory-side cache still holds.
   const int64_t row0 = ((int64_t)(gridDim.x - 1 - blockIdx.x) * NW + wave) * (RB * 32);
+  // Row m (0 .. 32 RB - 1) of this wave's tile in x / out, or -1.
+  // (AO: tiles of two neighbouring rows a of the pair tensor times 16 positions b, so that the
+  // 64-byte pieces of o for (a, b) and (a + 1, b) - rows (b, a) and (b, a + 1) of an ending
+  // node's output, one 128-byte line - are read by the same wave, halved the kernel's fetches
+  // of o and took 408 instead of 403 us: not used.)
+  auto row_at = [&](int m) -> int64_t {
+    const int64_t pr = row0 + m;
+    return pr < n_rows ? pr : -1;
+  };
 
   // PB: the bias' LayerNorm parameters as fp32, parked in LDS for the epilogue: fetched there
   // from global memory they would cost every tile a round trip that nothing hides.  (Visible
@@ -218,16 +230,17 @@ __global__ __launch_bounds__((TrCfg<T, KS>::NW * 64), 2) void transition_fused_k
   } else {
     typedef typename Vec8<TZ>::type VZ;
     const int n = lane & 31, g = lane >> 5;
-    const int64_t pr = row0 + n;
-    const int64_t prc = pr < n_rows ? pr : n_rows - 1;
-    const TZ* zp = x + ao.zmap(prc) + 8 * g;
+    const int64_t pr = row_at(n);
+    const int64_t prc = pr >= 0 ? pr : n_rows - 1;
+    const TZ* zp = x + prc * kCx + 8 * g;
+    const T* op = (const T*)ao.o + ao.omap(prc) + 8 * g;
     f32x8 zr[KS];   // the raw row, then x'
     V8 of[KS];      // the attention output of the row, then gated
 #pragma unroll
     for (int kk = 0; kk < KS; ++kk) zr[kk] = to_f32(load8<TZ>(zp + 16 * kk));
 #pragma unroll
     for (int kk = 0; kk < KS; ++kk)
-      of[kk] = load8<T>((const T*)ao.o + ((int64_t)(kk >> 1) * n_rows + prc) * 32 + 16 * (kk & 1) + 8 * g);
+      of[kk] = load8<T>(op + (int64_t)(kk >> 1) * n_rows * 32 + 16 * (kk & 1));
     V8 xg[KS];
     {
       f32x8 v[KS];
@@ -409,9 +422,8 @@ __global__ __launch_bounds__((TrCfg<T, KS>::NW * 64), 2) void transition_fused_k
     for (int ps = 0; ps < C::NPASS; ++ps) {
       int mj, m0;
       stage_coord<TZ>(ps, lane, mj, m0);
-      const int64_t pr = row0 + rb * 32 + mj;
-      if constexpr (AO) obase[rb][ps] = pr < n_rows ? ao.zmap(pr) + m0 : -1;
-      else obase[rb][ps] = pr < n_rows ? pr * kCx + m0 : -1;
+      const int64_t pr = row_at(rb * 32 + mj);
+      obase[rb][ps] = pr >= 0 ? pr * kCx + m0 : -1;
     }
   auto load_residual = [&](int ob0) {
     if (add_residual) {
@@ -573,16 +585,14 @@ __global__ __launch_bounds__((TrCfg<T, KS>::NW * 64), 2) void transition_fused_k
         mma32(accb, lds_pbw[4 * hb + u][lane], *reinterpret_cast<const V8*>(h2));   // lane <-> row, register <-> head
       }
     }
-    const int64_t pr = row0 + n;
-    if (pr < n_rows) {
-      // (AO: the bias is indexed like the tensor's rows in memory)
-      const int64_t prm = AO ? ao.zmap(pr) / kCx : pr;
+    const int64_t pr = row_at(n);
+    if (pr >= 0) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int head = acc_row(r, g);
         if (head < pb.heads) {
-          if (pb.out_f32) ((float*)pb.out)[(int64_t)head * n_rows + prm] = accb[r];
-          else ((T*)pb.out)[(int64_t)head * n_rows + prm] = from_f32<T>(accb[r]);
+          if (pb.out_f32) ((float*)pb.out)[(int64_t)head * n_rows + pr] = accb[r];
+          else ((T*)pb.out)[(int64_t)head * n_rows + pr] = from_f32<T>(accb[r]);
         }
       }
     }
@@ -700,9 +710,9 @@ int triattn_output_transition_fwd(const void* o, const void* z, const void* att_
     ao.o = o;
     ao.gamma = att_ln_w;
     ao.beta = att_ln_b;
-    ao.zmap.n_inner = n;
-    ao.zmap.stride_outer = transposed ? 128 : (int64_t)n * 128;
-    ao.zmap.stride_inner = transposed ? (int64_t)n * 128 : 128;
+    ao.omap.n_inner = n;
+    ao.omap.stride_outer = transposed ? 32 : (int64_t)n * 32;
+    ao.omap.stride_inner = transposed ? (int64_t)n * 32 : 32;
     ao.eps = att_eps;
     const int n_chunks = 16 * KS * n_factor / 32;
     if (pb_w) {
