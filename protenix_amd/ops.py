@@ -214,6 +214,37 @@ _class_cache: list = []     # (key, mask, (all ones, n_valid or None)), most rec
 capture_mask_class: Optional[tuple] = None
 
 
+# A mask whose class its maker knows (the pair stack's own padding of odd sizes): (mask, class),
+# looked up by identity, also while a graph is being recorded.
+_declared_mask: Optional[tuple] = None
+
+
+def declare_mask_class(mask: torch.Tensor, cls: tuple) -> None:
+    """Tells mask_class() the class of `mask` (a tensor built by the caller, who must not change
+    it afterwards and calls forget_mask() when done with it) so that nothing has to be looked at."""
+    global _declared_mask
+    _declared_mask = (mask, cls)
+
+
+def _is_declared(mask: torch.Tensor) -> bool:
+    # (the declared tensor itself, or the [n, n] view of it that the per-tensor loops of a batch of one make)
+    d = _declared_mask
+    return d is not None and (mask is d[0] or (
+        mask.dim() == 2 and mask.data_ptr() == d[0].data_ptr() and mask.numel() == d[0].numel()
+        and mask.is_contiguous()))
+
+
+def forget_mask(mask: torch.Tensor) -> None:
+    """Drops what is kept for a mask its maker is done with: a declared class, the cached class
+    and the cached converted copies (which hold the mask alive)."""
+    global _declared_mask
+    if _declared_mask is not None and _declared_mask[0] is mask:
+        _declared_mask = None
+    ptr = mask.untyped_storage().data_ptr()    # (entries may be views of it, one per pair tensor of a batch)
+    _class_cache[:] = [e for e in _class_cache if e[1].untyped_storage().data_ptr() != ptr]
+    _mask_cache[:] = [e for e in _mask_cache if e[1].untyped_storage().data_ptr() != ptr]
+
+
 def mask_class(mask: Optional[torch.Tensor]) -> tuple:
     """(all ones, n_valid) of a pair mask: n_valid is the number of valid tokens if the mask is
     [n, n] = m (x) m with m = n_valid ones followed by zeros (0 < n_valid < n), else None.
@@ -221,6 +252,8 @@ def mask_class(mask: Optional[torch.Tensor]) -> tuple:
     kept with the mask's storage, view geometry and version counter."""
     if mask is None:
         return (True, None)
+    if _is_declared(mask):
+        return _declared_mask[1]
     if mask.is_cuda and torch.cuda.is_current_stream_capturing():
         return capture_mask_class or (False, None)
     key = _mask_key(mask)
@@ -248,7 +281,11 @@ def mask_class(mask: Optional[torch.Tensor]) -> tuple:
 def padded_tail(mask: Optional[torch.Tensor], n: int) -> Optional[int]:
     """n_valid if the triangle attention treats this [n, n] mask as a padded tail (two launches:
     valid rows over valid keys without a mask, padded rows with it), else None."""
-    if mask is None or not prefix_mask_enabled or n < prefix_mask_min_n:
+    if mask is None or not prefix_mask_enabled:
+        return None
+    # (a declared mask - the pair stack's own padding of an odd size, a handful of rows - takes the
+    # two launches at any size: the valid rows then run exactly what the unpadded tensor would)
+    if n < prefix_mask_min_n and not _is_declared(mask):
         return None
     return mask_class(mask)[1]
 

@@ -98,3 +98,65 @@ def test_fused_launch_refusals():
         a[idx] = bad
         assert lib.ptx_triattn_output_transition_fwd(*a) != 0
     torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("mixed", [True, False])
+@pytest.mark.parametrize("n,n_pad", [(61, 0), (101, 0), (203, 0), (629, 0)])
+def test_sizes_padded_to_a_multiple_of_8(mixed, n, n_pad):
+    """N_token that 8 does not divide runs as the next multiple with the extra tokens masked
+    (protenix_amd.pairformer.pad_tokens_to): the same bits as the unpadded run, both
+    within tolerance of the oracle, inputs untouched / updated in place as asked."""
+    from protenix_amd import pairformer as pf
+    dt = torch.float32 if mixed else BF16
+    ref, prod = oracle_and_product(O.PairformerStack, P.PairformerStack, n_blocks=2, dtype=BF16)
+    prod = prod.to(dt)
+    s, z, pm = O.make_inputs(n, n_pad=n_pad, dtype=BF16)
+    pmd = pm.cuda() if n == 101 else None       # (a mask of all ones, or none)
+    with torch.no_grad():
+        s_ref, z_ref = ref(s.float(), z.float(), pm.float(), chunk_size=128 if n > 256 else None)
+    outs = {}
+    for pad_to in (8, 0):
+        keep = pf.pad_tokens_to, pf.pad_tokens_min_n
+        pf.pad_tokens_to, pf.pad_tokens_min_n = pad_to, 0
+        try:
+            zd = z.to("cuda", dt)
+            z_before = zd.clone()
+            with torch.no_grad(), torch.autocast("cuda", dtype=BF16, enabled=mixed):
+                s_o, z_o = prod(s.to("cuda", dt), zd, pmd)
+                assert torch.equal(zd, z_before) and z_o.shape == zd.shape and z_o.is_contiguous()
+                s_i, z_i = prod(s.to("cuda", dt), zd, pmd, inplace_safe=True)
+                assert z_i is zd and torch.equal(z_i, z_o) and torch.equal(s_i, s_o)
+            outs[pad_to] = (s_o, z_o)
+        finally:
+            pf.pad_tokens_to, pf.pad_tokens_min_n = keep
+    for pad_to in (8, 0):
+        assert rel_err(outs[pad_to][1], z_ref) <= tol(BF16)
+        assert rel_err(outs[pad_to][0], s_ref) <= tol(BF16)
+    print(f"padded vs unpadded: z {rel_err(outs[8][1], outs[0][1]):.2e} s {rel_err(outs[8][0], outs[0][0]):.2e}")
+    # masked tokens contribute exact zeros in the same summation order: bit for bit
+    assert torch.equal(outs[8][1], outs[0][1]) and torch.equal(outs[8][0], outs[0][0])
+
+
+def test_padded_block_fp32_and_graph():
+    """A single fp32 block at an odd size (padded internally) against the oracle, eager and
+    through a recorded graph."""
+    from protenix_amd import pairformer as pf
+    ref, prod = oracle_and_product(O.PairformerBlock, P.PairformerBlock)
+    s, z, pm = O.make_inputs(45, n_pad=0)
+    keep = pf.pad_tokens_min_n
+    pf.pad_tokens_min_n = 0
+    try:
+        with torch.no_grad():
+            s_ref, z_ref = ref(s, z, pm)
+            ops.kernel_timer = {}
+            s_o, z_o = prod(s.cuda(), z.cuda(), None)
+            assert "triattn_fwd_padded_rows" in ops.kernel_timer      # (ran as 48 tokens, 3 of them masked)
+            ops.kernel_timer = None
+            fast = P.Graphed(prod)
+            for _ in range(3):
+                s_g, z_g = fast(s.cuda(), z.cuda(), None)
+                assert torch.equal(z_g, z_o) and torch.equal(s_g, s_o)
+    finally:
+        ops.kernel_timer = None
+        pf.pad_tokens_min_n = keep
+    assert rel_err(z_o, z_ref) <= tol(torch.float32) and rel_err(s_o, s_ref) <= tol(torch.float32)
