@@ -349,6 +349,9 @@ __global__ __launch_bounds__((NWQ * 64), (sizeof(T) == 2 ? (R == 1 ? 16 / NWQ : 
     // 16u .. 16u+15 and 32+16u .. 32+16u+15 of the tile: complete from 48 + 16u keys on, empty
     // (and left out altogether) up to 16u.
     const int tile_keys = LAST_PARTIAL ? nk - key0 : kKeyTile;
+    // A wave whose queries all lie beyond the launch's range only helps to stage the tiles (the
+    // bias loads below stay unconditional: both paths then leave the same loads in flight).
+    if (q_ok_mask != 0ull) {
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
       const bool tail_tile = LAST_PARTIAL && tile_keys < 48 + 16 * u;
@@ -390,6 +393,7 @@ __global__ __launch_bounds__((NWQ * 64), (sizeof(T) == 2 ? (R == 1 ? 16 / NWQ : 
 #pragma unroll
         for (int c = 0; c < 2; ++c) mma32(acc_o[r], lds_kv[buf][r][4 + u * 2 + c][lane], out.pf[c]);
       }
+    }
     }
     fetch_bias(tile + 1, tb);
   };
@@ -489,15 +493,13 @@ int triattn_fwd_ex(const T* q, const T* k, const T* vt, const T* g, const T* tri
   // wave; with four waves per workgroup the K / V tiles of two rows leave room for three
   // workgroups only: no gain).  Per launch: 395 -> 356 us at n = 768 in the trunk; in a loop of attention updates
   // -7 % at n = 512, -3 % at 768, -11 % at 1536, -13 % at 2048.  Where 256 queries do not divide
-  // n the idle waves of a last workgroup would cost more than the rows save (+10 to +25 % at
-  // 256, 384, 640): those launches cover the whole blocks of 256 queries only, and a second
-  // launch with one row per wave takes the remaining queries of every row (per update at
-  // n = 640: 269 -> 266 us, 1000: 1017 -> 987, 1100: 1328 -> 1241; a remainder of a few queries
-  // costs a launch that stages every row's keys for them: 211 -> 222 us at n = 520, so short
-  // remainders of short rows stay with one row per wave throughout).
-  const int q_rest = n % 256;
-  const bool r2 = sizeof(T) == 2 && !mask && n >= 512 && row_count >= 2 &&
-                  (q_rest == 0 || (n >= 640 && (q_rest >= 64 || n >= 1024)));
+  // n, the waves of a row's last workgroup that have no queries skip the arithmetic and only
+  // help to stage the K / V tiles; such a workgroup still holds its place for as long as the
+  // staging takes (n = 776 against 768, same keys: +11 %), but a second launch for the
+  // remaining queries - one row per wave, two or four waves per workgroup - was no better
+  // (per update, against the split launches with every wave computing: 520 214 -> 208 us,
+  // 640 270 -> 255, 704 369 -> 332, 800 592 -> 550, 1032 1127 -> 1055, 1100 1239 -> 1214).
+  const bool r2 = sizeof(T) == 2 && !mask && n >= 512 && row_count >= 2;
   const int mk = mask ? kMaskGiven : n_keys % kKeyTile ? kMaskTail : kMaskNone;
   // one launch over the queries q_begin .. q_end-1 of the launch's rows
   auto launch = [&](int q_begin, int q_end, bool two_rows, bool wide8) {
@@ -532,9 +534,7 @@ int triattn_fwd_ex(const T* q, const T* k, const T* vt, const T* g, const T* tri
 #undef PTX_ATTN_LAUNCH_R
   };
   if (r2) {
-    const int q_main = (n / 256) * 256;
-    launch(0, q_main, true, false);
-    if (q_main < n) launch(q_main, n, false, false);
+    launch(0, n, true, false);
   } else {
     launch(0, n, false, wide);
   }

@@ -34,8 +34,8 @@ def test_config2_triattn_start_n384_pad32():
 @pytest.mark.parametrize("n,n_pad", [(520, 0), (600, 0), (640, 24), (777, 0), (777, 50)])
 def test_triattn_two_rows_per_wave_at_sizes_256_does_not_divide(mixed, starting, n, n_pad):
     """From 512 tokens on, launches without a mask take two rows per wave in workgroups of 256
-    queries; where 256 does not divide N those cover the whole blocks of 256 queries and a
-    second launch (one row per wave) takes the remaining queries of every row.  Against the
+    queries; where 256 does not divide N the waves of a row's last workgroup that have no queries
+    only help to stage the keys.  Against the
     oracle, with and without a padded tail (whose valid rows run over a prefix of the keys), and
     against the same module with the mask handed to the kernels as it is (one row per wave)."""
     from protenix_amd import ops
