@@ -81,6 +81,31 @@ def test_triattn_two_rows_per_wave_at_sizes_256_does_not_divide(mixed, starting,
         assert torch.equal(got, plain)
 
 
+@pytest.mark.parametrize("n", [513, 544, 552, 576, 608, 672, 700, 736, 767, 769, 800, 1032])
+def test_triattn_partial_workgroups_give_the_bits_of_the_masked_kernels(n):
+    """Every count of waves without queries in a row's last workgroup (two rows per wave, 256
+    queries per workgroup; those waves only stage the key tiles), with and without a partial key
+    tile: the same bits as the masked kernels (one row per wave, 128 queries per workgroup) given
+    a mask of ones that is not recognised as such."""
+    from protenix_amd import ops
+    prod = P.TriangleAttention(128, 32, 4)
+    O.seed_parameters_(prod, seed=n)
+    prod = prod.to("cuda", BF16).eval()
+    zd = _z(n, seed=n).cuda()
+    with torch.no_grad():
+        got = prod(zd, None)
+    keep = ops.mask_class
+    ops.mask_class = lambda m: (False, None)
+    ops._mask_cache.clear()
+    try:
+        with torch.no_grad():
+            plain = prod(zd, torch.ones(1, n, n, dtype=BF16, device="cuda"))
+    finally:
+        ops.mask_class = keep
+        ops._mask_cache.clear()
+    assert torch.isfinite(got.float()).all() and torch.equal(got, plain)
+
+
 def test_triattn_n1536_pad40_wide_workgroups():
     """From 1536 tokens on the attention core runs 8-wave workgroups (256 queries share the
     staged key tiles): oracle parity at the smallest such size, ending node, padded."""
