@@ -160,3 +160,36 @@ def test_padded_block_fp32_and_graph():
         ops.kernel_timer = None
         pf.pad_tokens_min_n = keep
     assert rel_err(z_o, z_ref) <= tol(torch.float32) and rel_err(s_o, s_ref) <= tol(torch.float32)
+
+
+@pytest.mark.parametrize("kw,n", [(dict(c_z=64, c_s=0), 327),
+                                  (dict(c_z=256, hidden_scale_up=True), 323)])
+def test_other_widths_padded_at_the_default_threshold(kw, n):
+    """The template stack's width (no single track) and the scaled-up width at sizes just above
+    the size from which odd sizes are padded: fp32 rows under bf16 autocast against the oracle,
+    and the same bits as without the padding."""
+    from protenix_amd import pairformer as pf
+    assert n >= pf.pad_tokens_min_n and n % pf.pad_tokens_to
+    ref, prod = oracle_and_product(O.PairformerStack, P.PairformerStack, n_blocks=1, dtype=BF16, **kw)
+    prod = prod.float()
+    c_s = kw.get("c_s", 384)
+    s, z, pm = O.make_inputs(n, c_z=kw["c_z"], dtype=BF16)
+    s_in = None if c_s == 0 else s.float()
+    with torch.no_grad():
+        s_ref, z_ref = ref(s_in, z.float(), pm.float(), chunk_size=64)
+    outs = {}
+    for pad_to in (8, 0):
+        keep = pf.pad_tokens_to
+        pf.pad_tokens_to = pad_to
+        try:
+            ops.kernel_timer = {}
+            with torch.no_grad(), torch.autocast("cuda", dtype=BF16):
+                outs[pad_to] = prod(None if s_in is None else s_in.cuda(), z.float().cuda(), None)
+            assert ("triattn_fwd_padded_rows" in ops.kernel_timer) == (pad_to == 8)
+        finally:
+            ops.kernel_timer = None
+            pf.pad_tokens_to = keep
+    assert rel_err(outs[8][1], z_ref) <= tol(BF16)
+    assert torch.equal(outs[8][1], outs[0][1])
+    if c_s:
+        assert rel_err(outs[8][0], s_ref) <= tol(BF16) and torch.equal(outs[8][0], outs[0][0])
