@@ -68,7 +68,7 @@ def _work(n: int, z_bytes: int) -> dict:
 
 def _attn_update_ms(times: dict) -> float:
     """Median time of the attention core per triangle-attention update: a padded batch from
-    600 tokens on runs it as two launches (valid rows, padded rows), timed under two names."""
+    480 tokens on runs it as two launches (valid rows, padded rows), timed under two names."""
     t = statistics.median(times["triattn_fwd"])
     if "triattn_fwd_padded_rows" in times:
         t += statistics.median(times["triattn_fwd_padded_rows"])

@@ -188,11 +188,12 @@ _mask_cache: list = []
 
 # Pair masks of padded batches are m (x) m with the padding at the end: the triangle attention
 # then runs its valid rows over the valid keys without a mask (see triangle_attention).  False
-# hands every mask to the kernels as it is (tests compare the two).  Below some 600 tokens the
-# second launch costs what the first one saves (measured: 113 against 108 us at N = 256, 331
-# against 328 at 512, 750 against 775 at 768, 1.42 against 1.59 ms at 1024).
+# hands every mask to the kernels as it is (tests compare the two).  Below some 480 tokens the
+# second launch costs what the first one saves (measured per update, two launches against the
+# masked kernel: 170 against 157 us at N = 384 with 32 padded tokens, 237 = 237 at 448, 293
+# against 305 at 512, 390 against 411 at 576, 1.42 against 1.59 ms at 1024).
 prefix_mask_enabled = True
-prefix_mask_min_n = 600
+prefix_mask_min_n = 480
 
 
 _CACHE_ENTRIES = 64      # masks kept per cache: a batch of pair masks has one entry per element

@@ -16,7 +16,7 @@ pytestmark = pytest.mark.gpu
 
 @pytest.fixture(autouse=True)
 def _every_size():
-    """The two-range path at every N (the host side takes it from some 600 tokens on)."""
+    """The two-range path at every N (the host side takes it from some 480 tokens on)."""
     keep = ops.prefix_mask_min_n
     ops.prefix_mask_min_n = 0
     yield
@@ -36,7 +36,7 @@ def _run(prod, z, mask, mixed, prefix):
 
 
 def test_short_rows_keep_one_launch():
-    ops.prefix_mask_min_n = 600
+    ops.prefix_mask_min_n = 480
     _, prod = oracle_and_product(O.TriangleAttention, P.TriangleAttention, 128, 32, 4, dtype=torch.bfloat16)
     z = torch.randn(1, 96, 96, 128).to(torch.bfloat16).cuda()
     ops.kernel_timer = {}
