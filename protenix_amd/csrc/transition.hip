@@ -413,6 +413,11 @@ __global__ __launch_bounds__((TrCfg<T, KS>::NW * 64), 2) void transition_fused_k
   // (fp32 rows of 256 channels: 32 residual vectors per lane do not fit beside the output
   // accumulators; the second half of the column blocks is requested after the first half's
   // stores, one serialised round trip per wave)
+  // (the lane index again, opaque to the compiler: the values derived from it up here would
+  // otherwise be carried through the chunk loop, in registers the AO instantiations do not
+  // have - they were spilled ahead of the prologue and read back here)
+  int lane_e = (int)(threadIdx.x & 63);
+  asm volatile("" : "+v"(lane_e));
   constexpr int GOB = (MIXED && NOB > 4) ? 4 : NOB;
   int64_t obase[RB][C::NPASS];
   VE_t resv[RB][GOB][C::NPASS];
@@ -421,7 +426,7 @@ __global__ __launch_bounds__((TrCfg<T, KS>::NW * 64), 2) void transition_fused_k
 #pragma unroll
     for (int ps = 0; ps < C::NPASS; ++ps) {
       int mj, m0;
-      stage_coord<TZ>(ps, lane, mj, m0);
+      stage_coord<TZ>(ps, lane_e, mj, m0);
       const int64_t pr = row_at(rb * 32 + mj);
       obase[rb][ps] = pr >= 0 ? pr * kCx + m0 : -1;
     }
@@ -459,8 +464,8 @@ __global__ __launch_bounds__((TrCfg<T, KS>::NW * 64), 2) void transition_fused_k
                 "staging tiles, normalised tiles and the bias weight fit the chunk buffers");
   V8 (*lds_pbw)[kWave] = reinterpret_cast<V8 (*)[kWave]>(reinterpret_cast<char*>(&lds_w[0][0][0][0]) + kPbwOffset);
   if constexpr (PB) {
-    static_assert(!PB || sizeof(V8) == 16, "one 16-byte piece per lane and fragment");
-    const uint32_t voff = (uint32_t)((min(lane & 31, pb.heads - 1) * kCx + 8 * (lane >> 5)) * sizeof(T));
+    static_assert(!PB || sizeof(V8) == 16, "one 16-byte piece per lane_e and fragment");
+    const uint32_t voff = (uint32_t)((min(lane_e & 31, pb.heads - 1) * kCx + 8 * (lane_e >> 5)) * sizeof(T));
     for (int f = wave; f < KS; f += NW)
       load_to_lds16_s<0>(uniform64((uint64_t)((const T*)pb.w + 16 * f)), voff, lds_address(&lds_pbw[f][0]));
   }
@@ -479,10 +484,10 @@ __global__ __launch_bounds__((TrCfg<T, KS>::NW * 64), 2) void transition_fused_k
         vals[r] = MIXED ? to_f32(from_f32<T>(acc_o[rb][ob][r])) : acc_o[rb][ob][r];
       if constexpr (AO) {
         // x' of the block's columns, as the attention stage would have stored it: its update
-        // goes from the fragment layout (lane <-> row, channels 16 u + 8 g .. + 7) through the
+        // goes from the fragment layout (lane_e <-> row, channels 16 u + 8 g .. + 7) through the
         // staging tile to the layout of the stores and meets the raw row there
         typedef typename Vec8<TZ>::type VZ;
-        const int n = lane & 31, g = lane >> 5;
+        const int n = lane_e & 31, g = lane_e >> 5;
         wave_lds_sync();
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
@@ -496,17 +501,17 @@ __global__ __launch_bounds__((TrCfg<T, KS>::NW * 64), 2) void transition_fused_k
 #pragma unroll
         for (int ps = 0; ps < C::NPASS; ++ps) {
           int mj, m0;
-          stage_coord<TZ>(ps, lane, mj, m0);
+          stage_coord<TZ>(ps, lane_e, mj, m0);
           resv[rb][ob % GOB][ps] = add_vec<TZ>(stage_get_vec<TZ>(st, mj, m0), resv[rb][ob % GOB][ps]);
         }
       }
       wave_lds_sync();
-      stage_put<TZ>(st, vals, lane);
+      stage_put<TZ>(st, vals, lane_e);
       wave_lds_sync();
 #pragma unroll
       for (int ps = 0; ps < C::NPASS; ++ps) {
         int mj, m0;
-        stage_coord<TZ>(ps, lane, mj, m0);
+        stage_coord<TZ>(ps, lane_e, mj, m0);
         VE_t v = stage_get_vec<TZ>(st, mj, m0);
         if (obase[rb][ps] >= 0) {
           if (add_residual) v = add_vec<TZ>(v, resv[rb][ob % GOB][ps]);
@@ -519,8 +524,8 @@ __global__ __launch_bounds__((TrCfg<T, KS>::NW * 64), 2) void transition_fused_k
 
   if constexpr (PB) {
     static_assert(!PB || (RB == 1 && sizeof(T) == 2), "pair-bias epilogue: one row block, 16-bit arithmetic");
-    const int n = lane & 31, g = lane >> 5;
-    const int m0c = (lane % C::LPM) * C::VE;   // as stage_coord: the same columns in every pass
+    const int n = lane_e & 31, g = lane_e >> 5;
+    const int m0c = (lane_e % C::LPM) * C::VE;   // as stage_coord: the same columns in every pass
     // LayerNorm statistics of the finished rows (as stored: TZ), two passes in fp32.  In the
     // read-back layout a row's 32 columns of one block sit in LPM neighbouring lanes.
     float mean[C::NPASS], rstd[C::NPASS];
@@ -564,7 +569,7 @@ __global__ __launch_bounds__((TrCfg<T, KS>::NW * 64), 2) void transition_fused_k
 #pragma unroll
         for (int ps = 0; ps < C::NPASS; ++ps) {
           int mj, m0;
-          stage_coord<TZ>(ps, lane, mj, m0);
+          stage_coord<TZ>(ps, lane_e, mj, m0);
           const int ob = 2 * hb + o2;
 #pragma unroll
           for (int e4 = 0; e4 < C::VE; e4 += 4) {
@@ -582,7 +587,7 @@ __global__ __launch_bounds__((TrCfg<T, KS>::NW * 64), 2) void transition_fused_k
       for (int u = 0; u < 4; ++u) {
         const u32x2* src = reinterpret_cast<const u32x2*>(stn + n * kPitchN + 16 * u + 8 * g);
         u32x2 h2[2] = {src[0], src[1]};
-        mma32(accb, lds_pbw[4 * hb + u][lane], *reinterpret_cast<const V8*>(h2));   // lane <-> row, register <-> head
+        mma32(accb, lds_pbw[4 * hb + u][lane_e], *reinterpret_cast<const V8*>(h2));   // lane_e <-> row, register <-> head
       }
     }
     const int64_t pr = row_at(n);
