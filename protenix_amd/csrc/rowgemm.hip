@@ -320,6 +320,15 @@ rowgemm_in_kernel(RowGemmInParams p) {
 
   while (true) {
     if (RES && tile >= n_tiles) break;
+    // kTriMulIn (at the register limit): the lane index and what is derived from it are formed
+    // again in every tile, from a copy the compiler cannot see through - carried across the
+    // loop they were spilled (88 bytes per lane instead of 44, six registers instead of four
+    // written back in every tile: the kernel's 1.08 times its algorithmic bytes written).
+    int lane_s = threadIdx.x & 63;
+    if constexpr (MODE == kTriMulIn) asm volatile("" : "+v"(lane_s));
+    const int lane = lane_s;
+    const int n = lane & 31, g = lane >> 5;
+    T* const sink = reinterpret_cast<T*>(g_store_sink) + lane * C::VE;
     // The projections at the head of an update walk the pair tensor back to front.  The kernel
     // before them has just written it front to back, so its tail is what the 256 MB memory-side
     // cache still holds; read front to back, a tensor larger than that cache evicts its own
