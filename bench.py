@@ -41,7 +41,7 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 # from profiles/trunk_n768_fp32_residual_hbm_traffic.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # on this benchmark, calibrated against a plain elementwise kernel of known size), not measured
 # in this run.  Algorithmic: 446976 + 147456 KiB.
-TRIATTN_FWD_TRAFFIC_BYTES_N768 = (523521 + 147459) * 1024
+TRIATTN_FWD_TRAFFIC_BYTES_N768 = (525117 + 147458) * 1024
 TRAFFIC_SOURCE = "profiles/trunk_n768_fp32_residual_hbm_traffic.txt (rocprofv3 --pmc, not measured in this run)"
 
 
