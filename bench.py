@@ -472,6 +472,39 @@ def main() -> int:
                             f"N_token={n}, fp32 tensors and parameters under torch.autocast(bfloat16)"}
             del st256, s6, z6, pm6, zw6, step256
             torch.cuda.empty_cache()
+            # a size that 8 does not divide, no pair mask (what the reference's inference passes):
+            # run as the next multiple of 8 with the extra tokens masked, and as it is
+            from protenix_amd import pairformer as pf
+            ref_odd = O.seed_parameters_(O.PairformerStack(n_blocks=4))
+            st_odd = P.PairformerStack(n_blocks=4)
+            st_odd.load_state_dict(ref_odd.state_dict())
+            st_odd = st_odd.to(dev).eval()
+            del ref_odd
+            s7, z7, _ = (t.to(dev) for t in O.make_inputs(700))
+            zw7 = torch.empty_like(z7)
+
+            def step_odd():
+                zw7.copy_(z7)
+                with amp(True):
+                    return st_odd(s7, zw7, None, inplace_safe=True)
+            odd = {}
+            for pad_to in (8, 0):
+                keep_pad = pf.pad_tokens_to
+                pf.pad_tokens_to = pad_to
+                try:
+                    _, per_odd, out_odd = timed(step_odd, 2, 5)
+                finally:
+                    pf.pad_tokens_to = keep_pad
+                odd[pad_to] = (statistics.median(per_odd) / 4, out_odd[1].clone())
+            shapes["odd_size_n700_4_blocks"] = {
+                "ms_per_block": round(odd[8][0], 3), "ms_per_block_unpadded": round(odd[0][0], 3),
+                "same_bits": bool(torch.equal(odd[8][1], odd[0][1])),
+                "workload": "PairformerStack 4 blocks, N_token=700, no pair mask, fp32 tensors under "
+                            "torch.autocast(bfloat16): as 704 tokens with 4 masked (the default from 320 "
+                            "tokens on; the two copies of the pair tensor weigh 12 times what they weigh "
+                            "in a trunk) against the rows as they are"}
+            del st_odd, s7, z7, zw7, step_odd, odd
+            torch.cuda.empty_cache()
             stack = None
             # stand-alone LayerNorm over c_z = 128 on the pair tensor's rows
             for dt, name, ckey in ((BF16, "bf16", "151MB"), (torch.float32, "fp32", "302MB")):
