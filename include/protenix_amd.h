@@ -34,7 +34,7 @@
 extern "C" {
 #endif
 
-#define PTX_ABI_VERSION 2
+#define PTX_ABI_VERSION 3
 #define PTX_API __attribute__((visibility("default")))
 
 /*

@@ -14,7 +14,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libprotenix_amd.so")
 
 PTX_F32, PTX_BF16, PTX_MIXED, PTX_F16 = 0, 1, 2, 3
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 _p = ctypes.c_void_p
 _i = ctypes.c_int
