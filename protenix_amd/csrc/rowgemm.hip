@@ -117,7 +117,13 @@ template <typename T, int MODE, int KS> struct InCfg {
   static constexpr int SL = Widths<KS>::SL;
   // (256-channel rows: the weights do not fit either; bf16 then takes the staged path too)
   static constexpr bool RES = sizeof(T) == 2 && MODE != kPairBias && KS <= 8;
-  static constexpr int NW = RES ? 8 : 4;   // waves per workgroup
+  // waves per workgroup: 8 where the weights are resident, and in the attention projection on
+  // 16-bit rows of 256 channels, whose ring of two 32 KB chunk buffers leaves room for one
+  // workgroup per compute unit only: with four waves that was one wave per SIMD and a pass of
+  // all weights through the L2 per 128 rows (875 -> 588 us per launch at N = 768).  The
+  // triangle multiplication's projection of that width needs more than the 256 registers two
+  // waves per SIMD leave it (with eight waves 536 bytes of spills, 597 -> 696 us): four waves.
+  static constexpr int NW = (RES || (sizeof(T) == 2 && KS > 8 && MODE == kTriAttnIn)) ? 8 : 4;
   // chunks of two 32-column weight tiles: {a,b} x hidden/32 channel blocks | q,k,g,v: one per
   // two heads, bias: 1 | the pair bias | c_z / 32 output column blocks
   static constexpr int NCH = MODE == kTriMulIn    ? 2 * (SL / 2)
@@ -127,7 +133,7 @@ template <typename T, int MODE, int KS> struct InCfg {
   // weight fragments held in LDS (2*SL per chunk; the resident triangle bias is one tile)
   static constexpr int NFRAG = RES ? (MODE == kTriAttnIn ? (NCH - 1) * 2 * SL + SL : NCH * 2 * SL)
                                    : Cfg<T>::NBUF * 2 * SL;
-  static constexpr int FPW = 2 * SL / 4;   // staged path: fragments per wave and chunk
+  static constexpr int FPW = 2 * SL / NW;  // staged path: fragments per wave and chunk
   static constexpr int MIN_WG = (RES || KS > 8) ? 1 : 2;
 };
 
@@ -228,7 +234,7 @@ rowgemm_in_kernel(RowGemmInParams p) {
   // Resident: waves 0-3 of all workgroups come first in the walk, then waves 4-7, so that a
   // last round that covers half the machine's waves still gives every CU (and SIMD) its share.
   int64_t tile = RES ? (int64_t)(wave >> 2) * (gridDim.x * 4) + blockIdx.x * 4 + (wave & 3)
-                     : (int64_t)blockIdx.x * 4 + wave;
+                     : (int64_t)blockIdx.x * NW + wave;
   const int64_t tile_step = (int64_t)gridDim.x * NW;
 
   // Weight fragment f = 2*SL * chunk + SL * tile + K step, from global memory straight into its
@@ -1017,7 +1023,7 @@ int launch_rowgemm_in(const RowGemmInParams& p, hipStream_t stream) {
   int64_t tiles = (p.n_rows + RB * 32 - 1) / (RB * 32);   // wave tiles, as in the kernel
   if (MODE == kTriMulIn) tiles = (int64_t)((p.n + 16 * RB - 1) / (16 * RB)) * (p.pitch / 8) * 4;
   if (tiles == 0) return 0;
-  int64_t blocks = (tiles + 3) / 4;
+  int64_t blocks = (tiles + IC::NW - 1) / IC::NW;
   if (IC::RES) blocks = std::min<int64_t>((tiles + IC::NW - 1) / IC::NW, device_cu_count());
   // (only the modes with channel-major vector stores have an element-wise variant)
   constexpr bool kHasScalarPath = MODE == kTriAttnIn || MODE == kTriMulOut;
